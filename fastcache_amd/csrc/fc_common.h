@@ -1,0 +1,127 @@
+// Shared host/device helpers for libfastcache_hip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include "../../include/fastcache_hip.h"
+
+#define FC_HEAD_DIM 128
+#define FC_WAVE 64
+
+// ---- error reporting -------------------------------------------------------------------------
+void fc_set_error(const char* fmt, ...);
+
+#define FC_REQUIRE(cond, code, ...)            \
+  do {                                         \
+    if (!(cond)) {                             \
+      fc_set_error(__VA_ARGS__);               \
+      return (code);                           \
+    }                                          \
+  } while (0)
+
+#define FC_CHECK_LAUNCH(name)                                                  \
+  do {                                                                         \
+    hipError_t e__ = hipGetLastError();                                        \
+    if (e__ != hipSuccess) {                                                   \
+      fc_set_error("%s: launch failed: %s", name, hipGetErrorString(e__));     \
+      return FC_ELAUNCH;                                                       \
+    }                                                                          \
+  } while (0)
+
+int fc_check_view(const fc_kv_view* v, const char* who);
+
+static inline int fc_elem_bytes(int dtype) { return dtype == FC_F32 ? 4 : 2; }
+
+// ---- device-side copy of a view ---------------------------------------------------------------
+// Passed by value as a kernel argument; strides are in elements.
+struct KvView {
+  char* base;
+  long long stride_layer, stride_block, stride_batch, stride_token, stride_head;
+  const int* block_tables;
+  const int* seq_lens;
+  int table_stride, block_size, block_shift;  // block_shift >= 0 when block_size is a power of two
+  int batch, num_kv_heads, max_seq_len, num_layers;
+};
+
+static inline KvView fc_make_view(const fc_kv_view* v) {
+  KvView d;
+  d.base = (char*)v->base;
+  d.stride_layer = v->stride_layer;
+  d.stride_block = v->stride_block;
+  d.stride_batch = v->stride_batch;
+  d.stride_token = v->stride_token;
+  d.stride_head = v->stride_head;
+  d.block_tables = v->block_tables;
+  d.seq_lens = v->seq_lens;
+  d.table_stride = v->table_stride;
+  d.block_size = v->block_size > 0 ? v->block_size : 1;
+  d.block_shift = -1;
+  for (int s = 0; s < 31; ++s)
+    if ((1 << s) == d.block_size) d.block_shift = s;
+  d.batch = v->batch;
+  d.num_kv_heads = v->num_kv_heads;
+  d.max_seq_len = v->max_seq_len;
+  d.num_layers = v->num_layers;
+  return d;
+}
+
+#ifdef __HIPCC__
+// Element offset of token s of sequence b (layer and head offsets are added by the caller).
+// Returns -1 for a paged view whose table entry is negative (unallocated).
+__device__ __forceinline__ long long fc_token_offset(const KvView& v, int b, int s) {
+  if (v.block_tables) {
+    int blk_i, slot;
+    if (v.block_shift >= 0) {
+      blk_i = s >> v.block_shift;
+      slot = s & (v.block_size - 1);
+    } else {
+      blk_i = s / v.block_size;
+      slot = s - blk_i * v.block_size;
+    }
+    int blk = v.block_tables[(long long)b * v.table_stride + blk_i];
+    if (blk < 0) return -1;
+    return (long long)blk * v.stride_block + (long long)slot * v.stride_token;
+  }
+  return (long long)b * v.stride_batch + (long long)s * v.stride_token;
+}
+
+__device__ __forceinline__ int fc_seq_len(const KvView& v, int b) {
+  // never trust a length beyond what the host validated the block table against
+  int n = v.seq_lens ? v.seq_lens[b] : v.max_seq_len;
+  return n < v.max_seq_len ? (n < 0 ? 0 : n) : v.max_seq_len;
+}
+
+__device__ __forceinline__ float fc_bf16_to_float(unsigned short h) {
+  return __uint_as_float(((unsigned)h) << 16);
+}
+// round-to-nearest-even fp32 -> bf16, NaN preserved (the rounding torch applies on .to(bfloat16))
+__device__ __forceinline__ unsigned short fc_float_to_bf16(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ float fc_half_to_float(unsigned short h) {
+  _Float16 x;
+  __builtin_memcpy(&x, &h, 2);
+  return (float)x;
+}
+__device__ __forceinline__ unsigned short fc_float_to_half(float f) {
+  _Float16 x = (_Float16)f;  // round-to-nearest-even
+  unsigned short h;
+  __builtin_memcpy(&h, &x, 2);
+  return h;
+}
+
+__device__ __forceinline__ float fc_wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float fc_wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+#endif  // __HIPCC__

@@ -1,0 +1,157 @@
+// Row-wise top-k selection with lowest-index tie-break and ascending-index output.
+//
+// One workgroup (4 wavefronts) per score row.  The row is mapped to order-preserving 32-bit
+// keys and staged in LDS; an MSB-first radix select (4 passes of 8 bits, LDS histogram) finds
+// the exact key T of the k-th largest element and how many elements equal to T are still
+// needed.  A final ordered pass keeps every key > T plus the first `need` keys == T in index
+// order, using wavefront ballots for the running ranks, so the output is ascending and
+// deterministic.  Rows too long for LDS are re-read from global memory (L2-resident).
+#include "fc_common.h"
+
+#define TK_THREADS 256
+#define TK_WAVES (TK_THREADS / FC_WAVE)
+#define TK_LDS_MAX_KEYS 15360  // 60 KiB of keys
+
+__device__ __forceinline__ unsigned tk_key(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;  // NaN ranks above +inf
+  if ((u & 0x7fffffffu) == 0u) u = 0u;                      // -0 == +0
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+template <bool LDS_KEYS>
+__global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restrict__ scores,
+                                                          int score_stride, int len,
+                                                          const int* __restrict__ row_lens,
+                                                          int rows_per_len, int row_lens_mod, int k,
+                                                          const int* __restrict__ n_kept,
+                                                          int* __restrict__ indices, int index_stride) {
+  extern __shared__ unsigned lds_keys[];
+  __shared__ unsigned hist[256];
+  __shared__ unsigned wave_tot[TK_WAVES];
+  __shared__ unsigned sel_bin, sel_remaining;
+  __shared__ unsigned w_eq[TK_WAVES], w_gt[TK_WAVES];
+
+  const int r = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = (row_lens || n_kept) ? (r / rows_per_len) % row_lens_mod : 0;
+  int n = row_lens ? row_lens[li] : len;
+  if (n > len) n = len;
+  int kk = n_kept ? n_kept[li] : k;
+  if (kk > n) kk = n;
+  if (kk > index_stride) kk = index_stride;
+  if (n <= 0 || kk <= 0) return;
+  const float* row = scores + (long long)r * score_stride;
+  int* out = indices + (long long)r * index_stride;
+
+  if (kk == n) {
+    for (int i = tid; i < n; i += TK_THREADS) out[i] = i;
+    return;
+  }
+
+  if (LDS_KEYS) {
+    for (int i = tid; i < n; i += TK_THREADS) lds_keys[i] = tk_key(row[i]);
+  }
+  auto key_at = [&](int i) -> unsigned { return LDS_KEYS ? lds_keys[i] : tk_key(row[i]); };
+
+  unsigned prefix = 0, mask = 0, remaining = (unsigned)kk;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    hist[tid] = 0;  // TK_THREADS == 256 bins
+    __syncthreads();
+    for (int i = tid; i < n; i += TK_THREADS) {
+      unsigned u = key_at(i);
+      if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    // suffix sums over bins: thread t owns bin 255 - t
+    const unsigned h = hist[255 - tid];
+    unsigned incl = h;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      unsigned up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    unsigned base = 0;
+    for (int w = 0; w < wave; ++w) base += wave_tot[w];
+    incl += base;
+    const unsigned excl = incl - h;  // elements in strictly larger bins
+    if (excl < remaining && remaining <= incl) {
+      sel_bin = 255u - (unsigned)tid;
+      sel_remaining = remaining - excl;
+    }
+    __syncthreads();
+    prefix |= sel_bin << shift;
+    mask |= 255u << shift;
+    remaining = sel_remaining;
+    __syncthreads();
+  }
+  const unsigned T = prefix;
+  const unsigned need = remaining;  // how many keys == T to keep (>= 1)
+
+  // each wave owns a contiguous segment, walked 64 keys at a time
+  const int seg = (((n + TK_WAVES - 1) / TK_WAVES) + 63) & ~63;
+  const int beg = wave * seg;
+  const int end = min(n, beg + seg);
+  unsigned eq_cnt = 0, gt_cnt = 0;
+  for (int i0 = beg; i0 < end; i0 += 64) {
+    int i = i0 + lane;
+    unsigned u = (i < end) ? key_at(i) : 0u;
+    bool live = i < end;
+    eq_cnt += __popcll(__ballot(live && u == T));
+    gt_cnt += __popcll(__ballot(live && u > T));
+  }
+  if (lane == 0) { w_eq[wave] = eq_cnt; w_gt[wave] = gt_cnt; }
+  __syncthreads();
+  unsigned eq_seen = 0, out_pos = 0;
+  {
+    unsigned eq_run = 0;
+    for (int w = 0; w < wave; ++w) {
+      unsigned take = need > eq_run ? min(need - eq_run, w_eq[w]) : 0u;
+      out_pos += w_gt[w] + take;
+      eq_run += w_eq[w];
+    }
+    eq_seen = eq_run;
+  }
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int i0 = beg; i0 < end; i0 += 64) {
+    int i = i0 + lane;
+    bool live = i < end;
+    unsigned u = live ? key_at(i) : 0u;
+    bool is_eq = live && u == T;
+    unsigned long long eqb = __ballot(is_eq);
+    unsigned my_rank = eq_seen + __popcll(eqb & lt_mask);
+    bool sel = live && (u > T || (is_eq && my_rank < need));
+    unsigned long long sb = __ballot(sel);
+    if (sel) out[out_pos + __popcll(sb & lt_mask)] = i;
+    eq_seen += __popcll(eqb);
+    out_pos += __popcll(sb);
+  }
+}
+
+extern "C" int fc_topk_select(const float* scores, int32_t score_stride, int32_t rows, int32_t len,
+                              const int32_t* row_lens, int32_t rows_per_len, int32_t row_lens_mod,
+                              int32_t k,
+                              const int32_t* n_kept, int32_t* indices, int32_t index_stride,
+                              void* stream) {
+  FC_REQUIRE(scores && indices, FC_EINVAL, "fc_topk_select: null pointer");
+  FC_REQUIRE(rows >= 0 && len >= 0 && score_stride >= len && index_stride >= 0, FC_EINVAL,
+             "fc_topk_select: bad sizes rows=%d len=%d score_stride=%d index_stride=%d", rows, len,
+             score_stride, index_stride);
+  FC_REQUIRE(n_kept != nullptr || (k >= 0 && k <= index_stride), FC_EINVAL,
+             "fc_topk_select: k=%d does not fit index_stride=%d", k, index_stride);
+  FC_REQUIRE((row_lens == nullptr && n_kept == nullptr) || (row_lens_mod > 0 && rows_per_len > 0),
+             FC_EINVAL, "fc_topk_select: rows_per_len and row_lens_mod must be positive when per-row sizes are given");
+  if (rows == 0 || len == 0) return FC_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (len <= TK_LDS_MAX_KEYS) {
+    hipLaunchKernelGGL((topk_kernel<true>), dim3(rows), dim3(TK_THREADS), (size_t)len * 4, st, scores,
+                       score_stride, len, row_lens, rows_per_len, row_lens_mod, k, n_kept, indices, index_stride);
+  } else {
+    hipLaunchKernelGGL((topk_kernel<false>), dim3(rows), dim3(TK_THREADS), 0, st, scores, score_stride,
+                       len, row_lens, rows_per_len, row_lens_mod, k, n_kept, indices, index_stride);
+  }
+  FC_CHECK_LAUNCH("fc_topk_select");
+  return FC_OK;
+}

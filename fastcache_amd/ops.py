@@ -1,0 +1,207 @@
+"""Functional layer over the C ABI: torch tensors in, torch tensors out.
+
+torch is used only for device memory and the current HIP stream; every computation is a call
+into libfastcache_hip.so.  All functions enqueue on ``torch.cuda.current_stream()`` and return
+without synchronising.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import FastcacheError, FcKvView, FcMlpWeights, check, current_stream, fn, ptr
+
+
+def _i32(t: Optional[torch.Tensor], name: str, device) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise FastcacheError(f"{name} must be a contiguous int32 tensor")
+    if t.device != device:
+        raise FastcacheError(f"{name} is on {t.device}, expected {device}")
+    return t
+
+
+# ---------------------------------------------------------------------------------------------
+# scoring
+# ---------------------------------------------------------------------------------------------
+def knorm_score(keys: FcKvView, device, score_stride: Optional[int] = None) -> torch.Tensor:
+    """``-||k||_2`` per (layer, sequence, kv head, token) -> fp32 ``[L, B, Hkv, stride]``."""
+    stride = keys.max_seq_len if score_stride is None else score_stride
+    out = torch.empty((keys.num_layers, keys.batch, keys.num_kv_heads, stride), dtype=torch.float32, device=device)
+    check(fn("fc_knorm_score")(C.byref(keys), out.data_ptr(), stride, current_stream()), "fc_knorm_score")
+    return out
+
+
+def knorm_mean_score(keys: FcKvView, device, score_stride: Optional[int] = None) -> torch.Tensor:
+    """Head-averaged key norm per (layer, sequence, token) -> fp32 ``[L, B, stride]``."""
+    stride = keys.max_seq_len if score_stride is None else score_stride
+    out = torch.empty((keys.num_layers, keys.batch, stride), dtype=torch.float32, device=device)
+    check(fn("fc_knorm_mean_score")(C.byref(keys), out.data_ptr(), stride, current_stream()),
+          "fc_knorm_mean_score")
+    return out
+
+
+def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size: int,
+                 causal_window: bool = True, reduction: str = "mean", scale: Optional[float] = None,
+                 seq_lens: Optional[torch.Tensor] = None, score_stride: Optional[int] = None) -> torch.Tensor:
+    """SnapKV observation-window scores -> fp32 ``[L, B, Hkv, stride]`` with the window positions
+    set to the per-layer maximum.  queries ``[L, B, Hq, W, D]`` (or ``[B, Hq, W, D]`` for one layer)."""
+    if queries.dim() == 4:
+        queries = queries.unsqueeze(0)
+    if not queries.is_contiguous():
+        queries = queries.contiguous()
+    _lib.require_gpu(queries, "queries")
+    L, B, Hq, W, D = queries.shape
+    if (L, B) != (keys.num_layers, keys.batch) or W != window or D != keys.head_dim:
+        raise FastcacheError(f"queries {tuple(queries.shape)} do not match the key view "
+                             f"(L={keys.num_layers}, B={keys.batch}, W={window}, D={keys.head_dim})")
+    if _lib.dtype_code(queries.dtype) != keys.dtype:
+        raise FastcacheError("queries and keys must share a dtype")
+    if Hq % keys.num_kv_heads:
+        raise FastcacheError("num_q_heads must be a multiple of num_kv_heads")
+    G = Hq // keys.num_kv_heads
+    if reduction not in ("mean", "sum"):
+        raise ValueError("reduction must be 'mean' or 'sum'")
+    out_scale = 1.0 / (W * G) if reduction == "mean" else 1.0
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    stride = keys.max_seq_len if score_stride is None else score_stride
+    dev = queries.device
+    out = torch.empty((L, B, keys.num_kv_heads, stride), dtype=torch.float32, device=dev)
+    st = current_stream()
+    check(fn("fc_snapkv_score")(C.byref(keys), queries.data_ptr(), Hq, window, kernel_size,
+                                int(causal_window), scale, out_scale, out.data_ptr(), stride, st),
+          "fc_snapkv_score")
+    ws = torch.empty((L,), dtype=torch.float32, device=dev)
+    check(fn("fc_snapkv_fill_window")(out.data_ptr(), stride, L, B, keys.num_kv_heads, ptr(seq_lens),
+                                      keys.max_seq_len, window, ws.data_ptr(), st), "fc_snapkv_fill_window")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# selection and compaction
+# ---------------------------------------------------------------------------------------------
+def topk_select(scores: torch.Tensor, k: int, row_lens: Optional[torch.Tensor] = None,
+                n_kept: Optional[torch.Tensor] = None, rows_per_len: int = 1) -> torch.Tensor:
+    """Indices of the ``k`` largest entries per row of ``scores[..., S]`` (fp32): ties to the lowest
+    index, output ascending, int32 ``[..., k]``.  With ``row_lens``/``n_kept`` (int32 ``[B]``) rows
+    ordered (..., b, head) take their valid length and kept count from entry ``b``
+    (``rows_per_len`` = heads per b); entries past a row's kept count are left at -1."""
+    _lib.require_gpu(scores, "scores")
+    if scores.dtype != torch.float32 or scores.stride(-1) != 1:
+        raise FastcacheError("scores must be fp32 with a contiguous last axis")
+    S = scores.shape[-1]
+    flat = scores.reshape(-1, S) if scores.is_contiguous() else None
+    if flat is None:
+        # rows must be equally spaced: allow a narrowed last axis of a contiguous buffer
+        lead = scores.shape[:-1]
+        stride = scores.stride(-2) if scores.dim() > 1 else S
+        expect = [stride]
+        for n in reversed(lead[1:]):
+            expect.append(expect[-1] * n)
+        if list(scores.stride()[:-1]) != list(reversed(expect)):
+            raise FastcacheError("scores rows must be equally spaced in memory")
+        rows, score_stride = math.prod(lead), stride
+    else:
+        rows, score_stride = flat.shape[0], S
+    dev = scores.device
+    row_lens = _i32(row_lens, "row_lens", dev)
+    n_kept = _i32(n_kept, "n_kept", dev)
+    per_row = row_lens is not None or n_kept is not None
+    mod = (row_lens if row_lens is not None else n_kept).numel() if per_row else 1
+    if n_kept is not None:
+        out = torch.full((*scores.shape[:-1], k), -1, dtype=torch.int32, device=dev)
+    else:
+        out = torch.empty((*scores.shape[:-1], k), dtype=torch.int32, device=dev)
+    check(fn("fc_topk_select")(scores.data_ptr(), score_stride, rows, S, ptr(row_lens), rows_per_len, mod, k,
+                               ptr(n_kept), out.data_ptr(), k, current_stream()), "fc_topk_select")
+    return out
+
+
+def compact(src_k: FcKvView, src_v: FcKvView, dst_k: FcKvView, dst_v: FcKvView, indices: torch.Tensor,
+            k: Optional[int] = None, n_kept: Optional[torch.Tensor] = None) -> None:
+    """dst token j <- src token indices[l, b, h, j]; indices int32 ``[L, B, Hkv or 1, stride]``."""
+    if indices.dtype != torch.int32 or indices.dim() != 4 or not indices.is_contiguous():
+        raise FastcacheError("indices must be a contiguous int32 [L, B, heads, k] tensor")
+    _lib.require_gpu(indices, "indices")
+    L, B, Hi, stride = indices.shape
+    if (L, B) != (src_k.num_layers, src_k.batch):
+        raise FastcacheError("indices do not match the views' layers/batch")
+    n_kept = _i32(n_kept, "n_kept", indices.device)
+    check(fn("fc_compact")(C.byref(src_k), C.byref(src_v), C.byref(dst_k), C.byref(dst_v), indices.data_ptr(),
+                           stride, Hi, stride if k is None else k, ptr(n_kept), current_stream()),
+          "fc_compact")
+
+
+def copy_tokens(src: FcKvView, dst: FcKvView, seg_start: int, count: int, dst_start: int) -> None:
+    check(fn("fc_copy_tokens")(C.byref(src), C.byref(dst), seg_start, count, dst_start, current_stream()),
+          "fc_copy_tokens")
+
+
+# ---------------------------------------------------------------------------------------------
+# CCM MLP
+# ---------------------------------------------------------------------------------------------
+def ccm_mlp(src: FcKvView, dst: FcKvView, weights: Tuple[torch.Tensor, ...], cf: int, seg_start: int,
+            seg_len: int, dst_start: int) -> None:
+    """weights = (w1 [L,128,cf*128], b1 [L,128], w2 [L,128,128], b2, w3, b3) in the KV dtype."""
+    w1, b1, w2, b2, w3, b3 = weights
+    L = src.num_layers
+    D = src.head_dim
+    shapes = [(L, D, cf * D), (L, D), (L, D, D), (L, D), (L, D, D), (L, D)]
+    for t, shp, name in zip(weights, shapes, ("w1", "b1", "w2", "b2", "w3", "b3")):
+        _lib.require_gpu(t, name)
+        if tuple(t.shape) != shp or not t.is_contiguous() or _lib.dtype_code(t.dtype) != src.dtype:
+            raise FastcacheError(f"{name} must be contiguous {shp} in the KV dtype, got {tuple(t.shape)} {t.dtype}")
+    w = FcMlpWeights(*(t.data_ptr() for t in weights))
+    check(fn("fc_ccm_mlp")(C.byref(src), C.byref(dst), C.byref(w), cf, seg_start, seg_len, dst_start,
+                           current_stream()), "fc_ccm_mlp")
+
+
+# ---------------------------------------------------------------------------------------------
+# decode
+# ---------------------------------------------------------------------------------------------
+def store_kv(k_cache: FcKvView, v_cache: FcKvView, k_new: torch.Tensor, v_new: torch.Tensor,
+             context_lens: torch.Tensor) -> None:
+    """Append ``k_new/v_new [L, B, Hkv, D]`` at position ``context_lens[b]`` of every sequence."""
+    for t, name in ((k_new, "k_new"), (v_new, "v_new")):
+        _lib.require_gpu(t, name)
+        if tuple(t.shape) != (k_cache.num_layers, k_cache.batch, k_cache.num_kv_heads, k_cache.head_dim) \
+                or not t.is_contiguous() or _lib.dtype_code(t.dtype) != k_cache.dtype:
+            raise FastcacheError(f"{name} must be contiguous [L, B, Hkv, D] in the cache dtype")
+    _i32(context_lens, "context_lens", k_new.device)
+    check(fn("fc_store_kv")(C.byref(k_cache), C.byref(v_cache), k_new.data_ptr(), v_new.data_ptr(),
+                            context_lens.data_ptr(), current_stream()), "fc_store_kv")
+
+
+def advance_lens(context_lens: torch.Tensor, delta: int = 1) -> None:
+    _i32(context_lens, "context_lens", context_lens.device)
+    _lib.require_gpu(context_lens, "context_lens")
+    check(fn("fc_advance_lens")(context_lens.data_ptr(), context_lens.numel(), delta, current_stream()),
+          "fc_advance_lens")
+
+
+def decode_attn_workspace(batch: int, num_q_heads: int, max_seq_len: int, device) -> torch.Tensor:
+    n = fn("fc_decode_attn_workspace_bytes")(batch, num_q_heads, max_seq_len)
+    if n < 0:
+        raise FastcacheError("fc_decode_attn_workspace_bytes: bad arguments")
+    return torch.empty((max(int(n), 256),), dtype=torch.uint8, device=device)
+
+
+def decode_attn(k_cache: FcKvView, v_cache: FcKvView, layer: int, q: torch.Tensor, context_lens: torch.Tensor,
+                scale: float, workspace: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q ``[B, Hq, D]`` -> out ``[B, Hq, D]`` for one layer of the cache views."""
+    _lib.require_gpu(q, "q")
+    if q.dim() != 3 or not q.is_contiguous() or _lib.dtype_code(q.dtype) != k_cache.dtype:
+        raise FastcacheError("q must be contiguous [B, Hq, D] in the cache dtype")
+    if out is None:
+        out = torch.empty_like(q)
+    _i32(context_lens, "context_lens", q.device)
+    check(fn("fc_decode_attn")(C.byref(k_cache), C.byref(v_cache), layer, q.data_ptr(), out.data_ptr(), q.shape[1],
+                               context_lens.data_ptr(), scale, workspace.data_ptr(), workspace.numel(),
+                               current_stream()), "fc_decode_attn")
+    return out

@@ -1,0 +1,214 @@
+/*
+ * fastcache_hip.h — C ABI of libfastcache_hip.so (gfx950 / MI355X).
+ *
+ * The reference (Ringssss/Fastcache) has no FFI for its KV-cache compression
+ * path: its boundary is a set of Python call signatures that end in torch ops,
+ * Triton kernels and two third-party wheels (kvpress, flash-attn).  Each entry
+ * point below names the reference call it stands in for (paths are relative to
+ * the reference root).
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer owned by the caller, except the
+ *     descriptor structs themselves (fc_kv_view, fc_mlp_weights), which are
+ *     read on the host during the call and may be freed after it returns;
+ *   - the call only ENQUEUES work on `stream` (a hipStream_t passed as void*;
+ *     NULL = the default stream): no allocation, no synchronisation, no global
+ *     state, so it may be recorded into a HIP graph;
+ *   - return value: FC_OK (0) or a negative FC_E* code; nothing is enqueued
+ *     when an error is returned; fc_last_error() gives a message for the
+ *     calling thread;
+ *   - head_dim must be 128 (every model family of the reference path);
+ *   - element types: FC_F32, FC_F16, FC_BF16.
+ */
+#ifndef FASTCACHE_HIP_H
+#define FASTCACHE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FC_ABI_VERSION 1
+
+enum { FC_F32 = 0, FC_F16 = 1, FC_BF16 = 2 };
+
+enum {
+  FC_OK = 0,
+  FC_EINVAL = -1,      /* bad argument (null pointer, non-positive size, unsupported dtype/head_dim) */
+  FC_EUNSUPPORTED = -2,/* shape outside what the kernels were built for */
+  FC_ELAUNCH = -3      /* hipLaunchKernel reported an error */
+};
+
+/*
+ * A strided view of one K (or V) cache, either
+ *   paged  (block_tables != NULL): nano-vllm pool kv_cache[kv][layer][block][slot][kv_head][d]
+ *          (nanovllm/engine/llava_model_runner.py:526-529); token s of sequence b lives in
+ *          block block_tables[b*table_stride + s/block_size], slot s%block_size;
+ *   dense  (block_tables == NULL): a HuggingFace-layout tensor [B, Hkv, S, D], possibly a
+ *          permuted view (llava_model_runner.py:863-868).
+ * Element address (in elements of `dtype` from `base`):
+ *   paged: layer*stride_layer + block*stride_block + slot*stride_token + head*stride_head + d
+ *   dense: layer*stride_layer + b*stride_batch     + s*stride_token    + head*stride_head + d
+ * The d axis is contiguous.  seq_lens[b] gives each sequence's token count (NULL in dense
+ * mode = every sequence has max_seq_len tokens).
+ */
+typedef struct fc_kv_view {
+  void* base;
+  int64_t stride_layer;
+  int64_t stride_block;
+  int64_t stride_batch;
+  int64_t stride_token;
+  int64_t stride_head;
+  const int32_t* block_tables;
+  int32_t table_stride;   /* entries per row of block_tables */
+  int32_t block_size;     /* 256 in the reference (nanovllm/engine/sequence.py:15) */
+  int32_t dtype;
+  int32_t num_layers;
+  int32_t batch;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t max_seq_len;
+  const int32_t* seq_lens;
+} fc_kv_view;
+
+int fc_abi_version(void);
+const char* fc_last_error(void);
+
+/*
+ * Knorm scoring.  scores[l][b][h][s] = -||K[l][b][h][s][:]||_2, fp32 accumulation, for
+ * s < seq_lens[b]; entries s >= seq_lens[b] are set to -inf.
+ * Replaces kvpress.KnormPress.score (third-party; reference call sites
+ * utils_ccm/utils_compress.py:22-24, 318-320, 347-348) evaluated per layer inside the
+ * attention forward hook (utils_compress.py:209-270).
+ * scores: float[num_layers][batch][num_kv_heads][score_stride].
+ */
+int fc_knorm_score(const fc_kv_view* keys, float* scores, int32_t score_stride, void* stream);
+
+/*
+ * Head-averaged key norms of the in-tree adapter: mean_norm[l][b][s] = mean_h ||K[l][b][h][s]||_2
+ * (nanovllm/kernels/kvpress_compressor.py:220-223).  Entries s >= seq_lens[b] are -inf.
+ * out: float[num_layers][batch][score_stride].
+ */
+int fc_knorm_mean_score(const fc_kv_view* keys, float* out, int32_t score_stride, void* stream);
+
+/*
+ * SnapKV scoring over an observation window.
+ *   queries: [num_layers][batch][num_q_heads][window][head_dim] (contiguous, dtype of keys) —
+ *            the already-rotated last `window` query positions;
+ *   A = softmax_fp32(Q K^T * scale) over all keys of kv head hq / (num_q_heads/num_kv_heads),
+ *       with (causal_window != 0) key position S-W+j masked for window query i when j > i;
+ *   v[hq][s] = sum_i A[hq][i][s] for s < S-W;  pooled = avg_pool1d(v, kernel, stride 1,
+ *   pad kernel/2, zeros counted);  scores[l][b][hkv][s] = out_scale * sum_{hq in group} pooled.
+ *   Entries S-W <= s < S are left for fc_snapkv_fill_window; entries s >= S are -inf.
+ * Replaces kvpress.SnapKVPress.score / compute_window_attention (third-party; reference
+ * call sites utils_ccm/utils_compress.py:310-312, 335-337; bench_kvpress_native.py:137-147;
+ * nanovllm/kernels/kvpress_compressor.py:139-143).
+ * Every sequence must have seq_len > window.  kernel_size must be odd and <= 63.
+ */
+int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_heads,
+                    int32_t window, int32_t kernel_size, int32_t causal_window,
+                    float scale, float out_scale,
+                    float* scores, int32_t score_stride, void* stream);
+
+/*
+ * Sets the window entries scores[l][b][h][S_b-W .. S_b) to the maximum over
+ * scores[l][:, :, :S_b-W] of the same layer, the way kvpress pads the observation window
+ * back in (F.pad(value=scores.max())) so that it always survives selection.
+ */
+int fc_snapkv_fill_window(float* scores, int32_t score_stride, int32_t num_layers, int32_t batch,
+                          int32_t num_kv_heads, const int32_t* seq_lens, int32_t max_seq_len,
+                          int32_t window, void* workspace /* float[num_layers] */, void* stream);
+
+/*
+ * Row-wise top-k with a defined order.  Row r of `rows` score rows has
+ * row_lens[(r / rows_per_len) % row_lens_mod] valid entries (row_lens == NULL: `len`) and keeps
+ * n_kept[(r / rows_per_len) % row_lens_mod] of them (n_kept == NULL: `k`); for rows ordered
+ * (layer, b, head) that is rows_per_len = heads, row_lens_mod = batch.  The kept scores are the
+ * largest ones, ties broken towards the lowest index; their indices are written in ASCENDING
+ * index order to indices[r*index_stride ...].  NaN sorts above +inf, -0 equals +0 (torch.topk's order).
+ * Replaces scores.topk(n_kept).indices of kvpress.ScorerPress.compress (third-party) and
+ * topk + sort of nanovllm/kernels/kvpress_compressor.py:225-226.
+ */
+int fc_topk_select(const float* scores, int32_t score_stride, int32_t rows, int32_t len,
+                   const int32_t* row_lens, int32_t rows_per_len, int32_t row_lens_mod,
+                   int32_t k, const int32_t* n_kept,
+                   int32_t* indices, int32_t index_stride, void* stream);
+
+/*
+ * Gather + compaction.  For each (layer, b, kv head): dst token j <- src token
+ * indices[(l*batch + b)*heads_in_index + (h % heads_in_index)][j] for j < n_kept[b] (or k).
+ * `dst` may alias `src` (same pool, same tables): indices must then be ascending, and the
+ * copy is ordered so that no source row is overwritten before it is read.
+ * Replaces keys.gather(2, idx) (nanovllm/kernels/kvpress_compressor.py:241-249) followed by
+ * LlavaModelRunner._write_compressed_kv_cache_fast (llava_model_runner.py:874-912), and the
+ * generated sparse_gather kernel (nanovllm/autocompress/kernels.py:321-346).
+ * Slots at and beyond n_kept keep their previous contents, as in the reference.
+ */
+int fc_compact(const fc_kv_view* src_k, const fc_kv_view* src_v,
+               const fc_kv_view* dst_k, const fc_kv_view* dst_v,
+               const int32_t* indices, int32_t index_stride, int32_t heads_in_index,
+               int32_t k, const int32_t* n_kept, void* stream);
+
+/*
+ * CCM three-layer MLP compressor over one token segment.
+ *   y = W3 relu(W2 relu(W1 x + b1) + b2) + b3,  x = concat of `cf` consecutive tokens of one head,
+ *   rounded to the storage dtype after every Linear (fp32 accumulation).
+ * Weights are nn.Linear layout [out][in] in the storage dtype, stacked over layers:
+ *   w1 [L][128][cf*128], w2/w3 [L][128][128], b1/b2/b3 [L][128].
+ * For each (layer, b, head): rows j < c = seg_len/cf read src tokens [seg_start + cf*j, +cf)
+ * and write dst token dst_start + j; the seg_len - c*cf remainder tokens are copied to
+ * dst_start + c + i.  `dst` may alias `src` when dst_start <= seg_start.
+ * Replaces KVCacheLinearDecoupleCompressor.compress_layer (utils_ccm/module_ccm_v11.py:666-694),
+ * KVCacheHybridCompressor.compress_layer (:883-925), BatchedGEMMCompressor._compress_batched
+ * (nanovllm/kernels/batched_compress.py:361-440) and its Triton kernel (:31-122).
+ */
+typedef struct fc_mlp_weights {
+  const void* w1; const void* b1;
+  const void* w2; const void* b2;
+  const void* w3; const void* b3;
+} fc_mlp_weights;
+
+int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w,
+               int32_t cf, int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream);
+
+/*
+ * Plain ordered token copy src[seg_start + i] -> dst[dst_start + i], i < count, per
+ * (layer, b, head); the pass-through branch of compress_layer when seg_len/cf < min_seq_len
+ * (module_ccm_v11.py:674-675).  dst may alias src when dst_start <= seg_start.
+ */
+int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst,
+                   int32_t seg_start, int32_t count, int32_t dst_start, void* stream);
+
+/*
+ * Append one new K/V row per sequence: cache[block_tables[b][len_b / bs]][len_b % bs] <- k_new[b], v_new[b]
+ * for every layer in the views (k_new/v_new: [num_layers][batch][num_kv_heads][head_dim]).
+ * The slot is computed on the device from context_lens so that the call can be replayed in a graph.
+ * Replaces store_kvcache (nanovllm/layers/attention.py:10-39) + the slot computation of
+ * LlavaModelRunner.prepare_decode (llava_model_runner.py:655-665).
+ * Rows with context_lens[b] < 0 are skipped.
+ */
+int fc_store_kv(const fc_kv_view* k_cache, const fc_kv_view* v_cache,
+                const void* k_new, const void* v_new, const int32_t* context_lens, void* stream);
+
+/* context_lens[b] += delta for b < batch where context_lens[b] >= 0 (device side, graph-replayable). */
+int fc_advance_lens(int32_t* context_lens, int32_t batch, int32_t delta, void* stream);
+
+/*
+ * Decode paged attention, one query token per sequence, for ONE layer `layer` of the views:
+ *   o[b][hq] = softmax_fp32(q[b][hq] . K[b][:len_b][hq/G]^T * scale) V[b][:len_b][hq/G]
+ * q, out: [batch][num_q_heads][head_dim] in the cache dtype (fp16/bf16).  context_lens[b] is the number
+ * of cached tokens attended (rows with context_lens[b] <= 0 produce zeros).
+ * Replaces flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens, block_table, softmax_scale,
+ * causal=True) at nanovllm/layers/attention.py:75-77.
+ * workspace: fc_decode_attn_workspace_bytes(batch, num_q_heads, max_splits) bytes, 256-byte aligned.
+ */
+int64_t fc_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t max_seq_len);
+int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer,
+                   const void* q, void* out, int32_t num_q_heads, const int32_t* context_lens,
+                   float scale, void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTCACHE_HIP_H */

@@ -1,0 +1,23 @@
+"""CPU oracle for the KV-cache compression path — TEST INFRASTRUCTURE, not product code.
+
+Each function restates, on the CPU with torch/numpy, what the reference computes at the
+file:line it cites (paths relative to the reference root).  Only the tests, the smoke check
+and the CPU-baseline leg of the benchmark may import this package; nothing under
+``fastcache_amd`` does.
+
+Pinning status (what independent check fixes each restatement; see tests/test_oracle_*.py):
+  paged.extract_kv / write_back      closed form dense[s] = pool[table[s // bs], s % bs], brute force
+  presses.knorm_score                float64 brute force of -sqrt(sum k^2)
+  presses.topk_lowest_index          pure-Python sorted() on rows with injected exact ties
+  presses.gather_tokens              integer-patterned payloads, brute-force loops
+  presses.adapter_compress_layer     index arithmetic by hand for streaming_llm / uniform stride
+  presses.snapkv_score               float64 loops on tiny shapes for the composition
+                                     matmul -> softmax -> slice -> reduce -> avg_pool1d -> group reduce;
+                                     the residual choices made by the third-party kvpress package
+                                     (causal mask inside the window, mean vs sum, window inside the
+                                     budget) cannot be checked offline: PARITY UNPINNED for those
+  ccm.*                              float64 loops for Linear/ReLU chain, reshape by hand
+  blocks.*                           invariants of the free deque / ref counts, hand-worked cases
+  attention.decode_attention         float64 loops; flash-attn itself is unavailable offline:
+                                     PARITY UNPINNED beyond the mathematical definition
+"""

@@ -1,0 +1,194 @@
+"""Oracle (test infrastructure): token scoring, selection and gathering.
+
+Two families are restated here.
+
+* The in-tree adapter ``KVPressCompressor._compress_layer``
+  (nanovllm/kernels/kvpress_compressor.py:169-251): one index set per batch row.
+* The kvpress-style presses the reference imports from the third-party ``kvpress`` package
+  (requirements.txt:13, ``kvpress>=0.3.0``, no lock file; call sites
+  utils_ccm/utils_compress.py:22-24, 200-349; nanovllm/autocompress/methods.py:484-491).  The
+  package is not vendored, so its published algorithm is restated: ``ScorerPress.compress`` keeps
+  ``n_kept = int(q_len * (1 - compression_ratio))`` tokens per (batch, kv head) by ``topk`` of
+  ``score`` and gathers K and V; ``KnormPress.score = -keys.norm(dim=-1)``;
+  ``SnapKVPress.score`` is the observation-window attention described at ``snapkv_score``.
+
+Selection order is fixed here (torch.topk leaves ties unspecified): largest score first, ties
+to the lowest index, output in ascending token order.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------------------------
+# kept-token count
+# --------------------------------------------------------------------------------------------
+def ratio_from_factor(compression_factor: float) -> float:
+    """``compression_ratio = 1.0 - 1.0 / compression_factor`` in double
+    (nanovllm/engine/llava_model_runner.py:389, kvpress_compressor.py:328)."""
+    return 1.0 - (1.0 / compression_factor)
+
+
+def n_kept_adapter(seq_len: int, compression_ratio: float) -> int:
+    """kvpress_compressor.py:193-194: ``max(int(S * (1 - r)), 1)`` in double arithmetic."""
+    return max(int(seq_len * (1 - compression_ratio)), 1)
+
+
+def n_kept_press(seq_len: int, compression_ratio: float) -> int:
+    """kvpress ``ScorerPress.compress``: ``int(q_len * (1 - compression_ratio))``."""
+    return int(seq_len * (1 - compression_ratio))
+
+
+# --------------------------------------------------------------------------------------------
+# scores
+# --------------------------------------------------------------------------------------------
+def knorm_score(keys: torch.Tensor) -> torch.Tensor:
+    """kvpress ``KnormPress.score``: ``-keys.norm(dim=-1)``; evaluated in fp32 whatever the
+    storage dtype.  keys ``[B, Hkv, S, D]`` -> ``[B, Hkv, S]`` fp32."""
+    return -torch.linalg.vector_norm(keys.float(), dim=-1)
+
+
+def knorm_mean_score(keys: torch.Tensor) -> torch.Tensor:
+    """kvpress_compressor.py:222-223: ``keys.norm(dim=-1).mean(dim=1)`` in the input dtype,
+    returned as fp32 values (each step rounded to the storage dtype as torch does)."""
+    norms = keys.norm(dim=-1)
+    return norms.mean(dim=1).float()
+
+
+def snapkv_score(queries: torch.Tensor, keys: torch.Tensor, window_size: int, kernel_size: int,
+                 causal_window: bool = True, reduction: str = "mean",
+                 scale: Optional[float] = None) -> torch.Tensor:
+    """kvpress ``SnapKVPress.score`` with pre-rotated window queries.
+
+    queries ``[B, Hq, W, D]`` (the last W positions), keys ``[B, Hkv, S, D]``.
+    logits = Q K^T / sqrt(D) over all S keys of kv head ``hq // G``; with ``causal_window`` the
+    key at position S-W+j is masked for window query i when j > i (the triu mask of
+    ``compute_window_attention``); softmax in fp32; the last W columns are dropped; reduce over the
+    W queries; ``avg_pool1d(kernel, padding=kernel//2, stride=1)`` (zero padding counted in the
+    divisor); reduce over the G query heads of each kv group; the window positions get the global
+    maximum of the tensor so that they are never pruned.  ``reduction`` is 'mean' (kvpress) or
+    'sum' (both reductions as sums); the two differ by the constant factor W*G.
+    Everything after the logits stays in fp32 (kvpress rounds the softmax to the query dtype;
+    this build keeps fp32 scores).  Returns ``[B, Hkv, S]`` fp32.
+    """
+    B, Hq, W, D = queries.shape
+    _, Hkv, S, _ = keys.shape
+    assert W == window_size and S > W, "sequence must be longer than the window"
+    G = Hq // Hkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    k_rep = keys.float().repeat_interleave(G, dim=1)                     # repeat_kv
+    logits = torch.matmul(queries.float(), k_rep.transpose(2, 3)) * scale  # [B,Hq,W,S]
+    if causal_window:
+        mask = torch.full((W, S), float("-inf"))
+        mask = torch.triu(mask, diagonal=S - W + 1)
+        logits = logits + mask
+    attn = F.softmax(logits, dim=-1, dtype=torch.float32)
+    attn = attn[..., :-W]
+    v = attn.mean(dim=-2) if reduction == "mean" else attn.sum(dim=-2)  # [B,Hq,S-W]
+    v = F.avg_pool1d(v, kernel_size=kernel_size, padding=kernel_size // 2, stride=1)
+    v = v.view(B, Hkv, G, S - W)
+    v = v.mean(2) if reduction == "mean" else v.sum(2)
+    return F.pad(v, (0, W), value=v.max().item())
+
+
+# --------------------------------------------------------------------------------------------
+# selection
+# --------------------------------------------------------------------------------------------
+def topk_lowest_index(scores: torch.Tensor, k: int) -> torch.Tensor:
+    """The ``k`` largest entries of each row of ``scores[..., S]``; ties to the lowest index;
+    indices returned ascending (int64).  NaN ranks above +inf and -0 equals +0, as torch.topk
+    orders them."""
+    s = scores.detach().to(torch.float32).numpy()
+    flat = s.reshape(-1, s.shape[-1])
+    out = np.empty((flat.shape[0], k), dtype=np.int64)
+    for r in range(flat.shape[0]):
+        row = flat[r] + 0.0                              # -0 -> +0
+        key = np.where(np.isnan(row), np.inf, row)
+        nan_first = np.isnan(row)
+        # stable sort on descending score: NaN first, then larger scores, ties keep index order
+        order = np.lexsort((np.arange(row.size), -key, ~nan_first))
+        out[r] = np.sort(order[:k])
+    return torch.from_numpy(out.reshape(*s.shape[:-1], k))
+
+
+def near_tie_rows(scores: torch.Tensor, k: int, rel: float = 1e-5) -> torch.Tensor:
+    """Rows whose k-th and (k+1)-th largest scores differ by less than ``rel`` relative: their kept
+    set is not determined at fp32 scoring accuracy and is left out of index comparisons."""
+    s = scores.float()
+    if k <= 0 or k >= s.shape[-1]:
+        return torch.zeros(s.shape[:-1], dtype=torch.bool)
+    top = torch.topk(s, k + 1, dim=-1).values
+    a, b = top[..., k - 1], top[..., k]
+    return (a - b).abs() < rel * a.abs()
+
+
+def gather_tokens(x: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+    """``x.gather(2, idx[..., None].expand(..., D))`` (kvpress_compressor.py:245-249).
+    x ``[B, H, S, D]``; idx ``[B, H, k]`` or ``[B, k]`` (shared by all heads)."""
+    if idx.dim() == 2:
+        idx = idx.unsqueeze(1).expand(-1, x.shape[1], -1)
+    return x.gather(2, idx.unsqueeze(-1).expand(-1, -1, -1, x.shape[-1])).contiguous()
+
+
+# --------------------------------------------------------------------------------------------
+# kvpress-style press = score + select + gather
+# --------------------------------------------------------------------------------------------
+def press_compress(keys: torch.Tensor, values: torch.Tensor, scores: torch.Tensor,
+                   compression_ratio: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """kvpress ``ScorerPress.compress``.  Returns ``(K', V', idx[B, Hkv, n_kept])``."""
+    if compression_ratio == 0:
+        S = keys.shape[2]
+        idx = torch.arange(S).expand(keys.shape[0], keys.shape[1], S)
+        return keys, values, idx
+    n = n_kept_press(keys.shape[2], compression_ratio)
+    idx = topk_lowest_index(scores, n)
+    return gather_tokens(keys, idx), gather_tokens(values, idx), idx
+
+
+# --------------------------------------------------------------------------------------------
+# the in-tree adapter
+# --------------------------------------------------------------------------------------------
+def adapter_indices(method: str, keys: torch.Tensor, compression_ratio: float, n_sink: int = 4,
+                    generator: Optional[torch.Generator] = None) -> Optional[torch.Tensor]:
+    """Index choice of ``KVPressCompressor._compress_layer`` (kvpress_compressor.py:193-238).
+    Returns int64 ``[B, n]`` ascending, or None when nothing is dropped."""
+    B, H, S, D = keys.shape
+    n = n_kept_adapter(S, compression_ratio)
+    if n >= S:                                                        # :197-198
+        return None
+    if method == "streaming_llm":                                     # :201-218
+        sink = min(n_sink, n)
+        recent = max(0, n - sink)
+        if recent > 0 and S > sink + recent:
+            idx = torch.cat([torch.arange(sink), torch.arange(S - recent, S)])
+        elif recent > 0:
+            idx = torch.arange(n)
+        else:
+            idx = torch.arange(sink)
+    elif method == "knorm":                                           # :220-226
+        m = knorm_mean_score(keys)                                    # [B, S]
+        return topk_lowest_index(m, min(n, S))
+    elif method == "random":                                          # :228-232
+        idx = torch.randperm(S, generator=generator)[:min(n, S)].sort().values
+    else:                                                             # :234-238
+        n = min(n, S)
+        step = max(1, S // n)
+        idx = torch.arange(0, S, step).long()[:n]
+    return idx.unsqueeze(0).expand(B, -1)                             # :241-242
+
+
+def adapter_compress_layer(method: str, keys: torch.Tensor, values: torch.Tensor,
+                           compression_ratio: float, n_sink: int = 4,
+                           generator: Optional[torch.Generator] = None
+                           ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``KVPressCompressor._compress_layer`` (kvpress_compressor.py:169-251)."""
+    idx = adapter_indices(method, keys, compression_ratio, n_sink, generator)
+    if idx is None:
+        return keys.contiguous(), values.contiguous()
+    return gather_tokens(keys, idx), gather_tokens(values, idx)
