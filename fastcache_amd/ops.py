@@ -77,9 +77,8 @@ def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size
     check(fn("fc_snapkv_score")(C.byref(keys), queries.data_ptr(), Hq, window, kernel_size,
                                 int(causal_window), scale, out_scale, out.data_ptr(), stride, st),
           "fc_snapkv_score")
-    ws = torch.empty((L,), dtype=torch.float32, device=dev)
     check(fn("fc_snapkv_fill_window")(out.data_ptr(), stride, L, B, keys.num_kv_heads, ptr(seq_lens),
-                                      keys.max_seq_len, window, ws.data_ptr(), st), "fc_snapkv_fill_window")
+                                      keys.max_seq_len, window, st), "fc_snapkv_fill_window")
     return out
 
 

@@ -118,7 +118,7 @@ int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_h
  */
 int fc_snapkv_fill_window(float* scores, int32_t score_stride, int32_t num_layers, int32_t batch,
                           int32_t num_kv_heads, const int32_t* seq_lens, int32_t max_seq_len,
-                          int32_t window, void* workspace /* float[num_layers] */, void* stream);
+                          int32_t window, void* stream);
 
 /*
  * Row-wise top-k with a defined order.  Row r of `rows` score rows has

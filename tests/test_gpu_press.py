@@ -69,3 +69,53 @@ def test_knorm_press_paged_inplace(dev, dtype, shape):
     assert torch.equal(pool.cpu().view(torch.uint8), exp_pool.view(torch.uint8))
     if n_tie == 0:
         assert torch.equal(pool.cpu().view(torch.uint8), ref_pool.view(torch.uint8))
+
+
+def _oracle_snapkv_scores(case, W, ksz, causal, reduction):
+    """[L, B, Hkv, S] fp32 scores from the dense K of every sequence (all sequences share S)."""
+    out = []
+    for l in range(case.dense_k.shape[0]):
+        out.append(opress.snapkv_score(case.queries[l], case.dense_k[l], W, ksz, causal, reduction))
+    return torch.stack(out)
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(num_layers=2, batch=2, num_q_heads=8, num_kv_heads=2, seq_len=300, window=64, ksz=7, dtype=torch.bfloat16),
+    dict(num_layers=1, batch=1, num_q_heads=4, num_kv_heads=4, seq_len=257, window=32, ksz=5, dtype=torch.float16),
+    dict(num_layers=1, batch=2, num_q_heads=14, num_kv_heads=2, seq_len=1000, window=64, ksz=7, dtype=torch.bfloat16),
+    dict(num_layers=1, batch=1, num_q_heads=8, num_kv_heads=1, seq_len=100, window=64, ksz=3, dtype=torch.bfloat16),
+    dict(num_layers=1, batch=1, num_q_heads=2, num_kv_heads=1, seq_len=520, window=48, ksz=7, dtype=torch.float16),
+])
+@pytest.mark.parametrize("causal,reduction", [(True, "mean"), (False, "sum")])
+def test_snapkv_scores_and_selection(dev, cfg, causal, reduction):
+    cfg = dict(cfg)
+    ksz = cfg.pop("ksz")
+    W = cfg["window"]
+    case = synth.snapkv_case(seed=11, keep_dense=True, **cfg)
+    ref = _oracle_snapkv_scores(case, W, ksz, causal, reduction)
+
+    pool = case.kv_cache.to(dev)
+    tables, lens = case.table_tensor(dev), case.lens_tensor(dev)
+    S = max(case.seq_lens)
+    kview = _lib.paged_view(pool[0], tables, lens, S)
+    got = ops.snapkv_score(kview, case.queries.to(dev), W, ksz, causal_window=causal, reduction=reduction,
+                           seq_lens=lens)
+    torch.cuda.synchronize()
+    got = got.cpu()
+    # scores within 1e-3 relative (fp32 accumulation); tiny probabilities get an absolute floor
+    torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-3 * float(ref.abs().mean()))
+
+    # the same scores through a dense (HuggingFace-layout) view
+    dense_k = case.dense_k.to(dev)          # keep alive: the view only holds its address
+    dview = _lib.dense_view(dense_k)
+    got_d = ops.snapkv_score(dview, case.queries.to(dev), W, ksz, causal_window=causal, reduction=reduction)
+    assert torch.equal(got_d.cpu(), got)
+
+    n = opress.n_kept_press(S, 0.75)
+    if n > W:
+        idx = ops.topk_select(got.to(dev), n).cpu().long()
+        ref_idx = opress.topk_lowest_index(ref, n)
+        tie = opress.near_tie_rows(ref[..., :S - W], n - W)
+        assert torch.equal(idx[~tie], ref_idx[~tie])
+        # the observation window always survives
+        assert (idx[..., -W:] == torch.arange(S - W, S)).all()
