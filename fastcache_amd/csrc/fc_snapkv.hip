@@ -27,6 +27,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 #define SK_ROWB 272       // LDS bytes per key row (256 + 16 pad)
 #define SK_NEG (-1.0e30f) // "minus infinity" that stays finite under subtraction
 #define SK_LAZY 40.0f     // allowed excess (log2 units) of a logit over the lane's offset
+#define SK_TBL 1024       // block-table entries of one sequence cached in LDS
 
 template <int DTYPE>
 __device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16 c) {
@@ -50,6 +51,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
   __shared__ __align__(16) char kbuf[2][SK_KT * SK_ROWB];
   __shared__ float vpart[2][NW][SK_KT];
   __shared__ float vraw[4][SK_KT];
+  __shared__ int tbl[SK_TBL];
 
   const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
   const int Hkv = kv.num_kv_heads;
@@ -87,6 +89,13 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
       qf[rb][ks] = ok ? *reinterpret_cast<const uint4*>(qp + ks * 32) : make_uint4(0, 0, 0, 0);
   }
 
+  // this sequence's block-table row, so that the tile loads do not wait on a table read each
+  const bool paged = kv.block_tables != nullptr;
+  const bool tbl_lds = paged && kv.block_shift >= 0 && ((S - 1) >> kv.block_shift) < SK_TBL;
+  if (tbl_lds) {
+    const int nblk = ((S - 1) >> kv.block_shift) + 1;
+    for (int i = tid; i < nblk; i += THREADS) tbl[i] = kv.block_tables[(long long)b * kv.table_stride + i];
+  }
   const char* kbase = kv.base + ((long long)l * kv.stride_layer + (long long)h * kv.stride_head) * 2;
   uint4 pre[CH];
   auto load_tile = [&](int t) {
@@ -97,7 +106,13 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
       const int s = t * SK_KT + key;
       pre[u] = make_uint4(0, 0, 0, 0);
       if (ch < CHUNKS && s < S) {
-        const long long off = fc_token_offset(kv, b, s);
+        long long off;
+        if (tbl_lds) {
+          const int blk = tbl[s >> kv.block_shift];
+          off = blk < 0 ? -1 : (long long)blk * kv.stride_block + (long long)(s & (kv.block_size - 1)) * kv.stride_token;
+        } else {
+          off = fc_token_offset(kv, b, s);
+        }
         if (off >= 0) pre[u] = *reinterpret_cast<const uint4*>(kbase + off * 2 + part * 16);
       }
     }
@@ -110,50 +125,113 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
     }
   };
 
-  // per-lane softmax state for the lane's 2 x 16 query rows (raw-logit units for the offset)
-  float m[2][16], ls[2][16];
+  // per-lane softmax state for the lane's 2 x 16 query rows: nm = -(offset * c), ls = sum of
+  // exp2(logit * c + nm) over the keys this lane has seen
+  float nm[2][16], ls[2][16];
 #pragma unroll
   for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { m[rb][i] = SK_NEG; ls[rb][i] = 0.f; }
+    for (int i = 0; i < 16; ++i) { nm[rb][i] = -SK_NEG; ls[rb][i] = 0.f; }
 
+  __syncthreads();  // tbl
   load_tile(0);
   store_tile(0);
   __syncthreads();
 
-  const int iters = 2 * T;
   const bool always_general = SW < SK_KT;
-  for (int it = 0; it < iters; ++it) {
-    const int t = it < T ? it : it - T;
-    const bool sweep2 = it >= T;
-    const int cur = it & 1;
 
-    if (sweep2 && it == T) {
-      // merge the per-lane states of each row across the 32 lanes of a half-wave, then turn
-      // (offset, sum) into (offset * c, 1 / sum)
+  auto logits = [&](int cur, int cb, f32x16 (&acc)[2]) {
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float mm = m[rb][i], ll = ls[rb][i];
+      for (int i = 0; i < 16; ++i) acc[rb][i] = 0.f;
+    const char* kb = &kbuf[cur][(cb * 32 + lrow) * SK_ROWB + lhalf * 16];
 #pragma unroll
-          for (int o = 1; o < 32; o <<= 1) {
-            const float m2 = __shfl_xor(mm, o, 64), l2 = __shfl_xor(ll, o, 64);
-            const float mn = fmaxf(mm, m2);
-            ll = ll * sk_exp2((mm - mn) * c) + l2 * sk_exp2((m2 - mn) * c);
-            mm = mn;
-          }
-          const int qa = qi[rb] + (i >> 2) * 8 + lhalf * 4 + (i & 3);
-          const bool ok = rb_valid[rb] && qa < W;
-          m[rb][i] = mm * c;
-          ls[rb][i] = ok ? 1.0f / ll : 0.f;
-        }
+    for (int ks = 0; ks < 8; ++ks) {
+      const uint4 bf = *reinterpret_cast<const uint4*>(kb + ks * 32);
+      acc[0] = sk_mfma<DTYPE>(qf[0][ks], bf, acc[0]);
+      acc[1] = sk_mfma<DTYPE>(qf[1][ks], bf, acc[1]);
     }
-    if (sweep2 && t >= 1 && tid < SK_KT) {
+  };
+
+  // ================= sweep 1: per-lane softmax statistics ======================================
+  for (int t = 0; t < T; ++t) {
+    const int cur = t & 1;
+    load_tile(t + 1 < T ? t + 1 : 0);   // the tile after the last one is tile 0 of sweep 2
+    const int tile_end = (t + 1) * SK_KT;
+    const bool masked_tile = tile_end > S || (causal && tile_end > SW + 1);
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      f32x16 acc[2];
+      logits(cur, cb, acc);
+      // keys past the sequence end, and (causal) window keys later than the query, are masked
+      if (masked_tile) {
+        const int s = t * SK_KT + cb * 32 + lrow;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+          // query index of register i is qi[rb] + lhalf*4 + (i/4)*8 + i%4: compare against constants
+          const int d = causal ? s - SW - qi[rb] - lhalf * 4 : -1;
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (s >= S || d > ((i >> 2) * 8 + (i & 3))) acc[rb][i] = SK_NEG;
+        }
+      }
+      // largest exponent argument relative to the lane's current offsets: does any offset have to move?
+      float worst = -1.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        worst = fmaxf(worst, fmaxf(fmaf(acc[0][i], c, nm[0][i]), fmaf(acc[1][i], c, nm[1][i])));
+      // A lane-row whose keys were all masked so far still has the SK_NEG offset, for which only
+      // exact differences are safe; shapes with fewer scored keys than one tile therefore always
+      // take the general update (after tile 0 every lane-row has a real offset otherwise).
+      if (always_general || __any(worst > SK_LAZY)) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const float tt = -acc[rb][i] * c;
+            const float mn = fminf(nm[rb][i], tt);
+            ls[rb][i] = ls[rb][i] * sk_exp2(mn - nm[rb][i]) + sk_exp2(mn - tt);
+            nm[rb][i] = mn;
+          }
+      } else {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) ls[rb][i] += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
+      }
+    }
+    store_tile(cur ^ 1);
+    __syncthreads();
+  }
+
+  // merge the per-lane states of each row across the 32 lanes of a half-wave and fold the
+  // normaliser into the offset: p = exp2(logit * c + nm), nm = -(max * c) - log2(sum)
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float mm = nm[rb][i], ll = ls[rb][i];
+#pragma unroll
+      for (int o = 1; o < 32; o <<= 1) {
+        const float m2 = __shfl_xor(mm, o, 64), l2 = __shfl_xor(ll, o, 64);
+        const float mn = fminf(mm, m2);
+        ll = ll * sk_exp2(mn - mm) + l2 * sk_exp2(mn - m2);
+        mm = mn;
+      }
+      const int qa = qi[rb] + (i >> 2) * 8 + lhalf * 4 + (i & 3);
+      const bool ok = rb_valid[rb] && qa < W;
+      nm[rb][i] = ok ? mm - __builtin_amdgcn_logf(ll) : SK_NEG;   // v_log_f32 is log2
+    }
+
+  // ================= sweep 2: probabilities, per-key sums, moving average ======================
+  for (int t = 0; t < T; ++t) {
+    const int cur = (T + t) & 1;
+    if (t >= 1 && tid < SK_KT) {
       // fold the wavefronts' partial sums of tile t-1 (fixed order) into the ring
       float v = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) v += vpart[(it - 1) & 1][w][tid];
+      for (int w = 0; w < NW; ++w) v += vpart[cur ^ 1][w][tid];
       vraw[(t - 1) & 3][tid] = v;
       // moving average for tile t-3: its neighbours t-4 .. t-2 are complete
       if (t >= 3) {
@@ -169,86 +247,30 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
         }
       }
     }
-
-    const bool more = it + 1 < iters;
-    if (more) load_tile((it + 1) < T ? it + 1 : it + 1 - T);
-
-    // ---- logits of this tile, one 32-key column block at a time: 2 row blocks x 32 keys -------
-    const int tile_end = (t + 1) * SK_KT;
-    const bool masked_tile = !sweep2 && (tile_end > S || (causal && tile_end > SW + 1));
+    const bool more = t + 1 < T;
+    if (more) load_tile(t + 1);
 #pragma unroll
     for (int cb = 0; cb < 2; ++cb) {
       f32x16 acc[2];
+      logits(cur, cb, acc);
+      float vs = 0.f;
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[rb][i] = 0.f;
-      const char* kb = &kbuf[cur][(cb * 32 + lrow) * SK_ROWB + lhalf * 16];
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const uint4 bf = *reinterpret_cast<const uint4*>(kb + ks * 32);
-        acc[0] = sk_mfma<DTYPE>(qf[0][ks], bf, acc[0]);
-        acc[1] = sk_mfma<DTYPE>(qf[1][ks], bf, acc[1]);
-      }
-
-      if (!sweep2) {
-        // keys past the sequence end, and (causal) window keys later than the query, are masked
-        if (masked_tile) {
-          const int s = t * SK_KT + cb * 32 + lrow;
-#pragma unroll
-          for (int rb = 0; rb < 2; ++rb) {
-            // query index of register i is qi[rb] + lhalf*4 + (i/4)*8 + i%4: compare against constants
-            const int d = causal ? s - SW - qi[rb] - lhalf * 4 : -1;
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-              if (s >= S || d > ((i >> 2) * 8 + (i & 3))) acc[rb][i] = SK_NEG;
-          }
-        }
-        // exponent arguments relative to the lane's current offsets; the largest one tells
-        // whether any offset has to move
-        float worst = -1.f;
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) worst = fmaxf(worst, (acc[rb][i] - m[rb][i]) * c);
-        // A lane-row whose keys were all masked so far still has the SK_NEG offset; its
-        // differences must be formed before scaling ((-1e30) - (-1e30) = 0 exactly), so shapes with
-        // fewer scored keys than one tile always take the general update.
-        if (always_general || __any(worst > SK_LAZY)) {
-#pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const float mn = fmaxf(m[rb][i], acc[rb][i]);
-              ls[rb][i] = ls[rb][i] * sk_exp2((m[rb][i] - mn) * c) + sk_exp2((acc[rb][i] - mn) * c);
-              m[rb][i] = mn;
-            }
-        } else {
-#pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) ls[rb][i] += sk_exp2((acc[rb][i] - m[rb][i]) * c);
-        }
-      } else {
-        float vs = 0.f;
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) vs = fmaf(sk_exp2(fmaf(acc[rb][i], c, -m[rb][i])), ls[rb][i], vs);
-        vs += __shfl_xor(vs, 32, 64);
-        if (lane < 32) vpart[cur][wave][cb * 32 + lane] = vs;
-      }
+        for (int i = 0; i < 16; ++i) vs += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
+      vs += __shfl_xor(vs, 32, 64);
+      if (lane < 32) vpart[cur][wave][cb * 32 + lane] = vs;
     }
-
     if (more) store_tile(cur ^ 1);
     __syncthreads();
   }
+  const int last_buf = (2 * T - 1) & 1;
 
   // ---- drain: last tile's sums, then the moving average of the last three tiles ------------
   if (tid < SK_KT) {
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) v += vpart[(iters - 1) & 1][w][tid];
+    for (int w = 0; w < NW; ++w) v += vpart[last_buf][w][tid];
     vraw[(T - 1) & 3][tid] = v;
   }
   __syncthreads();

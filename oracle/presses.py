@@ -104,14 +104,19 @@ def topk_lowest_index(scores: torch.Tensor, k: int) -> torch.Tensor:
     """The ``k`` largest entries of each row of ``scores[..., S]``; ties to the lowest index;
     indices returned ascending (int64).  NaN ranks above +inf and -0 equals +0, as torch.topk
     orders them."""
-    s = scores.detach().to(torch.float32).numpy()
+    sc = scores.detach().to(torch.float32) + 0.0             # -0 -> +0
+    if not torch.isnan(sc).any():
+        # stable ascending sort of the negated scores: larger score first, ties keep index order
+        order = torch.sort(-sc, dim=-1, stable=True).indices[..., :k]
+        return torch.sort(order, dim=-1).values
+    s = sc.numpy()
     flat = s.reshape(-1, s.shape[-1])
     out = np.empty((flat.shape[0], k), dtype=np.int64)
     for r in range(flat.shape[0]):
-        row = flat[r] + 0.0                              # -0 -> +0
+        row = flat[r]
         key = np.where(np.isnan(row), np.inf, row)
         nan_first = np.isnan(row)
-        # stable sort on descending score: NaN first, then larger scores, ties keep index order
+        # NaN first, then larger scores, ties keep index order
         order = np.lexsort((np.arange(row.size), -key, ~nan_first))
         out[r] = np.sort(order[:k])
     return torch.from_numpy(out.reshape(*s.shape[:-1], k))
