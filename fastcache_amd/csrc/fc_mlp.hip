@@ -1,0 +1,345 @@
+// CCM compressor: Linear(cf*128 -> 128) -> ReLU -> Linear(128 -> 128) -> ReLU -> Linear(128 -> 128)
+// over rows made of `cf` consecutive tokens of one head, fp16/bf16 storage, fp32 accumulation,
+// each Linear's output rounded to the storage dtype.  Reads and writes the caches in place.
+//
+// Shape of the work: one workgroup of 4 wavefronts (one per SIMD, full register file) per group of (sequence, head) columns of one
+// layer; a wavefront owns 64 rows of one column per iteration.  The three GEMMs are chained
+// through registers without any transposition:
+//   layer 1 (transposed)  H1^T = W1 * X^T   A = W1 rows from LDS, B = X token rows straight
+//                                           from HBM (16-byte loads, each element read once);
+//   layer 2 (transposed)  H2^T = W2 * H1^T  B = layer 1's accumulators, converted in place;
+//   layer 3               Y = H2 * W3^T     A = layer 2's accumulators, B = W3 rows from LDS.
+// A 32x32 accumulator block holds, per lane, 16 values of one token column; taking registers
+// 0..7 and 8..15 as two k-steps gives a complete, if permuted, set of 16 k indices across the two
+// half-waves, so the next layer's weights are stored in LDS with the same permutation
+// ([0-3, 8-11 | 4-7, 12-15] inside every group of 16) and no data moves between lanes.
+// Layer 3's accumulators hold 32 consecutive output features across a half-wave, so its stores
+// are contiguous 64-byte segments.
+//
+// W2 and W3 (permuted) stay in LDS for the life of the workgroup; W1 streams through a double
+// buffer one 128-column chunk (one source token) at a time, shared by the wavefronts; each
+// wavefront prefetches the X rows of the next chunk into registers while it multiplies the current one.
+// In-place safety: output row j lands on token dst_start + j <= seg_start + cf*j; all rows of an
+// iteration are read before the workgroup barrier that precedes its stores, and later iterations
+// read tokens no earlier iteration writes.
+#include "fc_common.h"
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+#define ML_WAVES 4
+#define ML_THREADS (ML_WAVES * 64)
+#define ML_ROWB 272                 // LDS bytes per weight row: 128 elements + 16 bytes of padding
+#define ML_WBYTES (128 * ML_ROWB)   // one 128 x 128 weight block in LDS
+
+template <int DTYPE>
+__device__ __forceinline__ f32x16 ml_mfma(const uint4& a, const uint4& b, f32x16 c) {
+  if constexpr (DTYPE == FC_BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+}
+
+// two fp32 -> packed storage dtype, round to nearest even
+template <int DTYPE>
+__device__ __forceinline__ unsigned ml_pack2(float a, float b) {
+  f32x2 v = {a, b};
+  if constexpr (DTYPE == FC_BF16)
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+  else
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2));
+}
+
+template <int DTYPE>
+__device__ __forceinline__ float ml_to_float(unsigned short h) {
+  return DTYPE == FC_BF16 ? fc_bf16_to_float(h) : fc_half_to_float(h);
+}
+
+// relu(round(acc + bias)) for 8 consecutive accumulator registers -> one MFMA operand.
+// Registers i0..i0+7 of a block hold features fb + (i/4)*8 + lhalf*4 + i%4.
+template <int DTYPE>
+__device__ __forceinline__ uint4 ml_act_operand(const f32x16& acc, int i0, const float* __restrict__ bias, int fb,
+                                                int lhalf) {
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int i = i0 + e;
+    v[e] = acc[i] + bias[fb + (i >> 2) * 8 + lhalf * 4 + (i & 3)];
+  }
+  unsigned p[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    // ReLU after rounding equals rounding after ReLU; a negative pair member is zeroed in the packed word
+    unsigned w = ml_pack2<DTYPE>(v[2 * e], v[2 * e + 1]);
+    if (w & 0x8000u) w &= 0xffff0000u;
+    if (w & 0x80000000u) w &= 0x0000ffffu;
+    p[e] = w;
+  }
+  return make_uint4(p[0], p[1], p[2], p[3]);
+}
+
+template <int DTYPE>
+__global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView dst, const char* __restrict__ w1,
+                                                            const char* __restrict__ b1, const char* __restrict__ w2,
+                                                            const char* __restrict__ b2, const char* __restrict__ w3,
+                                                            const char* __restrict__ b3, int cf, int seg_start,
+                                                            int c_rows, int dst_start, int wpc, int ncols) {
+  extern __shared__ __align__(16) char lds[];
+  char* w1buf = lds;                       // 2 x ML_WBYTES
+  char* w2buf = lds + 2 * ML_WBYTES;       // permuted
+  char* w3buf = lds + 3 * ML_WBYTES;       // permuted
+  float* bias = reinterpret_cast<float*>(lds + 4 * ML_WBYTES);  // [3][128] fp32
+
+  const int l = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int cols_per_wg = ML_WAVES / wpc;
+  const int col = blockIdx.x * cols_per_wg + wave / wpc;
+  const int sub = wave % wpc;
+  const bool col_ok = col < ncols;
+  const int H = src.num_kv_heads;
+  const int b = col_ok ? col / H : 0, h = col_ok ? col - (col / H) * H : 0;
+  const int K1 = cf * 128;
+
+  // ---- resident weights: W2, W3 with the k permutation, biases as fp32 ------------------------------
+  {
+    const char* w2l = w2 + (long long)l * 128 * 128 * 2;
+    const char* w3l = w3 + (long long)l * 128 * 128 * 2;
+    // 8-byte pieces: piece p of a row holds k = 4p .. 4p+3; inside each group of 4 pieces the order
+    // becomes [0, 2, 1, 3]
+    for (int i = tid; i < 128 * 32; i += ML_THREADS) {
+      const int n = i >> 5, p = i & 31;
+      const int q = p & 3;
+      const int pp = (p & ~3) | ((q == 1) ? 2 : (q == 2) ? 1 : q);
+      *reinterpret_cast<uint2*>(w2buf + n * ML_ROWB + pp * 8) = *reinterpret_cast<const uint2*>(w2l + (n * 128 + p * 4) * 2);
+      *reinterpret_cast<uint2*>(w3buf + n * ML_ROWB + pp * 8) = *reinterpret_cast<const uint2*>(w3l + (n * 128 + p * 4) * 2);
+    }
+    for (int i = tid; i < 384; i += ML_THREADS) {
+      const int which = i >> 7, n = i & 127;
+      const char* bp = which == 0 ? b1 : which == 1 ? b2 : b3;
+      bias[i] = ml_to_float<DTYPE>(*reinterpret_cast<const unsigned short*>(bp + ((long long)l * 128 + n) * 2));
+    }
+  }
+
+  // W1 chunk kc covers columns [kc*128, kc*128+128) of W1[l]: 2048 pieces of 16 bytes
+  constexpr int WCH = 2048 / ML_THREADS;
+  const char* w1l = w1 + (long long)l * 128 * K1 * 2;
+  uint4 wpre[WCH];
+  auto w1_load = [&](int kc) {
+#pragma unroll
+    for (int u = 0; u < WCH; ++u) {
+      const int ch = tid + u * ML_THREADS;  // row n = ch / 16, part = ch % 16
+      wpre[u] = *reinterpret_cast<const uint4*>(w1l + ((long long)(ch >> 4) * K1 + kc * 128) * 2 + (ch & 15) * 16);
+    }
+  };
+  auto w1_store = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < WCH; ++u) {
+      const int ch = tid + u * ML_THREADS;
+      *reinterpret_cast<uint4*>(w1buf + buf * ML_WBYTES + (ch >> 4) * ML_ROWB + (ch & 15) * 16) = wpre[u];
+    }
+  };
+
+  const int rows_per_iter = 64 * wpc;
+  const int n_iter = (c_rows + rows_per_iter - 1) / rows_per_iter;
+  const int q_total = n_iter * cf;      // W1 chunk q = (iteration q / cf, token kc = q % cf) sits in buffer q & 1
+  const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lhalf * 16;
+  char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2;
+
+  // X rows of chunk q for this lane: 2 token blocks x 8 k-steps of 16 bytes
+  auto x_load = [&](uint4 (&xf)[2][8], int q) {
+    const int it = q / cf, kc = q - it * cf;
+    const int row0 = it * rows_per_iter + sub * 64;
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+      const int r = row0 + tb * 32 + lrow;
+      long long off = -1;
+      if (col_ok && r < c_rows) off = fc_token_offset(src, b, seg_start + cf * r + kc);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+        xf[tb][ks] = off >= 0 ? *reinterpret_cast<const uint4*>(sbase + off * 2 + ks * 32) : make_uint4(0, 0, 0, 0);
+    }
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+
+  // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+1's rows load into `xnext`;
+  // after the last chunk of an iteration, layers 2 and 3 and the stores.
+  auto stage = [&](uint4 (&xcur)[2][8], uint4 (&xnext)[2][8], int q) {
+    const int it = q / cf, kc = q - it * cf;
+    const bool more = q + 1 < q_total;
+    if (more) x_load(xnext, q + 1);
+    __syncthreads();  // chunk q is in w1buf[q & 1]; every wavefront is done with chunk q - 1
+    if (more) w1_load((kc + 1 < cf) ? kc + 1 : 0);
+    {
+      const char* wa = w1buf + (q & 1) * ML_WBYTES + lrow * ML_ROWB + lhalf * 16;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+          const uint4 a = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + ks * 32);
+          acc[mb][0] = ml_mfma<DTYPE>(a, xcur[0][ks], acc[mb][0]);
+          acc[mb][1] = ml_mfma<DTYPE>(a, xcur[1][ks], acc[mb][1]);
+        }
+      }
+    }
+    if (more) w1_store((q + 1) & 1);
+    if (kc != cf - 1) return;
+
+    // ---- layer 2: H2^T = W2 * H1^T, B operand taken from layer 1's accumulators -------------------
+    uint4 hf[2][8];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb) {
+        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0, bias, mb * 32, lhalf);
+        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8, bias, mb * 32, lhalf);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+      }
+    {
+      const char* wa = w2buf + lrow * ML_ROWB + lhalf * 16;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+          const uint4 a = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + g * 32);
+          acc[mb][0] = ml_mfma<DTYPE>(a, hf[0][g], acc[mb][0]);
+          acc[mb][1] = ml_mfma<DTYPE>(a, hf[1][g], acc[mb][1]);
+        }
+      }
+    }
+    // ---- layer 3: Y = H2 * W3^T, A operand taken from layer 2's accumulators ---------------------
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb) {
+        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0, bias + 128, mb * 32, lhalf);
+        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8, bias + 128, mb * 32, lhalf);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+      }
+    {
+      // acc[nb][tb] now accumulates Y[tb block rows][nb block features]
+      const char* wb = w3buf + lrow * ML_ROWB + lhalf * 16;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+          const uint4 bw = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB + g * 32);
+          acc[nb][0] = ml_mfma<DTYPE>(hf[0][g], bw, acc[nb][0]);
+          acc[nb][1] = ml_mfma<DTYPE>(hf[1][g], bw, acc[nb][1]);
+        }
+      }
+    }
+    // every wavefront of the group has consumed this iteration's source rows: stores may alias them
+    __syncthreads();
+    const int row0 = it * rows_per_iter + sub * 64;
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        // registers 4*i4 .. 4*i4+3 are 4 consecutive rows
+        const int r0 = row0 + tb * 32 + i4 * 8 + lhalf * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = r0 + e;
+          long long off = -1;
+          if (col_ok && r < c_rows) off = fc_token_offset(dst, b, dst_start + r);
+          if (off >= 0) {
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+              const float y = acc[nb][tb][i4 * 4 + e] + bias[256 + nb * 32 + lrow];
+              const unsigned w = ml_pack2<DTYPE>(y, 0.f);
+              *reinterpret_cast<unsigned short*>(dbase + off * 2 + (nb * 32 + lrow) * 2) = (unsigned short)(w & 0xffff);
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+  };
+
+  uint4 xa[2][8], xb[2][8];
+  w1_load(0);
+  w1_store(0);
+  x_load(xa, 0);
+  for (int q = 0; q < q_total; q += 2) {
+    stage(xa, xb, q);
+    if (q + 1 < q_total) stage(xb, xa, q + 1);
+  }
+}
+
+extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int32_t seg_start, int32_t count,
+                              int32_t dst_start, void* stream);
+
+extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int32_t cf,
+                          int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream) {
+  const char* who = "fc_ccm_mlp";
+  int rc;
+  if ((rc = fc_check_view(src, who)) || (rc = fc_check_view(dst, who))) return rc;
+  FC_REQUIRE(src->dtype == dst->dtype && src->num_layers == dst->num_layers && src->batch == dst->batch &&
+                 src->num_kv_heads == dst->num_kv_heads,
+             FC_EINVAL, "%s: source and destination views disagree", who);
+  FC_REQUIRE(src->dtype == FC_F16 || src->dtype == FC_BF16, FC_EUNSUPPORTED, "%s: fp16/bf16 caches only", who);
+  FC_REQUIRE(w && w->w1 && w->b1 && w->w2 && w->b2 && w->w3 && w->b3, FC_EINVAL, "%s: null weights", who);
+  FC_REQUIRE(cf >= 1 && cf <= 64, FC_EINVAL, "%s: compression factor %d out of range", who, cf);
+  FC_REQUIRE(seg_start >= 0 && seg_len >= 0 && dst_start >= 0, FC_EINVAL, "%s: negative range", who);
+  FC_REQUIRE((int64_t)seg_start + seg_len <= src->max_seq_len, FC_EINVAL,
+             "%s: segment [%d, %d) exceeds the source view's max_seq_len %d", who, seg_start, seg_start + seg_len,
+             src->max_seq_len);
+  const int c = seg_len / cf;
+  const int rem = seg_len - c * cf;
+  FC_REQUIRE((int64_t)dst_start + c + rem <= dst->max_seq_len, FC_EINVAL,
+             "%s: output [%d, %d) exceeds the destination view's max_seq_len %d", who, dst_start,
+             dst_start + c + rem, dst->max_seq_len);
+  hipStream_t st = (hipStream_t)stream;
+  if (c > 0) {
+    const int ncols = src->batch * src->num_kv_heads;
+    int wpc = 1;
+    while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && 64 * wpc * 2 <= c) wpc *= 2;
+    const int cols_per_wg = ML_WAVES / wpc;
+    dim3 grid((ncols + cols_per_wg - 1) / cols_per_wg, src->num_layers);
+    const size_t lds = 4 * ML_WBYTES + 3 * 128 * sizeof(float);
+    KvView s = fc_make_view(src), d = fc_make_view(dst);
+    if (src->dtype == FC_BF16) {
+      static bool attr_bf16 = false;
+      if (!attr_bf16) {
+        hipFuncSetAttribute((const void*)mlp_kernel<FC_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_bf16 = true;
+      }
+      hipLaunchKernelGGL((mlp_kernel<FC_BF16>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,
+                         (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,
+                         (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);
+    } else {
+      static bool attr_f16 = false;
+      if (!attr_f16) {
+        hipFuncSetAttribute((const void*)mlp_kernel<FC_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_f16 = true;
+      }
+      hipLaunchKernelGGL((mlp_kernel<FC_F16>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,
+                         (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,
+                         (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);
+    }
+    FC_CHECK_LAUNCH(who);
+  }
+  if (rem > 0) return fc_copy_tokens(src, dst, seg_start + c * cf, rem, dst_start + c, stream);
+  return FC_OK;
+}

@@ -1,0 +1,94 @@
+"""GPU parity: decode paged attention, KV append and length advance vs the CPU oracle.
+
+Tolerance: attention outputs within 2e-2 absolute in fp16/bf16 (fp32 softmax and accumulation on
+both sides; the reference's flash-attn rounds the probabilities to the storage dtype before the PV
+product, this kernel keeps them in fp32).
+"""
+import pytest
+import torch
+
+from fastcache_amd import _lib, ops, synth
+from oracle import attention as oattn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,lens", [
+    (4, 4, [1, 255, 256, 257, 700]),
+    (8, 2, [33, 1024, 513]),
+    (14, 2, [300, 17]),
+    (16, 1, [129, 0, 600]),
+])
+def test_decode_attention(dev, dtype, Hq, Hkv, lens):
+    L, B = 2, len(lens)
+    case = synth.make_paged_case(seed=21, num_layers=L, batch=B, num_kv_heads=Hkv, seq_lens=[max(n, 1) for n in lens],
+                                 dtype=dtype, reserve_tokens=8)
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(L, B, Hq, 128, generator=g).to(dtype)
+    width = max(len(t) for t in case.block_tables) + 2
+    tables = case.table_tensor("cpu", width)
+    lens_t = torch.tensor(lens, dtype=torch.int32)
+    scale = 128 ** -0.5
+
+    pool = case.kv_cache.to(dev)
+    tab_d, len_d = tables.to(dev), lens_t.to(dev)
+    max_len = width * 256
+    kview = _lib.paged_view(pool[0], tab_d, None, max_len)
+    vview = _lib.paged_view(pool[1], tab_d, None, max_len)
+    ws = ops.decode_attn_workspace(B, Hq, max_len, dev)
+    for layer in range(L):
+        ref = oattn.decode_attention(q[layer], case.kv_cache[0, layer], case.kv_cache[1, layer], lens_t, tables, scale)
+        got = ops.decode_attn(kview, vview, layer, q[layer].to(dev), len_d, scale, ws)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(got.cpu().float(), ref.float(), atol=2e-2, rtol=0)
+        # much tighter in practice: fp32 math on both sides, one rounding at the end
+        assert float((got.cpu().float() - ref.float()).abs().max()) < 4e-3
+
+
+def test_block_permutation_invariance(dev):
+    """Moving the pages around (with the table following) leaves the output bit-identical."""
+    dtype, Hq, Hkv, lens = torch.float16, 8, 4, [900, 300, 77]
+    case = synth.make_paged_case(seed=2, num_layers=1, batch=3, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype)
+    nb = case.kv_cache.shape[2]
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(1))
+    pool2 = torch.empty_like(case.kv_cache)
+    pool2[:, :, perm] = case.kv_cache                       # block i moves to perm[i]
+    tables1 = case.table_tensor("cpu")
+    tables2 = torch.where(tables1 >= 0, perm[tables1.clamp_min(0).long()].int(), tables1)
+    q = torch.randn(3, Hq, 128, generator=torch.Generator().manual_seed(3)).to(dtype).to(dev)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device=dev)
+    outs = []
+    for pool, tab in ((case.kv_cache, tables1), (pool2, tables2)):
+        p, t = pool.to(dev), tab.to(dev)
+        kv = [_lib.paged_view(p[i], t, None, t.shape[1] * 256) for i in range(2)]
+        ws = ops.decode_attn_workspace(3, Hq, t.shape[1] * 256, dev)
+        outs.append(ops.decode_attn(kv[0], kv[1], 0, q, lens_d, 128 ** -0.5, ws).cpu())
+    assert torch.equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_store_kv_and_advance(dev, dtype):
+    L, B, Hkv = 3, 4, 2
+    lens = [5, 255, 256, 511]
+    case = synth.make_paged_case(seed=9, num_layers=L, batch=B, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype,
+                                 reserve_tokens=4)
+    g = torch.Generator().manual_seed(1)
+    k_new = torch.randn(L, B, Hkv, 128, generator=g).to(dtype)
+    v_new = torch.randn(L, B, Hkv, 128, generator=g).to(dtype)
+    ref = case.kv_cache.clone()
+    for layer in range(L):
+        slots = torch.tensor([oattn.decode_slot(case.block_tables[b], lens[b]) for b in range(B)])
+        oattn.store_kv(ref[0, layer], ref[1, layer], k_new[layer], v_new[layer], slots)
+
+    pool = case.kv_cache.to(dev)
+    tab = case.table_tensor(dev)
+    len_d = torch.tensor(lens, dtype=torch.int32, device=dev)
+    max_len = tab.shape[1] * 256
+    kview = _lib.paged_view(pool[0], tab, None, max_len)
+    vview = _lib.paged_view(pool[1], tab, None, max_len)
+    ops.store_kv(kview, vview, k_new.to(dev), v_new.to(dev), len_d)
+    ops.advance_lens(len_d, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(pool.cpu().view(torch.uint8), ref.view(torch.uint8))
+    assert len_d.cpu().tolist() == [n + 1 for n in lens]

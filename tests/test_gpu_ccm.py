@@ -1,0 +1,99 @@
+"""GPU parity: the CCM MLP compressor kernel vs the CPU oracle.
+
+Tolerance.  Both sides accumulate in fp32 and round to the storage dtype after every Linear, but in
+a different summation order, so a hidden activation can round to the neighbouring fp16/bf16 value
+and move the final output by about one unit in the last place of the storage dtype (2^-10 relative
+for fp16, 2^-7 for bf16).  The check is therefore: error norm / reference norm <= 1e-3, and every
+element within 1e-3 * max|ref| + 2 ulp(storage) of the reference.
+"""
+import pytest
+import torch
+
+from fastcache_amd import _lib, ops, synth
+from oracle import ccm as occm
+from oracle import paged as opaged
+
+pytestmark = pytest.mark.gpu
+
+
+def stacked(sd, group, L, dtype, dev):
+    out = []
+    for i in (0, 3, 6):
+        out.append(torch.stack([sd[f"{group}.{l}.{i}.weight"] for l in range(L)]).to(dtype).contiguous().to(dev))
+        out.append(torch.stack([sd[f"{group}.{l}.{i}.bias"] for l in range(L)]).to(dtype).contiguous().to(dev))
+    return tuple(out)
+
+
+def assert_mlp_close(got, ref, dtype):
+    got, ref = got.float(), ref.float()
+    ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    scale = float(ref.abs().max())
+    rel = float((got - ref).norm() / ref.norm())
+    assert rel <= 1e-3, f"relative error norm {rel:.3e}"
+    err = (got - ref).abs()
+    bound = 1e-3 * scale + 2 * ulp * ref.abs().clamp_min(scale * 2.0 ** -14)
+    assert bool((err <= bound).all()), f"max excess {float((err - bound).max()):.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cf,S,img", [(2, 640, 576), (5, 1003, 0), (2, 70, 37), (3, 200, 64)])
+def test_ccm_mlp_paged_inplace(dev, dtype, cf, S, img):
+    L, B, H = 2, 3, 4
+    case = synth.ccm_case(seed=5, num_layers=L, batch=B, num_kv_heads=H, image_tokens=img, text_tokens=S - img,
+                          dtype=dtype)
+    sd = occm.reference_init_state_dict("linear_decouple", L, 128, cf, seed=7)
+    it_len = [img, S - img]
+    # oracle: extract -> LinearDecouple forward -> write back, per sequence
+    ref_pool = case.kv_cache.clone()
+    for tab in case.block_tables:
+        hf = opaged.extract_kv(ref_pool, tab, S)
+        out = occm.linear_decouple_forward(hf, it_len, sd, cf, 1)
+        opaged.write_back(ref_pool, out, tab)
+    C = occm.compressed_length(S, it_len, cf, 1)
+
+    pool = case.kv_cache.to(dev)
+    tables, lens = case.table_tensor(dev), case.lens_tensor(dev)
+    views = [_lib.paged_view(pool[p], tables, lens, S) for p in range(2)]
+    groups = {"image": ("compress_ik", "compress_iv"), "text": ("compress_tk", "compress_tv")}
+    w = {g: stacked(sd, g, L, dtype, dev) for pair in groups.values() for g in pair}
+    dst = 0
+    for seg, (s0, n) in (("image", (0, img)), ("text", (img, S - img))):
+        if n == 0:
+            continue
+        for plane in range(2):
+            ops.ccm_mlp(views[plane], views[plane], w[groups[seg][plane]], cf, s0, n, dst)
+        dst += n // cf + n % cf
+    torch.cuda.synchronize()
+    assert dst == C
+    got = pool.cpu()
+    # compare token by token through the tables (the MLP rows and the copied remainder rows)
+    for tab in case.block_tables:
+        g = opaged.extract_kv(got, tab, C)
+        r = opaged.extract_kv(ref_pool, tab, C)
+        for (gk, gv), (rk, rv) in zip(g, r):
+            assert_mlp_close(gk, rk, dtype)
+            assert_mlp_close(gv, rv, dtype)
+    # everything past the compressed length is untouched
+    for b, tab in enumerate(case.block_tables):
+        full_g = opaged.extract_kv(got, tab, S)
+        full_o = opaged.extract_kv(case.kv_cache, tab, S)
+        for (gk, gv), (ok, ov) in zip(full_g, full_o):
+            assert torch.equal(gk[:, :, C:], ok[:, :, C:]) and torch.equal(gv[:, :, C:], ov[:, :, C:])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_ccm_mlp_dense_out_of_place(dev, dtype):
+    L, B, H, S, cf = 1, 2, 3, 333, 4
+    torch.manual_seed(3)
+    k = torch.randn(L, B, H, S, 128).to(dtype)
+    sd = occm.reference_init_state_dict("hybrid", L, 128, cf, seed=9)
+    ref_k, _ = occm.compress_segment(k[0], k[0], sd, "compress_tk", "compress_tk", 0, cf, 1)
+    C = ref_k.shape[2]
+    kd = k.to(dev)
+    out = torch.zeros(L, B, H, C, 128, dtype=dtype, device=dev)
+    ops.ccm_mlp(_lib.dense_view(kd), _lib.dense_view(out), stacked(sd, "compress_tk", L, dtype, dev), cf, 0, S, 0)
+    torch.cuda.synchronize()
+    assert_mlp_close(out[0].cpu(), ref_k, dtype)
+    # remainder tokens are copied bit-exactly
+    n = (S // cf) * cf
+    assert torch.equal(out[0, :, :, S // cf:].cpu(), k[0, :, :, n:])
