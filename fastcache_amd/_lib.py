@@ -68,6 +68,7 @@ SIGNATURES = {
     "fc_ccm_mlp": (C.c_int, [_V, _V, C.POINTER(FcMlpWeights), _I, _I, _I, _I, _VP]),
     "fc_copy_tokens": (C.c_int, [_V, _V, _I, _I, _I, _VP]),
     "fc_store_kv": (C.c_int, [_V, _V, _VP, _VP, _VP, _VP]),
+    "fc_store_kv_slots": (C.c_int, [_VP, C.c_int64, _VP, C.c_int64, _VP, _VP, _VP, _I, _I, _I, _VP]),
     "fc_advance_lens": (C.c_int, [_VP, _I, _I, _VP]),
     "fc_decode_attn_workspace_bytes": (C.c_int64, [_I, _I, _I]),
     "fc_decode_attn": (C.c_int, [_V, _V, _I, _VP, _VP, _I, _VP, _F, _VP, C.c_int64, _VP]),

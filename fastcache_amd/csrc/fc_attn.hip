@@ -241,6 +241,20 @@ __global__ __launch_bounds__(256) void store_kv_kernel(KvView kc, KvView vc, con
   }
 }
 
+// one new row per token i: cache[slot_mapping[i]] <- key[i], value[i]; a row is row_bytes long
+__global__ __launch_bounds__(256) void store_slots_kernel(const char* __restrict__ key, long long key_stride_b,
+                                                          const char* __restrict__ value, long long value_stride_b,
+                                                          char* __restrict__ k_cache, char* __restrict__ v_cache,
+                                                          const int* __restrict__ slot_mapping, int row_bytes) {
+  const int i = blockIdx.x;
+  const long long slot = slot_mapping[i];
+  if (slot < 0) return;
+  for (int o = threadIdx.x * 16; o < row_bytes; o += 256 * 16) {
+    *reinterpret_cast<uint4*>(k_cache + slot * row_bytes + o) = *reinterpret_cast<const uint4*>(key + i * key_stride_b + o);
+    *reinterpret_cast<uint4*>(v_cache + slot * row_bytes + o) = *reinterpret_cast<const uint4*>(value + i * value_stride_b + o);
+  }
+}
+
 __global__ void advance_lens_kernel(int* lens, int n, int delta) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n && lens[i] >= 0) lens[i] += delta;
@@ -265,6 +279,26 @@ extern "C" int fc_store_kv(const fc_kv_view* k_cache, const fc_kv_view* v_cache,
   else
     hipLaunchKernelGGL((store_kv_kernel<2>), grid, dim3(256), 0, st, k, v, (const char*)k_new, (const char*)v_new,
                        context_lens);
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_store_kv_slots(const void* key, int64_t key_stride, const void* value, int64_t value_stride,
+                                 void* k_cache, void* v_cache, const int32_t* slot_mapping, int32_t num_tokens,
+                                 int32_t row_elems, int32_t dtype, void* stream) {
+  const char* who = "fc_store_kv_slots";
+  FC_REQUIRE(key && value && k_cache && v_cache && slot_mapping, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EINVAL, "%s: unknown dtype %d", who, dtype);
+  FC_REQUIRE(num_tokens >= 0 && row_elems > 0, FC_EINVAL, "%s: bad sizes", who);
+  const int eb = fc_elem_bytes(dtype);
+  FC_REQUIRE(((int64_t)row_elems * eb) % 16 == 0 && (key_stride * eb) % 16 == 0 && (value_stride * eb) % 16 == 0,
+             FC_EINVAL, "%s: rows and strides must be multiples of 16 bytes", who);
+  FC_REQUIRE((((uintptr_t)key | (uintptr_t)value | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0, FC_EINVAL,
+             "%s: pointers must be 16-byte aligned", who);
+  if (num_tokens == 0) return FC_OK;
+  hipLaunchKernelGGL(store_slots_kernel, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream, (const char*)key,
+                     (long long)key_stride * eb, (const char*)value, (long long)value_stride * eb, (char*)k_cache,
+                     (char*)v_cache, slot_mapping, row_elems * eb);
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }

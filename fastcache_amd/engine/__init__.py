@@ -1,0 +1,3 @@
+"""Host-side mirror of the reference's nano-vllm engine pieces that the compression path touches."""
+from .block_manager import Block, BlockManager  # noqa: F401
+from .sequence import Sequence, SequenceStatus  # noqa: F401

@@ -1,0 +1,205 @@
+"""The compression hooks of nano-vllm's model runner over a paged KV pool
+(nanovllm/engine/llava_model_runner.py: ``allocate_kv_cache`` :498-539, ``prepare_decode``
+:637-674, ``compress_kv_cache_batch`` :712-793, ``_extract_kv_cache_fast`` :824-872,
+``_write_compressed_kv_cache_fast`` :874-912, ``start_background_compression`` :1046-1094).
+
+The model forward is not part of this build; a ``PagedKVRunner`` owns the pool and offers the same
+method names, bookkeeping dictionaries and return values, so an engine loop written against the
+reference runner drives it unchanged.  Compressors that expose ``paged_forward`` (every compressor
+of this package) are run in place on the pages for all sequences of equal length at once; any
+other callable goes through extract -> call -> write back, with the copies done by HIP kernels.
+"""
+from __future__ import annotations
+
+import threading
+import time
+from typing import Dict, List, Optional, Sequence as Seq, Tuple
+
+import torch
+
+from .. import _lib, ops
+from ..utils.context import set_context
+from .sequence import Sequence
+
+LayerKV = Tuple[torch.Tensor, torch.Tensor]
+
+
+class PagedKVRunner:
+    def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int, num_blocks: int, dtype: torch.dtype,
+                 device, block_size: int = 256, compressor=None, batched_compressor=None, image_token_len: int = 576):
+        self.num_hidden_layers, self.num_key_value_heads, self.head_dim = num_layers, num_kv_heads, head_dim
+        self.block_size = block_size
+        self.device = torch.device(device)
+        self.kv_cache = torch.zeros(2, num_layers, num_blocks, block_size, num_kv_heads, head_dim, dtype=dtype,
+                                    device=self.device)
+        self.compressor = compressor
+        self.batched_compressor = batched_compressor
+        self.use_batched_compressor = batched_compressor is not None
+        self.image_token_len = image_token_len
+        self._compressed_lens: Dict[int, int] = {}
+        self._blocks_to_free: Dict[int, List[int]] = {}
+        self._lock = threading.Lock()
+        self._compress_stream: Optional[torch.cuda.Stream] = None
+
+    # -- tables -----------------------------------------------------------------------------------
+    def preare_block_tables(self, seqs: Seq[Sequence]) -> torch.Tensor:
+        """int32 ``[B, max blocks]`` right-padded with -1 (llava_model_runner.py:541-549; the
+        reference spells it this way)."""
+        width = max(len(s.block_table) for s in seqs)
+        rows = [s.block_table + [-1] * (width - len(s.block_table)) for s in seqs]
+        return torch.tensor(rows, dtype=torch.int32, pin_memory=True).to(self.device, non_blocking=True)
+
+    def _table_and_lens(self, tables: Seq[Seq[int]], lens: Seq[int]):
+        width = max(len(t) for t in tables)
+        tt = torch.tensor([list(t) + [-1] * (width - len(t)) for t in tables], dtype=torch.int32, device=self.device)
+        return tt, torch.tensor(list(lens), dtype=torch.int32, device=self.device)
+
+    # -- paged <-> HuggingFace layout ----------------------------------------------------------------
+    def _extract_kv_cache_fast(self, block_table: List[int], seq_len: int) -> List[LayerKV]:
+        """One ``(K, V)`` pair per layer, each ``[1, Hkv, S, D]``, copied out of the pages."""
+        L, H, D = self.num_hidden_layers, self.num_key_value_heads, self.head_dim
+        need = -(-seq_len // self.block_size)
+        table = [b for b in block_table[:need] if b >= 0]
+        seq_len = min(seq_len, len(table) * self.block_size)
+        if seq_len == 0:
+            return []
+        tt, ll = self._table_and_lens([table], [seq_len])
+        out = torch.empty((2, L, 1, H, seq_len, D), dtype=self.kv_cache.dtype, device=self.device)
+        for p in range(2):
+            ops.copy_tokens(_lib.paged_view(self.kv_cache[p], tt, ll, seq_len), _lib.dense_view(out[p]), 0, seq_len, 0)
+        return [(out[0, l], out[1, l]) for l in range(L)]
+
+    def _write_compressed_kv_cache_fast(self, compressed_kv: List[LayerKV], block_table: List[int]) -> None:
+        """Write ``[1, Hkv, C, D]`` pairs into the leading blocks of ``block_table``; slots past ``C``
+        keep their contents."""
+        if not compressed_kv:
+            return
+        C = compressed_kv[0][0].shape[2]
+        table = []
+        for b in block_table:
+            if b < 0:
+                break
+            table.append(b)
+        C = min(C, len(table) * self.block_size)
+        if C == 0:
+            return
+        tt, ll = self._table_and_lens([table], [C])
+        for p in range(2):
+            src = torch.stack([kv[p] for kv in compressed_kv])        # [L, 1, Hkv, C, D]
+            ops.copy_tokens(_lib.dense_view(src), _lib.paged_view(self.kv_cache[p], tt, ll, C), 0, C, 0)
+
+    # -- compression ---------------------------------------------------------------------------------
+    def _active_compressor(self):
+        if self.use_batched_compressor and self.batched_compressor is not None:
+            return self.batched_compressor
+        return self.compressor
+
+    def _compress_enqueue(self, seqs: Seq[Sequence], image_len: int) -> Tuple[int, int]:
+        """Enqueue the compression of ``seqs`` on the current stream and update the bookkeeping;
+        returns (elements before, elements after)."""
+        comp = self._active_compressor()
+        L, H, D = self.num_hidden_layers, self.num_key_value_heads, self.head_dim
+        orig = after = 0
+        result: Dict[int, int] = {}
+        if hasattr(comp, "paged_forward"):
+            groups: Dict[int, List[Sequence]] = {}
+            for s in seqs:
+                groups.setdefault(len(s), []).append(s)
+            for S, group in groups.items():
+                tt, ll = self._table_and_lens([s.block_table for s in group], [S] * len(group))
+                it_len = [image_len, max(1, S - image_len)]
+                C = comp.paged_forward(self.kv_cache, tt, ll, S, it_len)
+                for s in group:
+                    result[s.seq_id] = C
+                orig += 2 * L * H * D * S * len(group)
+                after += 2 * L * H * D * C * len(group)
+        else:
+            for s in seqs:
+                S = len(s)
+                hf = self._extract_kv_cache_fast(s.block_table, S)
+                it_len = [image_len, max(1, S - image_len)]
+                with torch.no_grad():
+                    out = comp(hf, it_len=it_len)
+                self._write_compressed_kv_cache_fast(out, s.block_table)
+                result[s.seq_id] = out[0][0].shape[2]
+                orig += sum(k.numel() + v.numel() for k, v in hf)
+                after += sum(k.numel() + v.numel() for k, v in out)
+        with self._lock:
+            for s in seqs:
+                C = result[s.seq_id]
+                self._compressed_lens[s.seq_id] = C
+                keep = -(-C // self.block_size)
+                if len(s.block_table) > keep:
+                    self._blocks_to_free[s.seq_id] = s.block_table[keep:]
+        return orig, after
+
+    def compress_kv_cache_batch(self, seqs: List[Sequence], image_len: Optional[int] = None) -> Tuple[float, float]:
+        """Compress the KV of ``seqs`` in place; returns ``(seconds, elements before / after)`` after a
+        device synchronisation (llava_model_runner.py:712-793)."""
+        if self._active_compressor() is None:
+            return 0.0, 1.0
+        if image_len is None:
+            image_len = self.image_token_len
+        t0 = time.time()
+        orig, after = self._compress_enqueue(seqs, image_len)
+        torch.cuda.synchronize()
+        return time.time() - t0, (orig / after if after > 0 else 1.0)
+
+    def get_blocks_to_free(self, seq_id: int) -> List[int]:
+        return self._blocks_to_free.pop(seq_id, [])
+
+    def get_compressed_block_count(self, seq_id: int) -> int:
+        if seq_id not in self._compressed_lens:
+            return -1
+        return -(-self._compressed_lens[seq_id] // self.block_size)
+
+    def clear_compressed_lens(self, seq_ids: Optional[List[int]] = None) -> None:
+        with self._lock:
+            if seq_ids is None:
+                self._compressed_lens.clear()
+            else:
+                for i in seq_ids:
+                    self._compressed_lens.pop(i, None)
+
+    # -- asynchronous variant: one side stream, two events --------------------------------------------
+    def start_background_compression(self, seqs: List[Sequence], image_len: Optional[int] = None):
+        """Enqueue the compression on the side stream behind everything already on the current stream;
+        returns the event that fires when it is done (llava_model_runner.py:1046-1094).  Bookkeeping
+        is updated immediately; consumers must ``wait_compression`` before touching those sequences."""
+        if self._active_compressor() is None:
+            return None
+        if image_len is None:
+            image_len = self.image_token_len
+        if self._compress_stream is None:
+            self._compress_stream = torch.cuda.Stream(device=self.device)
+        ready = torch.cuda.Event()
+        ready.record()
+        self._compress_stream.wait_event(ready)
+        with torch.cuda.stream(self._compress_stream):
+            self._compress_enqueue(seqs, image_len)
+            done = torch.cuda.Event()
+            done.record(self._compress_stream)
+        return done
+
+    def wait_compression(self, event) -> None:
+        if event is not None:
+            event.synchronize()
+
+    # -- decode metadata ------------------------------------------------------------------------------
+    def prepare_decode(self, seqs: List[Sequence]):
+        """``positions = context_lens = kv_cache_len``; the new token's slot is position ``kv_cache_len``
+        of the sequence (llava_model_runner.py:637-674)."""
+        input_ids, positions, slots, lens = [], [], [], []
+        for s in seqs:
+            n = s.kv_cache_len
+            input_ids.append(s.last_token)
+            positions.append(n)
+            lens.append(n)
+            bi, pos = divmod(n, self.block_size)
+            blk = s.block_table[bi] if bi < len(s.block_table) else s.block_table[-1]
+            slots.append(blk * self.block_size + pos)
+        mk = lambda x, dt: torch.tensor(x, dtype=dt, pin_memory=True).to(self.device, non_blocking=True)
+        input_ids, positions = mk(input_ids, torch.int64), mk(positions, torch.int64)
+        set_context(False, slot_mapping=mk(slots, torch.int32), context_lens=mk(lens, torch.int32),
+                    block_tables=self.preare_block_tables(seqs))
+        return input_ids, positions

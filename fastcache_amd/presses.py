@@ -1,0 +1,226 @@
+"""kvpress-style press objects with the call surface the reference uses, computed by HIP kernels.
+
+The reference takes its presses from the third-party ``kvpress`` package
+(utils_ccm/utils_compress.py:22-24) and wraps them in ``ScorerPressWithTime``
+(utils_compress.py:200-324): dataclass fields ``compression_ratio`` (+ ``window_size``,
+``kernel_size``, ``n_sink``), ``score(module, hidden_states, keys, values, attentions, kwargs)``
+-> ``[B, Hkv, S]``, ``compress(...)`` -> ``(keys, values)``, ``forward_hook`` registered on every
+``layer.self_attn`` by the context manager ``with press(model): ...``, and ``press_select``.
+This module provides the same objects.  Scoring, selection and gathering run in
+libfastcache_hip; torch only allocates and, for SnapKV inside a live model, projects the window
+queries.
+
+Two choices the reference leaves open are fixed here: ties in the selection go to the lowest token
+index, and the kept tokens come out in ascending position order (``torch.topk`` guarantees neither).
+"""
+from __future__ import annotations
+
+import math
+import time
+from contextlib import contextmanager
+from dataclasses import dataclass
+from typing import Generator, Optional
+
+import torch
+from torch import nn
+
+from . import _lib, ops
+
+
+def _cache_layer_kv(cache, layer_idx):
+    if hasattr(cache, "key_cache"):                       # transformers 4.x DynamicCache
+        return cache.key_cache[layer_idx], cache.value_cache[layer_idx]
+    layer = cache.layers[layer_idx]                       # transformers 5.x
+    return layer.keys, layer.values
+
+
+def _set_cache_layer_kv(cache, layer_idx, k, v):
+    if hasattr(cache, "key_cache"):
+        cache.key_cache[layer_idx], cache.value_cache[layer_idx] = k, v
+    else:
+        cache.layers[layer_idx].keys, cache.layers[layer_idx].values = k, v
+
+
+def _seen_tokens(cache, layer_idx):
+    if hasattr(cache, "seen_tokens"):
+        return cache.seen_tokens
+    return cache.get_seq_length(layer_idx)
+
+
+@dataclass
+class ScorerPress:
+    """Prune the ``compression_ratio`` fraction of tokens with the lowest ``score`` in every
+    (batch, kv head) row, during pre-filling only."""
+    compression_ratio: float = 0.0
+
+    def __post_init__(self):
+        assert 0 <= self.compression_ratio < 1, "Compression ratio must be between 0 and 1"
+        self.totalTime = 0
+
+    def reset_timeCheck(self):
+        """utils_compress.py:202-203."""
+        self.totalTime = 0
+
+    # -- to be provided by each press -------------------------------------------------------------
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        raise NotImplementedError
+
+    # -- selection + gather -------------------------------------------------------------------------
+    def n_kept(self, q_len: int) -> int:
+        return int(q_len * (1 - self.compression_ratio))
+
+    def select(self, scores: torch.Tensor, n_kept: int) -> torch.Tensor:
+        """int32 ``[B, Hkv, n_kept]`` ascending positions of the ``n_kept`` best scores per row."""
+        return ops.topk_select(scores.contiguous(), n_kept)
+
+    def compress(self, module, hidden_states, keys, values, attentions, kwargs):
+        if self.compression_ratio == 0:
+            return keys, values
+        scores = self.score(module, hidden_states, keys, values, attentions, kwargs)
+        q_len = hidden_states.shape[1] if hidden_states is not None else keys.shape[2]
+        n = self.n_kept(q_len)
+        B, H, S, D = keys.shape
+        idx = self.select(scores, n).view(1, B, H, n)
+        out_k = torch.empty((B, H, n, D), dtype=keys.dtype, device=keys.device)
+        out_v = torch.empty_like(out_k)
+        ops.compact(_lib.dense_view(keys), _lib.dense_view(values), _lib.dense_view(out_k), _lib.dense_view(out_v), idx)
+        return out_k, out_v
+
+    # -- HuggingFace hook protocol (utils_compress.py:209-299) ---------------------------------------
+    def forward_hook(self, module: nn.Module, input, kwargs: dict, output):
+        cache = kwargs.get("past_key_value", kwargs.get("past_key_values"))
+        if cache is None:
+            cache = output[-1]
+        attentions = output[1] if len(output) == 3 else None
+        hidden_states = kwargs["hidden_states"]
+        q_len = hidden_states.shape[1]
+        if _seen_tokens(cache, module.layer_idx) > q_len:      # decoding: leave the cache alone
+            return output
+        keys, values = _cache_layer_kv(cache, module.layer_idx)
+        start = time.time()
+        keys, values = self.compress(module, hidden_states, keys, values, attentions, kwargs)
+        _set_cache_layer_kv(cache, module.layer_idx, keys, values)
+        self.totalTime += time.time() - start
+        return output
+
+    @contextmanager
+    def __call__(self, model) -> Generator:
+        layers = model.model.layers if hasattr(model, "model") and hasattr(model.model, "layers") else model.layers
+        hooks = []
+        try:
+            for layer in layers:
+                hooks.append(layer.self_attn.register_forward_hook(self.forward_hook, with_kwargs=True))
+            yield
+        finally:
+            for h in hooks:
+                h.remove()
+
+
+@dataclass
+class KnormPress(ScorerPress):
+    """``score = -||k||_2``: keys with a small norm are kept."""
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        return ops.knorm_score(_lib.dense_view(keys), keys.device)[0]
+
+
+@dataclass
+class SnapKVPress(ScorerPress):
+    """Attention of the last ``window_size`` queries over the prefix, average-pooled.
+
+    ``causal_window`` applies the causal mask among the window positions (kvpress does);
+    ``reduction`` is 'mean' (kvpress) or 'sum' over the window queries and over the query heads of a
+    group — the two differ by the constant ``window_size * group``;  with ``window_in_budget`` (kvpress)
+    the always-kept window counts towards ``n_kept``, otherwise it is kept on top of it.
+    Scores stay in fp32 (kvpress rounds the softmax to the query dtype).
+    """
+    compression_ratio: float = 0.0
+    window_size: int = 64
+    kernel_size: int = 5
+    causal_window: bool = True
+    reduction: str = "mean"
+    window_in_budget: bool = True
+
+    def n_kept(self, q_len: int) -> int:
+        n = int(q_len * (1 - self.compression_ratio))
+        return n if self.window_in_budget else min(q_len, n + self.window_size)
+
+    def window_queries(self, module, hidden_states, kwargs) -> torch.Tensor:
+        """Rotated queries of the last ``window_size`` positions, ``[B, Hq, W, D]``: given directly as
+        ``kwargs['queries']`` (synthetic runs), or projected from ``hidden_states`` with the attention
+        module's own ``q_proj`` (+ ``q_norm``) and the rotary ``position_embeddings``."""
+        if kwargs is not None and kwargs.get("queries") is not None:
+            return kwargs["queries"]
+        W = self.window_size
+        bsz = hidden_states.shape[0]
+        num_heads = module.config.num_attention_heads
+        q = module.q_proj(hidden_states[:, -W:]).view(bsz, W, num_heads, module.head_dim)
+        if hasattr(module, "q_norm"):
+            q = module.q_norm(q)
+        q = q.transpose(1, 2)
+        cos, sin = kwargs["position_embeddings"]
+        cos, sin = cos[:, -W:].unsqueeze(1), sin[:, -W:].unsqueeze(1)
+        half = q.shape[-1] // 2
+        rot = torch.cat((-q[..., half:], q[..., :half]), dim=-1)
+        return (q * cos + rot * sin).contiguous()
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        S = keys.shape[2]
+        assert S > self.window_size, "Query length should be greater than the window size"
+        q = self.window_queries(module, hidden_states, kwargs)
+        head_dim = keys.shape[-1]
+        return ops.snapkv_score(_lib.dense_view(keys), q.to(keys.dtype), self.window_size, self.kernel_size,
+                                self.causal_window, self.reduction, 1.0 / math.sqrt(head_dim))[0]
+
+
+@dataclass
+class StreamingLLMPress(ScorerPress):
+    """Keep the first ``n_sink`` tokens and the most recent ones."""
+    compression_ratio: float = 0.0
+    n_sink: int = 4
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        q_len = hidden_states.shape[1] if hidden_states is not None else keys.shape[2]
+        assert q_len > self.n_sink, f"Input should contain more tokens than n_sink={self.n_sink}"
+        n_pruned = q_len - int(q_len * (1 - self.compression_ratio))
+        scores = torch.ones(keys.shape[:3], dtype=torch.float32, device=keys.device)
+        scores[:, :, self.n_sink:self.n_sink + n_pruned] = 0
+        return scores
+
+
+@dataclass
+class RandomPress(ScorerPress):
+    """Uniformly random scores (baseline)."""
+    compression_ratio: float = 0.0
+    seed: Optional[int] = None
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        g = None
+        if self.seed is not None:
+            g = torch.Generator(device=keys.device).manual_seed(self.seed)
+        return torch.rand(keys.shape[:3], dtype=torch.float32, device=keys.device, generator=g)
+
+
+# names the reference gives its timed subclasses (utils_compress.py:302-324)
+KnormPressWithTime = KnormPress
+SnapKVPressWithTime = SnapKVPress
+StreamingLLMPressWithTime = StreamingLLMPress
+RandomPressWithTime = RandomPress
+
+
+def press_select(compression_method: str = "Knorm", compression_ratio: float = 0.8) -> ScorerPress:
+    """utils_compress.py:327-349.  'ExpectedAttention', 'TOVA' and 'Quantized' are not part of this
+    build and raise; any other name gives the Knorm press, as in the reference."""
+    if compression_method == "StreamingLLM":
+        press = StreamingLLMPress(compression_ratio=compression_ratio)
+    elif compression_method == "RandomPress":
+        press = RandomPress(compression_ratio=compression_ratio)
+    elif compression_method == "SnapKV":
+        press = SnapKVPress(compression_ratio=compression_ratio)
+    elif compression_method in ("ExpectedAttention", "TOVA", "Quantized"):
+        raise NotImplementedError(f"press '{compression_method}' is outside the KV-cache compression path "
+                                  "built here (Knorm, SnapKV, StreamingLLM, RandomPress)")
+    else:
+        press = KnormPress(compression_ratio=compression_ratio)
+    press.reset_timeCheck()
+    return press

@@ -1,0 +1,2 @@
+"""Host-side mirror of the reference's ``utils_ccm`` compressor modules, running on HIP kernels."""
+from .module_ccm import KVCacheHybridCompressor, KVCacheLinearDecoupleCompressor  # noqa: F401

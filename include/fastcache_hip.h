@@ -191,6 +191,18 @@ int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst,
 int fc_store_kv(const fc_kv_view* k_cache, const fc_kv_view* v_cache,
                 const void* k_new, const void* v_new, const int32_t* context_lens, void* stream);
 
+/*
+ * The same append with host-computed slots: for token i < num_tokens,
+ *   k_cache[slot_mapping[i]] <- key[i], v_cache[slot_mapping[i]] <- value[i],
+ * a row being row_elems = num_kv_heads*head_dim contiguous elements; key/value rows are
+ * key_stride/value_stride elements apart; k_cache/v_cache are one layer's planes viewed as
+ * [num_blocks*block_size][row_elems].  Negative slots are skipped.
+ * Replaces store_kvcache(key, value, k_cache, v_cache, slot_mapping) (nanovllm/layers/attention.py:32-39).
+ */
+int fc_store_kv_slots(const void* key, int64_t key_stride, const void* value, int64_t value_stride,
+                      void* k_cache, void* v_cache, const int32_t* slot_mapping, int32_t num_tokens,
+                      int32_t row_elems, int32_t dtype, void* stream);
+
 /* context_lens[b] += delta for b < batch where context_lens[b] >= 0 (device side, graph-replayable). */
 int fc_advance_lens(int32_t* context_lens, int32_t batch, int32_t delta, void* stream);
 

@@ -1,0 +1,322 @@
+"""GPU parity of the reference-surface objects: CCM modules, the kvpress adapter, press objects and
+the runner / engine hooks, each against the CPU oracle on the same seeded inputs."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from fastcache_amd import synth
+from fastcache_amd.engine import BlockManager, Sequence
+from fastcache_amd.engine.kv_runner import PagedKVRunner
+from fastcache_amd.engine.llm_hooks import free_compressed_blocks
+from fastcache_amd.kernels import BatchedGEMMCompressor, KVPressCompressor, MiniCPMKVCompressor
+from fastcache_amd.presses import KnormPress, RandomPress, SnapKVPress, StreamingLLMPress
+from fastcache_amd.utils_ccm import KVCacheHybridCompressor, KVCacheLinearDecoupleCompressor
+from oracle import ccm as occm
+from oracle import paged as opaged
+from oracle import pipeline as opipe
+from oracle import presses as opress
+from test_gpu_ccm import assert_mlp_close
+from test_host_logic import llava_cfg, minicpm_cfg
+
+pytestmark = pytest.mark.gpu
+
+
+def rand_kv(L, B, H, S, dtype, seed=0, permuted=True):
+    """Per-layer (k, v) in the layout the runner hands to compressors: [B, H, S, D] views of [B, S, H, D]."""
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for _ in range(L):
+        k = torch.randn(B, S, H, 128, generator=g).to(dtype)
+        v = torch.randn(B, S, H, 128, generator=g).to(dtype)
+        out.append((k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)) if permuted else
+                   (k.permute(0, 2, 1, 3).contiguous(), v.permute(0, 2, 1, 3).contiguous()))
+    return out
+
+
+def to_dev(kv, dev):
+    return [(k.to(dev), v.to(dev)) for k, v in kv]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_decouple_module(dev, dtype):
+    L, B, H, S, cf = 2, 2, 4, 77, 2
+    torch.manual_seed(3)
+    m = KVCacheLinearDecoupleCompressor(llava_cfg(L, H), compression_factor=cf).to(dev).to(dtype).eval()
+    sd = occm.reference_init_state_dict("linear_decouple", L, 128, cf, seed=3)
+    kv = rand_kv(L, B, H, S, dtype)
+    ref = occm.linear_decouple_forward(kv, [41, 36], sd, cf, 1)
+    out = m(to_dev(kv, dev), it_len=[41, 36])
+    assert len(out) == L
+    for (ok, ov), (rk, rv) in zip(out, ref):
+        assert ok.is_contiguous() and ok.shape == rk.shape and ok.dtype == dtype
+        assert_mlp_close(ok.cpu(), rk, dtype)
+        assert_mlp_close(ov.cpu(), rv, dtype)
+    # a checkpoint in the reference's state-dict layout loads and changes the result accordingly
+    sd2 = occm.reference_init_state_dict("linear_decouple", L, 128, cf, seed=4)
+    m.load_state_dict(sd2)
+    ref2 = occm.linear_decouple_forward(kv, [41, 36], sd2, cf, 1)
+    out2 = m(to_dev(kv, dev), it_len=[41, 36])
+    assert_mlp_close(out2[1][0].cpu(), ref2[1][0], dtype)
+
+
+def test_hybrid_and_minicpm_modules(dev):
+    dtype, L, B, H, S = torch.bfloat16, 2, 1, 4, 203
+    torch.manual_seed(8)
+    h = KVCacheHybridCompressor(minicpm_cfg(L), compression_factor=5, min_seq_len=2).to(dev).to(dtype).eval()
+    hsd = occm.reference_init_state_dict("hybrid", L, 128, 5, seed=8)
+    kv = rand_kv(L, B, H, S, dtype, seed=1)
+    ref = occm.hybrid_forward(kv, [0, S], hsd, 5, 2)
+    out = h(to_dev(kv, dev), it_len=[0, S])
+    for (ok, ov), (rk, rv) in zip(out, ref):
+        assert_mlp_close(ok.cpu(), rk, dtype)
+        assert_mlp_close(ov.cpu(), rv, dtype)
+    with pytest.raises(TypeError):
+        h(to_dev(kv, dev), it_len=[64, S - 64])
+    # image segment too short to compress is passed through unchanged
+    ref_p = occm.hybrid_forward(kv, [7, S - 7], hsd, 5, 2)
+    out_p = h(to_dev(kv, dev), it_len=[7, S - 7])
+    assert torch.equal(out_p[0][0][:, :, :7].cpu(), kv[0][0][:, :, :7])
+    assert_mlp_close(out_p[0][1].cpu(), ref_p[0][1], dtype)
+    # short sequences come back unchanged (min_seq_len guard)
+    short = rand_kv(L, B, H, 6, dtype, seed=2)
+    out_s = h(to_dev(short, dev), it_len=[0, 6])
+    assert torch.equal(out_s[0][0].cpu(), short[0][0])
+
+    torch.manual_seed(9)
+    mc = MiniCPMKVCompressor(minicpm_cfg(L)).to(dev).to(dtype).eval()
+    msd = occm.reference_init_state_dict("minicpm", L, 128, 5, seed=9)
+    for it_len in ([0, S], [60, S - 60]):
+        ref_m = occm.minicpm_forward(kv, it_len, msd, 5, 2)
+        out_m = mc(to_dev(kv, dev), it_len=it_len)
+        assert out_m[0][0].shape == ref_m[0][0].shape
+        assert_mlp_close(out_m[1][0].cpu(), ref_m[1][0], dtype)
+
+
+def test_batched_compressor_equals_original(dev):
+    dtype, L, B, H, S, cf = torch.float16, 3, 2, 2, 64, 2
+    torch.manual_seed(2)
+    orig = KVCacheLinearDecoupleCompressor(llava_cfg(L, H), compression_factor=cf).to(dev).to(dtype).eval()
+    bat = BatchedGEMMCompressor(num_layers=L, num_heads=H, head_dim=128, compression_factor=cf)
+    bat.load_from_original_compressor(orig)
+    kv = to_dev(rand_kv(L, B, H, S, dtype, seed=5), dev)
+    a = orig(kv, it_len=[40, 24])
+    b = bat(kv, it_len=[40, 24])
+    for (ak, av), (bk, bv) in zip(a, b):
+        assert torch.equal(ak, bk) and torch.equal(av, bv)          # same kernel, same weights: bit-identical
+    part = bat.compress_layers(kv, 1, 3, it_len=[40, 24])
+    assert len(part) == 2 and torch.equal(part[0][0], a[1][0]) and torch.equal(part[1][1], a[2][1])
+    assert bat.compress_layers(kv, 2, 2) == []
+
+
+@pytest.mark.parametrize("method", ["streaming_llm", "knorm", "snapkv", "h2o", "random"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kvpress_adapter(dev, method, dtype):
+    L, B, H, S = 2, 3, 4, 150
+    comp = KVPressCompressor(method=method, compression_ratio=1.0 - 1.0 / 3)
+    kv = rand_kv(L, B, H, S, dtype, seed=7)
+    out = comp(to_dev(kv, dev), it_len=[10, 140])
+    n = comp.get_compressed_length(S)
+    for (k, v), (ok, ov) in zip(kv, out):
+        assert ok.shape == (B, H, n, 128) and ok.is_contiguous()
+        if method == "random":
+            # RNG-dependent: kept rows are rows of the input, in ascending position order, same for K and V
+            pos = [(k[0, 0] == ok[0, 0, j].cpu()).all(-1).nonzero()[0, 0].item() for j in range(n)]
+            assert pos == sorted(set(pos))
+            assert torch.equal(ov[0, 0].cpu(), v[0, 0, pos])
+            continue
+        rk, rv = opress.adapter_compress_layer(method, k, v, comp.compression_ratio)
+        if method == "knorm":
+            m = opress.knorm_mean_score(k)
+            tie = opress.near_tie_rows(m, n)
+            if dtype == torch.bfloat16:      # bf16 means collide often; only untied rows are defined
+                tie |= (torch.sort(m, -1).values.diff(dim=-1) == 0).any(-1)
+            sel = ~tie
+            assert torch.equal(ok.cpu()[sel], rk[sel]) and torch.equal(ov.cpu()[sel], rv[sel])
+        else:
+            assert torch.equal(ok.cpu(), rk) and torch.equal(ov.cpu(), rv)
+    # nothing to drop: inputs returned contiguous
+    same = KVPressCompressor("knorm", 0.0)(to_dev(kv, dev))
+    assert torch.equal(same[0][0].cpu(), kv[0][0])
+
+
+def test_press_objects_compress(dev):
+    dtype, B, Hq, Hkv, S, W = torch.bfloat16, 2, 8, 2, 400, 64
+    g = torch.Generator().manual_seed(3)
+    k = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    q = torch.randn(B, Hq, W, 128, generator=g).to(dtype)
+    hidden = torch.zeros(B, S, 1)
+    kd, vd = k.to(dev), v.to(dev)
+    # Knorm
+    ck, cv = KnormPress(0.5).compress(None, hidden, kd, vd, None, {})
+    sc = opress.knorm_score(k)
+    rk, rv, ridx = opress.press_compress(k, v, sc, 0.5)
+    tie = opress.near_tie_rows(sc, 200)
+    assert torch.equal(ck.cpu()[~tie], rk[~tie]) and torch.equal(cv.cpu()[~tie], rv[~tie])
+    # SnapKV with the rotated window queries handed in
+    press = SnapKVPress(compression_ratio=0.75, window_size=W, kernel_size=7)
+    ck, cv = press.compress(None, hidden, kd, vd, None, {"queries": q.to(dev)})
+    sc = opress.snapkv_score(q, k, W, 7)
+    rk, rv, _ = opress.press_compress(k, v, sc, 0.75)
+    tie = opress.near_tie_rows(sc[..., :S - W], 100 - W)
+    assert ck.shape == (B, Hkv, 100, 128)
+    assert torch.equal(ck.cpu()[~tie], rk[~tie]) and torch.equal(cv.cpu()[~tie], rv[~tie])
+    got_sc = press.score(None, hidden, kd, vd, None, {"queries": q.to(dev)})
+    torch.testing.assert_close(got_sc.cpu(), sc, rtol=1e-3, atol=1e-3 * float(sc.abs().mean()))
+    # StreamingLLM: sinks + most recent tokens
+    ck, _ = StreamingLLMPress(0.5, n_sink=4).compress(None, hidden, kd, vd, None, {})
+    assert torch.equal(ck.cpu(), torch.cat([k[:, :, :4], k[:, :, 204:]], dim=2))
+    # Random: seeded, right size, rows of the input
+    ck, _ = RandomPress(0.5, seed=1).compress(None, hidden, kd, vd, None, {})
+    assert ck.shape == (B, Hkv, 200, 128)
+
+
+class _FakeAttn(torch.nn.Module):
+    """Attention stand-in that appends K/V to a cache object the way HF layers do."""
+
+    def __init__(self, layer_idx):
+        super().__init__()
+        self.layer_idx = layer_idx
+
+    def forward(self, hidden_states=None, past_key_value=None, k=None, v=None):
+        past_key_value.key_cache[self.layer_idx] = k
+        past_key_value.value_cache[self.layer_idx] = v
+        past_key_value.seen_tokens = k.shape[2]
+        return hidden_states, None, past_key_value
+
+
+def test_press_hook_protocol(dev):
+    """``with press(model)`` prunes the cache during pre-fill and leaves decode steps alone."""
+    L, B, H, S = 2, 1, 2, 64
+    layers = torch.nn.ModuleList([torch.nn.Module() for _ in range(L)])
+    for i, lay in enumerate(layers):
+        lay.self_attn = _FakeAttn(i)
+    model = SimpleNamespace(model=SimpleNamespace(layers=layers))
+    cache = SimpleNamespace(key_cache=[None] * L, value_cache=[None] * L, seen_tokens=0)
+    kv = to_dev(rand_kv(L, B, H, S, torch.float16, seed=11, permuted=False), dev)
+    hidden = torch.zeros(B, S, 8, device=dev)
+    press = KnormPress(0.5)
+    with press(model):
+        for i, lay in enumerate(layers):
+            lay.self_attn(hidden_states=hidden, past_key_value=cache, k=kv[i][0], v=kv[i][1])
+    assert all(kc.shape[2] == 32 for kc in cache.key_cache) and press.totalTime > 0
+    # decode step: cache longer than the query -> untouched
+    cache.seen_tokens = 33
+    with press(model):
+        layers[0].self_attn(hidden_states=hidden[:, :1], past_key_value=cache, k=cache.key_cache[0], v=cache.value_cache[0])
+    assert cache.key_cache[0].shape[2] == 32
+    assert len(layers[0].self_attn._forward_hooks) == 0             # hooks removed on exit
+
+
+def _fill_pool_from_case(runner, case, seqs):
+    """Copy a synthetic case's pages into the runner's pool following the block manager's tables."""
+    for b, s in enumerate(seqs):
+        for i, blk in enumerate(case.block_tables[b][:len(s.block_table)]):
+            runner.kv_cache[:, :, s.block_table[i]] = case.kv_cache[:, :, blk].to(runner.device)
+
+
+@pytest.mark.parametrize("backend", ["mlp", "batched", "kvpress", "callable"])
+def test_runner_compress_free_and_decode(dev, backend):
+    dtype, L, H, img, txt = torch.float16, 2, 4, 300, 213
+    S = img + txt
+    lens = [S, S, 400]
+    case = synth.make_paged_case(seed=31, num_layers=L, batch=3, num_kv_heads=H, seq_lens=lens, dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0)
+    torch.manual_seed(12)
+    mlp = KVCacheLinearDecoupleCompressor(llava_cfg(L, H), compression_factor=2).to(dev).to(dtype).eval()
+    sd = {k: v.detach().cpu().float() for k, v in mlp.state_dict().items()}
+    kw = {}
+    if backend == "mlp":
+        kw["compressor"] = mlp
+    elif backend == "batched":
+        bat = BatchedGEMMCompressor(L, H, 128, 2)
+        bat.load_from_original_compressor(mlp)
+        kw["compressor"], kw["batched_compressor"] = mlp, bat
+    elif backend == "kvpress":
+        kw["compressor"] = KVPressCompressor("streaming_llm", 1.0 - 1.0 / 3)
+    else:
+        kw["compressor"] = lambda hf, it_len: mlp(hf, it_len=it_len)      # no paged_forward: generic path
+    runner = PagedKVRunner(L, H, 128, num_blocks=16, dtype=dtype, device=dev, image_token_len=img, **kw)
+    bm = BlockManager(16, 256)
+    seqs = [Sequence(list(range(1000 * i, 1000 * i + n))) for i, n in enumerate(lens)]
+    for s in seqs:
+        bm.allocate(s)
+    _fill_pool_from_case(runner, case, seqs)
+    tables_before = [list(s.block_table) for s in seqs]
+    pool_before = runner.kv_cache.cpu()
+
+    # oracle: the reference's per-sequence loop on the CPU
+    ref_pool = pool_before.clone()
+    if backend == "kvpress":
+        def oracle_comp(hf, i, n):
+            return [opress.adapter_compress_layer("streaming_llm", k, v, 1.0 - 1.0 / 3) for k, v in hf]
+    else:
+        def oracle_comp(hf, i, n):
+            return occm.linear_decouple_forward(hf, [img, max(1, n - img)], sd, 2, 1)
+    ref_lens, ref_free, ref_ratio = opipe.compress_batch(ref_pool, tables_before, lens, oracle_comp)
+
+    sec, ratio = runner.compress_kv_cache_batch(seqs)
+    assert sec > 0 and abs(ratio - ref_ratio) < 1e-9
+    for i, s in enumerate(seqs):
+        assert runner._compressed_lens[s.seq_id] == ref_lens[i]
+        assert runner.get_compressed_block_count(s.seq_id) == -(-ref_lens[i] // 256)
+        assert runner._blocks_to_free.get(s.seq_id, []) == ref_free.get(i, [])
+    got_pool = runner.kv_cache.cpu()
+    for i, (tab, n) in enumerate(zip(tables_before, lens)):
+        C = ref_lens[i]
+        g = opaged.extract_kv(got_pool, tab, n)
+        r = opaged.extract_kv(ref_pool, tab, n)
+        for (gk, gv), (rk, rv) in zip(g, r):
+            if backend == "kvpress":
+                assert torch.equal(gk, rk) and torch.equal(gv, rv)     # gathered bytes and stale tail: bit-exact
+            else:
+                assert_mlp_close(gk[:, :, :C], rk[:, :, :C], dtype)
+                assert torch.equal(gk[:, :, C:], rk[:, :, C:]) and torch.equal(gv[:, :, C:], rv[:, :, C:])
+
+    # block release: tables truncated, tail ids appended to the free deque in table order
+    free_before = list(bm.free_block_ids)
+    freed = free_compressed_blocks(bm, runner, seqs)
+    expect_tail = [b for i in range(3) for b in ref_free.get(i, [])]
+    assert freed == len(expect_tail) and list(bm.free_block_ids) == free_before + expect_tail
+    for i, s in enumerate(seqs):
+        assert s.block_table == tables_before[i][:-(-ref_lens[i] // 256)]
+        assert s.kv_cache_len == ref_lens[i] and s.is_compressed
+    assert len(bm.free_block_ids) + len(bm.used_block_ids) == 16
+
+    # one decode step's metadata follows the compressed lengths
+    for s in seqs:
+        s.append_token(7)
+        bm.may_append(s)
+    ids, pos = runner.prepare_decode(seqs)
+    from fastcache_amd.utils.context import get_context
+    ctx = get_context()
+    assert pos.tolist() == [s.kv_cache_len for s in seqs] == ctx.context_lens.tolist()
+    exp_slots = [s.block_table[s.kv_cache_len // 256] * 256 + s.kv_cache_len % 256 for s in seqs]
+    assert ctx.slot_mapping.tolist() == exp_slots and ctx.block_tables.shape[0] == 3
+
+
+def test_background_compression_event_protocol(dev):
+    dtype, L, H, S = torch.bfloat16, 2, 2, 600
+    case = synth.make_paged_case(seed=4, num_layers=L, batch=2, num_kv_heads=H, seq_lens=[S, S], dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0)
+    runner = PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0,
+                           compressor=KVPressCompressor("knorm", 0.5))
+    bm = BlockManager(8, 256)
+    seqs = [Sequence(list(range(i * 1000, i * 1000 + S))) for i in range(2)]
+    for s in seqs:
+        bm.allocate(s)
+    _fill_pool_from_case(runner, case, seqs)
+    sync_runner = PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0,
+                                compressor=KVPressCompressor("knorm", 0.5))
+    sync_runner.kv_cache.copy_(runner.kv_cache)
+    sync_runner.compress_kv_cache_batch(seqs)
+    done = runner.start_background_compression(seqs)
+    assert done is not None
+    runner.wait_compression(done)
+    assert done.query()
+    assert torch.equal(runner.kv_cache, sync_runner.kv_cache)       # same result as the synchronous path
+    assert runner._compressed_lens == sync_runner._compressed_lens
+    assert PagedKVRunner(L, H, 128, 2, dtype, dev).start_background_compression(seqs) is None
+    runner.clear_compressed_lens([seqs[0].seq_id])
+    assert seqs[0].seq_id not in runner._compressed_lens and seqs[1].seq_id in runner._compressed_lens

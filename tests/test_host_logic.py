@@ -1,0 +1,191 @@
+"""Host-side logic without a GPU: block manager and sequence state against the oracle's restatement,
+module construction (parameter names and seeded initialisation), press arithmetic, error paths."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from fastcache_amd.engine import BlockManager, Sequence
+from fastcache_amd.engine.kv_runner import PagedKVRunner
+from fastcache_amd.engine.llm_hooks import free_compressed_blocks
+from fastcache_amd.kernels import BatchedGEMMCompressor, KVPressCompressor, MiniCPMKVCompressor, create_kvpress_compressor
+from fastcache_amd.presses import KnormPress, SnapKVPress, StreamingLLMPress, press_select
+from fastcache_amd.utils_ccm import KVCacheHybridCompressor, KVCacheLinearDecoupleCompressor
+from oracle import blocks as oblocks
+from oracle import ccm as occm
+
+
+def llava_cfg(L=2, H=4, D=128):
+    return SimpleNamespace(text_config=SimpleNamespace(num_hidden_layers=L, num_key_value_heads=H, hidden_size=H * D,
+                                                       head_dim=D, num_attention_heads=H))
+
+
+def minicpm_cfg(L=2, Hq=28, Hkv=4, D=128):
+    return SimpleNamespace(architectures=["MiniCPMV"], num_hidden_layers=L, num_key_value_heads=Hkv,
+                           num_attention_heads=Hq, hidden_size=Hq * D)
+
+
+class FakeRunner:
+    def __init__(self, lens):
+        self._compressed_lens = dict(lens)
+        self._blocks_to_free = {}
+        self.block_size = 256
+
+    def get_compressed_block_count(self, seq_id):
+        if seq_id not in self._compressed_lens:
+            return -1
+        return -(-self._compressed_lens[seq_id] // self.block_size)
+
+
+def test_block_manager_matches_oracle_through_compression_and_decode():
+    bm = BlockManager(num_blocks=12, block_size=256)
+    pool = oblocks.PoolState(num_blocks=12)
+    seqs, states = [], []
+    base = 0
+    for n in (1000, 300, 700):
+        s = Sequence(list(range(base, base + n)))       # unique tokens: every block is a cache miss
+        base += n
+        bm.allocate(s)
+        st = oblocks.SeqState(s.seq_id, n)
+        oblocks.allocate(pool, st)
+        seqs.append(s)
+        states.append(st)
+        assert s.block_table == st.block_table
+    comp = {seqs[0].seq_id: 500, seqs[2].seq_id: 140}    # seqs[1] stays uncompressed
+    runner = FakeRunner(comp)
+    freed = free_compressed_blocks(bm, runner, seqs)
+    ofreed = sum(len(oblocks.free_compressed_blocks(pool, st, comp.get(st.seq_id))) for st in states)
+    assert freed == ofreed == 4
+    for s, st in zip(seqs, states):
+        assert s.block_table == st.block_table and s.kv_cache_len == st.kv_cache_len
+        assert s.is_compressed == st.is_compressed
+    assert list(bm.free_block_ids) == list(pool.free)
+    assert bm.used_block_ids == pool.used
+    assert len(bm.free_block_ids) + len(bm.used_block_ids) == 12
+    # decode: kv length grows by one per token; a block is taken exactly when kv_len % 256 == 1
+    s, st = seqs[0], states[0]
+    for step in range(20):
+        s.append_token(1)
+        st.append_token()
+        assert bm.can_append(s) == oblocks.can_append(pool, st)
+        bm.may_append(s)
+        oblocks.may_append(pool, st)
+        assert s.block_table == st.block_table and s.kv_cache_len == st.kv_cache_len == 501 + step
+    assert len(s.block_table) == 3 and list(bm.free_block_ids) == list(pool.free)
+    # the last kept block lost its prefix-cache hash
+    assert bm.blocks[seqs[2].block_table[-1]].hash == -1
+
+
+def test_block_manager_prefix_cache_and_specific_free():
+    bm = BlockManager(8, 256)
+    a = Sequence(list(range(600)))
+    b = Sequence(list(range(600)))                      # same prefix: the two full blocks are shared
+    bm.allocate(a)
+    bm.allocate(b)
+    assert a.block_table[:2] == b.block_table[:2] and a.block_table[2] != b.block_table[2]
+    assert b.num_cached_tokens == 512
+    assert bm.blocks[a.block_table[0]].ref_count == 2
+    bm.free_specific_blocks([a.block_table[0], 7])      # 7 is not in use: ignored
+    assert bm.blocks[a.block_table[0]].ref_count == 1 and a.block_table[0] in bm.used_block_ids
+    bm.free_blocks_after_compression(b, 1)
+    assert len(b.block_table) == 1
+    bm.deallocate(a)
+    assert not a.block_table
+
+
+def test_sequence_state():
+    s = Sequence([1, 2, 3])
+    assert not s.is_compressed and s.kv_cache_len == 3 and s.kv_num_blocks == 1
+    s.append_token(4)
+    assert s.kv_cache_len == 4
+    s.kv_cache_len = 300
+    s.append_token(5)
+    assert s.is_compressed and s.kv_cache_len == 301 and s.kv_num_blocks == 2 and len(s) == 5
+
+
+def test_module_parameter_names_and_seeded_init():
+    torch.manual_seed(123)
+    m = KVCacheLinearDecoupleCompressor(llava_cfg(), compression_factor=2, min_seq_len=1)
+    sd = occm.reference_init_state_dict("linear_decouple", 2, 128, 2, seed=123)
+    msd = m.state_dict()
+    assert set(msd) == set(sd)
+    assert all(torch.equal(msd[k], sd[k]) for k in sd)
+    assert list(msd)[0] == "compress_tk.0.0.weight" and "attention.1.bias" in msd
+    assert (m.n_layer, m.nhead, m.head_dim, m.compression_factor, m.min_seq_len) == (2, 4, 128, 2, 1)
+
+    torch.manual_seed(5)
+    h = KVCacheHybridCompressor(minicpm_cfg(), compression_factor=5, min_seq_len=2)
+    hsd = occm.reference_init_state_dict("hybrid", 2, 128, 5, seed=5)
+    assert set(h.state_dict()) == set(hsd) and all(torch.equal(h.state_dict()[k], hsd[k]) for k in hsd)
+    assert h.compress_ik is None and h.compress_iv is None and h.head_dim == 128
+
+    torch.manual_seed(6)
+    mc = MiniCPMKVCompressor(minicpm_cfg())
+    csd = occm.reference_init_state_dict("minicpm", 2, 128, 5, seed=6)
+    assert all(torch.equal(mc.state_dict()[k], csd[k]) for k in csd)
+    assert (mc.compression_factor, mc.min_seq_len) == (5, 2)
+
+
+def test_batched_compressor_layout_and_loading():
+    torch.manual_seed(1)
+    orig = KVCacheLinearDecoupleCompressor(llava_cfg(), compression_factor=2)
+    b = BatchedGEMMCompressor(num_layers=2, num_heads=4, head_dim=128, compression_factor=2)
+    assert b.w1_tk.shape == (2, 256, 128) and b.b3_iv.shape == (2, 128)
+    assert float(b.b1_tk.abs().sum()) == 0                     # zero biases, Xavier weights
+    b.load_from_original_compressor(orig)
+    ow = occm.batched_weights_from_state_dict(orig.state_dict(), "compress_iv", 2)
+    for got, want in zip((b.w1_iv, b.b1_iv, b.w2_iv, b.b2_iv, b.w3_iv, b.b3_iv), ow):
+        assert torch.equal(got.detach(), want)
+    names = [n for n, _ in b.named_parameters()]
+    assert names[:6] == ["w1_tk", "b1_tk", "w2_tk", "b2_tk", "w3_tk", "b3_tk"]
+
+
+def test_kvpress_adapter_surface():
+    with pytest.raises(ValueError):
+        KVPressCompressor(method="nope")
+    c = create_kvpress_compressor("knorm", compression_factor=5)
+    assert c.compression_ratio == 1.0 - 1.0 / 5
+    assert c.get_compressed_length(1000) == 199               # double-arithmetic truncation kept
+    assert c.get_compressed_length(2) == 1
+    assert abs(c.compression_factor - 5.0) < 1e-9
+    assert "knorm" in repr(c) and len(KVPressCompressor.SUPPORTED_METHODS) == 8
+    cfg = SimpleNamespace(num_hidden_layers=3, num_attention_heads=8, num_key_value_heads=2, hidden_size=1024)
+    c2 = KVPressCompressor("snapkv", 0.5, config=cfg)
+    assert (c2.num_layers, c2.num_kv_heads, c2.head_dim) == (3, 2, 128)
+    assert c2.forward([]) == []
+
+
+def test_press_objects_surface():
+    p = press_select("SnapKV", 0.75)
+    assert isinstance(p, SnapKVPress) and p.window_size == 64 and p.kernel_size == 5 and p.totalTime == 0
+    assert p.n_kept(4096) == 1024
+    assert SnapKVPress(0.75, window_in_budget=False).n_kept(4096) == 1088
+    assert isinstance(press_select("anything else", 0.5), KnormPress)
+    assert isinstance(press_select("StreamingLLM", 0.5), StreamingLLMPress)
+    with pytest.raises(NotImplementedError):
+        press_select("TOVA", 0.5)
+    with pytest.raises(AssertionError):
+        KnormPress(compression_ratio=1.0)
+    # ratio 0 returns the inputs untouched without touching the device
+    k = torch.zeros(1, 1, 4, 128)
+    assert KnormPress(0.0).compress(None, None, k, k, None, {})[0] is k
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    from fastcache_amd._lib import FastcacheError
+    m = KVCacheLinearDecoupleCompressor(llava_cfg(L=1, H=1))
+    kv = [(torch.zeros(1, 1, 8, 128, dtype=torch.float16), torch.zeros(1, 1, 8, 128, dtype=torch.float16))]
+    with pytest.raises(FastcacheError):
+        m(kv, it_len=[4, 4])
+    with pytest.raises(FastcacheError):
+        KnormPress(0.5).compress(None, torch.zeros(1, 8, 1), kv[0][0], kv[0][1], None, {})
+
+
+def test_hybrid_image_branch_raises_like_reference():
+    h = KVCacheHybridCompressor(minicpm_cfg(L=1), compression_factor=2, min_seq_len=1)
+    kv = [(torch.zeros(1, 4, 16, 128), torch.zeros(1, 4, 16, 128))]
+    with pytest.raises(TypeError):
+        h(kv, it_len=[8, 8])
+    with pytest.raises(TypeError):
+        h._paged_segments(16, [8, 8])
+    assert h._paged_segments(16, [0, 16]) == [("compress_tk", "compress_tv", 0, 16)]

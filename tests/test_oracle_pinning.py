@@ -1,0 +1,314 @@
+"""Pins the CPU oracle against independent statements of the same mathematics: float64 loops,
+closed forms, brute force on tiny inputs, hand-worked cases.  A plausible mistake in the oracle
+(dropped term, wrong index, transposed operand, wrong rounding point) fails one of these.
+The reference holds no golden vectors or known-answer tests for this path."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as oattn
+from oracle import blocks as oblocks
+from oracle import ccm as occm
+from oracle import paged as opaged
+from oracle import presses as opress
+
+
+# ---- paged <-> dense ---------------------------------------------------------------------------------
+def test_extract_closed_form_and_roundtrip():
+    L, NB, bs, H, D = 2, 7, 8, 3, 4
+    pool = torch.arange(2 * L * NB * bs * H * D, dtype=torch.float32).view(2, L, NB, bs, H, D)
+    table, S = [5, 2, 6], 19
+    hf = opaged.extract_kv(pool, table, S)
+    assert len(hf) == L
+    for l, (k, v) in enumerate(hf):
+        assert k.shape == (1, H, S, D)
+        for s in range(S):                       # dense[s] = pool[table[s // bs], s % bs]
+            assert torch.equal(k[0, :, s], pool[0, l, table[s // bs], s % bs])
+            assert torch.equal(v[0, :, s], pool[1, l, table[s // bs], s % bs])
+    # write-back of a shorter sequence: leading slots replaced, everything else untouched
+    before = pool.clone()
+    C = 11
+    comp = [(-(k[:, :, :C]).contiguous(), (v[:, :, :C] * 2).contiguous()) for k, v in hf]
+    opaged.write_back(pool, comp, table)
+    for l in range(L):
+        for s in range(S):
+            got = pool[0, l, table[s // bs], s % bs]
+            want = -before[0, l, table[s // bs], s % bs] if s < C else before[0, l, table[s // bs], s % bs]
+            assert torch.equal(got, want)
+    untouched = [b for b in range(NB) if b not in table[:2]]
+    assert torch.equal(pool[:, :, untouched], before[:, :, untouched])
+
+
+def test_write_back_stops_at_negative_block_and_table_end():
+    pool = torch.zeros(2, 1, 4, 4, 1, 2)
+    k = torch.ones(1, 1, 10, 2)
+    opaged.write_back(pool, [(k, k)], [1, -1, 2])
+    assert pool[0, 0, 1].sum() == 8 and pool[0, 0, 2].sum() == 0
+    pool.zero_()
+    opaged.write_back(pool, [(k, k)], [3])          # table shorter than needed: only 4 tokens land
+    assert pool.sum() == 2 * 8
+
+
+# ---- scores --------------------------------------------------------------------------------------------
+def test_knorm_score_float64():
+    g = torch.Generator().manual_seed(0)
+    k = torch.randn(2, 3, 17, 128, generator=g)
+    ref = -np.sqrt((k.double().numpy() ** 2).sum(-1))
+    np.testing.assert_allclose(opress.knorm_score(k).numpy(), ref, rtol=1e-6)
+    assert (opress.knorm_score(k) <= 0).all()
+    kb = k.bfloat16()
+    ref_b = -np.sqrt((kb.double().numpy() ** 2).sum(-1))      # fp32 math on the stored values
+    np.testing.assert_allclose(opress.knorm_score(kb).numpy(), ref_b, rtol=1e-6)
+
+
+def test_knorm_mean_score_is_largest_norm_rule():
+    k = torch.zeros(1, 2, 4, 128)
+    k[0, 0, 1, 0], k[0, 1, 1, 0] = 3.0, 5.0          # token 1: norms 3 and 5 -> mean 4
+    k[0, 0, 2, 0] = 2.0                              # token 2: mean 1
+    m = opress.knorm_mean_score(k)
+    assert m.tolist() == [[0.0, 4.0, 1.0, 0.0]]
+
+
+def _snapkv_loops(q, k, W, ks, causal, red):
+    B, Hq, _, D = q.shape
+    _, Hkv, S, _ = k.shape
+    G = Hq // Hkv
+    out = np.zeros((B, Hkv, S))
+    for b in range(B):
+        for h in range(Hq):
+            v = [0.0] * (S - W)
+            for i in range(W):
+                logits = [float((q[b, h, i].double() * k[b, h // G, s].double()).sum()) / math.sqrt(D) for s in range(S)]
+                if causal:
+                    logits = [x if s - (S - W) <= i else -1e300 for s, x in enumerate(logits)]
+                mx = max(logits)
+                e = [math.exp(x - mx) for x in logits]
+                z = sum(e)
+                for s in range(S - W):
+                    v[s] += e[s] / z
+            if red == "mean":
+                v = [x / W for x in v]
+            pooled = [sum(v[s + j] for j in range(-(ks // 2), ks // 2 + 1) if 0 <= s + j < S - W) / ks
+                      for s in range(S - W)]
+            for s in range(S - W):
+                out[b, h // G, s] += pooled[s] / (G if red == "mean" else 1)
+    out[:, :, S - W:] = out[:, :, :S - W].max()
+    return out
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("red", ["mean", "sum"])
+def test_snapkv_score_float64_loops(causal, red):
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(2, 4, 4, 8, generator=g)
+    k = torch.randn(2, 2, 21, 8, generator=g)
+    got = opress.snapkv_score(q, k, 4, 3, causal, red).double().numpy()
+    np.testing.assert_allclose(got, _snapkv_loops(q, k, 4, 3, causal, red), rtol=2e-5, atol=1e-7)
+
+
+def test_snapkv_window_is_never_pruned_and_counts_in_budget():
+    g = torch.Generator().manual_seed(2)
+    q, k = torch.randn(1, 2, 8, 16, generator=g), torch.randn(1, 2, 40, 16, generator=g)
+    sc = opress.snapkv_score(q, k, 8, 5)
+    idx = opress.topk_lowest_index(sc, 12)
+    assert (idx[..., -8:] == torch.arange(32, 40)).all()       # window kept, inside the 12
+
+
+# ---- selection -----------------------------------------------------------------------------------------
+def test_topk_matches_python_sorted_with_ties():
+    rng = np.random.default_rng(0)
+    for _ in range(50):
+        n = int(rng.integers(2, 40))
+        k = int(rng.integers(1, n + 1))
+        vals = rng.integers(0, 5, size=n).astype(np.float32)      # many exact ties
+        order = sorted(range(n), key=lambda i: (-vals[i], i))[:k]
+        want = sorted(order)
+        got = opress.topk_lowest_index(torch.from_numpy(vals)[None], k)[0].tolist()
+        assert got == want
+
+
+def test_topk_special_values():
+    x = torch.tensor([[0.0, -0.0, float("nan"), float("inf"), -float("inf"), 1.0]])
+    assert opress.topk_lowest_index(x, 1).tolist() == [[2]]         # NaN first
+    assert opress.topk_lowest_index(x, 2).tolist() == [[2, 3]]
+    assert opress.topk_lowest_index(x, 4).tolist() == [[0, 2, 3, 5]]  # +0 and -0 tie -> index 0
+
+
+def test_gather_tokens_bruteforce():
+    x = torch.arange(2 * 3 * 5 * 4).view(2, 3, 5, 4)
+    idx = torch.tensor([[[4, 0], [1, 1], [2, 3]], [[0, 1], [3, 4], [2, 2]]])
+    out = opress.gather_tokens(x, idx)
+    for b in range(2):
+        for h in range(3):
+            for j in range(2):
+                assert torch.equal(out[b, h, j], x[b, h, idx[b, h, j]])
+    shared = opress.gather_tokens(x, torch.tensor([[1, 3], [0, 4]]))
+    assert torch.equal(shared[1, 2, 1], x[1, 2, 4])
+
+
+def test_n_kept_double_arithmetic():
+    # int(S * (1 - (1 - 1/cf))) loses a token for many (S, cf): the quirk is part of the contract
+    r = opress.ratio_from_factor(5)
+    assert opress.n_kept_adapter(1000, r) == 199
+    assert opress.n_kept_adapter(1024, opress.ratio_from_factor(2)) == 512
+    assert opress.n_kept_adapter(3, 0.99) == 1
+    assert opress.n_kept_press(4096, 0.75) == 1024
+
+
+def test_adapter_index_rules_by_hand():
+    k = torch.zeros(2, 1, 20, 128)
+    # streaming: 4 sinks + recent
+    idx = opress.adapter_indices("streaming_llm", k, 0.5)
+    assert idx[0].tolist() == [0, 1, 2, 3] + list(range(14, 20))
+    # n_kept <= n_sink: sinks only; 20 * (1 - 0.9) = 1.9999999999999996 truncates to ONE token
+    assert opress.adapter_indices("streaming_llm", k, 0.9)[0].tolist() == [0]
+    assert opress.adapter_indices("streaming_llm", k, 0.85)[0].tolist() == [0, 1, 2]
+    # uniform stride for every other method: arange(0, S, S // n)[:n]
+    assert opress.adapter_indices("snapkv", k, 0.7)[0].tolist() == [0, 3, 6, 9, 12, 15]
+    assert opress.adapter_indices("h2o", k, 0.7)[0].tolist() == [0, 3, 6, 9, 12, 15]
+    # nothing dropped
+    assert opress.adapter_indices("knorm", k, 0.0) is None
+    # random: sorted, unique, right count
+    r = opress.adapter_indices("random", k, 0.5, generator=torch.Generator().manual_seed(0))[0].tolist()
+    assert r == sorted(set(r)) and len(r) == 10
+
+
+# ---- CCM MLP ------------------------------------------------------------------------------------------
+def test_mlp3_float64_and_rounding_points():
+    sd = occm.reference_init_state_dict("hybrid", 2, 128, 2, seed=0)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(3, 256, generator=g)
+    # fp32: plain chain in float64
+    w = {i: (sd[f"compress_tk.1.{i}.weight"].double(), sd[f"compress_tk.1.{i}.bias"].double()) for i in (0, 3, 6)}
+    h = torch.relu(x.double() @ w[0][0].T + w[0][1])
+    h = torch.relu(h @ w[3][0].T + w[3][1])
+    ref = h @ w[6][0].T + w[6][1]
+    np.testing.assert_allclose(occm.mlp3(x, sd, "compress_tk", 1).double().numpy(), ref.numpy(), rtol=1e-4, atol=1e-5)
+    # fp16: operands and every layer output are rounded to fp16, accumulation is wider
+    xh = x.half()
+    def lin(inp, i):
+        wt, bs = sd[f"compress_tk.1.{i}.weight"].half().double(), sd[f"compress_tk.1.{i}.bias"].half().double()
+        return (inp.double() @ wt.T + bs).half()
+    ref_h = lin(torch.relu(lin(torch.relu(lin(xh, 0)), 3)), 6)
+    got_h = occm.mlp3(xh, sd, "compress_tk", 1)
+    assert got_h.dtype == torch.float16
+    # float64 vs float32 accumulation may flip a rounding: at most one fp16 ulp, rarely
+    diff = (got_h.float() - ref_h.float()).abs()
+    assert float(diff.max()) <= 2.0 ** -10 * float(ref_h.float().abs().max())
+    assert float((diff > 0).float().mean()) < 0.05
+
+
+def test_reference_init_matches_torch_construction_order():
+    """Same draws as constructing tk, tv, ik, iv, attention with nn.Linear after manual_seed."""
+    import torch.nn as nn
+    torch.manual_seed(11)
+    mods = {}
+    for g in ("compress_tk", "compress_tv", "compress_ik", "compress_iv"):
+        mods[g] = [nn.Sequential(nn.Linear(256, 128), nn.ReLU(), nn.Dropout(0.4), nn.Linear(128, 128), nn.ReLU(),
+                                 nn.Dropout(0.4), nn.Linear(128, 128)) for _ in range(2)]
+    sd = occm.reference_init_state_dict("linear_decouple", 2, 128, 2, seed=11)
+    for g, lst in mods.items():
+        for l, m in enumerate(lst):
+            for i in (0, 3, 6):
+                assert torch.equal(sd[f"{g}.{l}.{i}.weight"], m[i].weight)
+                assert torch.equal(sd[f"{g}.{l}.{i}.bias"], m[i].bias)
+    assert "attention.1.weight" in sd and sd["attention.0.weight"].shape == (1, 128)
+    assert not any(k.startswith("compress_ik") for k in occm.reference_init_state_dict("hybrid", 2, 128, 2, 0))
+
+
+def test_compress_segment_reshape_and_remainder_by_hand():
+    sd = occm.reference_init_state_dict("hybrid", 1, 128, 3, seed=1)
+    g = torch.Generator().manual_seed(4)
+    k = torch.randn(1, 2, 11, 128, generator=g)
+    ck, cv = occm.compress_segment(k, k, sd, "compress_tk", "compress_tv", 0, 3, 1)
+    assert ck.shape == (1, 2, 3 + 2, 128)
+    # row j of head h is the concatenation of tokens 3j, 3j+1, 3j+2
+    for h in range(2):
+        for j in range(3):
+            row = torch.cat([k[0, h, 3 * j], k[0, h, 3 * j + 1], k[0, h, 3 * j + 2]])
+            torch.testing.assert_close(ck[0, h, j], occm.mlp3(row[None], sd, "compress_tk", 0)[0])
+            torch.testing.assert_close(cv[0, h, j], occm.mlp3(row[None], sd, "compress_tv", 0)[0])
+    assert torch.equal(ck[:, :, 3:], k[:, :, 9:])                   # remainder passed through
+    # min_seq_len guard returns the inputs
+    a, b = occm.compress_segment(k[:, :, :2], k[:, :, :2], sd, "compress_tk", "compress_tv", 0, 3, 1)
+    assert a.shape[2] == 2 and torch.equal(a, k[:, :, :2])
+
+
+def test_forward_variants_lengths_and_errors():
+    L = 1
+    sd = occm.reference_init_state_dict("linear_decouple", L, 128, 2, seed=2)
+    kv = [(torch.randn(1, 1, 20, 128), torch.randn(1, 1, 20, 128))]
+    out = occm.linear_decouple_forward(kv, [7, 13], sd, 2, 1)
+    assert out[0][0].shape[2] == (3 + 1) + (6 + 1) == occm.compressed_length(20, [7, 13], 2, 1)
+    hsd = occm.reference_init_state_dict("hybrid", L, 128, 2, seed=2)
+    assert occm.hybrid_forward(kv, [0, 20], hsd, 2, 1)[0][0].shape[2] == 10
+    with pytest.raises(TypeError):
+        occm.hybrid_forward(kv, [7, 13], hsd, 2, 1)
+    # image segment too short to compress: passed through, no error
+    assert occm.hybrid_forward(kv, [1, 19], hsd, 2, 1)[0][0].shape[2] == 1 + 9 + 1
+    msd = occm.reference_init_state_dict("minicpm", L, 128, 5, seed=2)
+    assert occm.minicpm_forward(kv, [0, 20], msd, 5, 2)[0][0].shape[2] == 4
+    # batched re-arrangement is the same function (W_batched = W.T)
+    w = occm.batched_weights_from_state_dict(sd, "compress_tk", L)
+    x = torch.randn(L, 6, 256)
+    torch.testing.assert_close(occm.batched_mlp_forward(x, *w)[0], occm.mlp3(x[0], sd, "compress_tk", 0))
+
+
+# ---- block accounting ----------------------------------------------------------------------------------
+def test_block_release_invariants_by_hand():
+    pool = oblocks.PoolState(num_blocks=10, block_size=256)
+    a, b = oblocks.SeqState(0, 1000), oblocks.SeqState(1, 300)
+    oblocks.allocate(pool, a)
+    oblocks.allocate(pool, b)
+    assert a.block_table == [0, 1, 2, 3] and b.block_table == [4, 5]
+    assert list(pool.free) == [6, 7, 8, 9] and len(pool.free) + len(pool.used) == 10
+    freed = oblocks.free_compressed_blocks(pool, a, 500)         # ceil(500/256) = 2 blocks kept
+    assert freed == [2, 3] and a.block_table == [0, 1] and a.kv_cache_len == 500
+    assert list(pool.free) == [6, 7, 8, 9, 2, 3]                 # appended in table order (FIFO reuse)
+    assert oblocks.free_compressed_blocks(pool, b, None) == [] and not b.is_compressed
+    # decode growth: a new block exactly when kv_len % 256 == 1, taken from the head of the deque
+    a.kv_cache_len_override = 512
+    a.append_token()                                             # kv_len 513
+    assert oblocks.can_append(pool, a)
+    oblocks.may_append(pool, a)
+    assert a.block_table == [0, 1, 6]
+    a.append_token()
+    oblocks.may_append(pool, a)
+    assert a.block_table == [0, 1, 6]
+    assert len(pool.free) + len(pool.used) == 10
+
+
+# ---- decode attention -------------------------------------------------------------------------------------
+def test_decode_attention_float64_loops_and_special_cases():
+    g = torch.Generator().manual_seed(5)
+    NB, bs, Hkv, Hq, D = 5, 4, 2, 4, 8
+    kc = torch.randn(NB, bs, Hkv, D, generator=g)
+    vc = torch.randn(NB, bs, Hkv, D, generator=g)
+    q = torch.randn(3, Hq, D, generator=g)
+    lens = torch.tensor([6, 1, 0], dtype=torch.int32)
+    table = torch.tensor([[3, 1, -1], [4, -1, -1], [-1, -1, -1]], dtype=torch.int32)
+    out = oattn.decode_attention(q, kc, vc, lens, table, 0.3)
+    for b in range(3):
+        for h in range(Hq):
+            n = int(lens[b])
+            if n == 0:
+                assert torch.equal(out[b, h], torch.zeros(D))
+                continue
+            ks = [kc[table[b, s // bs], s % bs, h // 2].double() for s in range(n)]
+            vs = [vc[table[b, s // bs], s % bs, h // 2].double() for s in range(n)]
+            logit = [float((q[b, h].double() * kk).sum()) * 0.3 for kk in ks]
+            mx = max(logit)
+            w = [math.exp(x - mx) for x in logit]
+            ref = sum(wi * vi for wi, vi in zip(w, vs)) / sum(w)
+            np.testing.assert_allclose(out[b, h].double().numpy(), ref.numpy(), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(out[1, 0], vc[4, 0, 0])                # one cached token: output is its V row
+
+
+def test_decode_slot_rule():
+    assert oattn.decode_slot([7, 3], 300) == 3 * 256 + 44
+    assert oattn.decode_slot([7, 3], 512) == 3 * 256 + 0           # no block yet: falls back to the last one
+    k = torch.zeros(2, 4, 1, 2)
+    oattn.store_kv(k, k.clone(), torch.ones(1, 1, 2), torch.ones(1, 1, 2), torch.tensor([5]))
+    assert k.view(8, 1, 2)[5].sum() == 2 and k.sum() == 2
