@@ -1,0 +1,254 @@
+"""The five benchmark configurations at full size on the GPU.
+
+Each test runs the whole pass at the configured shape and checks it (a) against the CPU oracle on
+a sample the oracle finishes in seconds, and (b) through size-independent properties over ALL of
+it: ascending unique in-range indices, gathered rows equal to the source rows they name, untouched
+bytes past the compressed length, two independent code paths (paged in place vs dense out of place)
+agreeing bit for bit, graph replays equal to eager launches, block accounting invariants.
+"""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from fastcache_amd import _lib, ops, paged_press, synth
+from fastcache_amd.engine import BlockManager, Sequence
+from fastcache_amd.engine.decode_graph import DecodeGraph
+from fastcache_amd.engine.kv_runner import PagedKVRunner
+from fastcache_amd.engine.llm_hooks import free_compressed_blocks
+from fastcache_amd.utils_ccm import KVCacheHybridCompressor, KVCacheLinearDecoupleCompressor
+from oracle import attention as oattn
+from oracle import ccm as occm
+from oracle import paged as opaged
+from oracle import pipeline as opipe
+from oracle import presses as opress
+from test_gpu_ccm import assert_mlp_close
+
+pytestmark = pytest.mark.gpu
+
+
+def dense_from_pool(pool_plane, tables, S):
+    """[L, B, Hkv, S, D] gathered from pages with torch indexing (test-side check only)."""
+    L, NB, bs, H, Dh = pool_plane.shape
+    nblk = -(-S // bs)
+    t = tables[:, :nblk].long()
+    x = pool_plane[:, t]                                        # [L, B, nblk, bs, H, D]
+    return x.reshape(L, t.shape[0], nblk * bs, H, Dh)[:, :, :S].permute(0, 1, 3, 2, 4)
+
+
+def check_index_properties(idx, S, n):
+    assert idx.shape[-1] == n
+    assert int(idx.min()) >= 0 and int(idx.max()) < S
+    assert bool((idx[..., 1:] > idx[..., :-1]).all())           # ascending, hence unique
+
+
+def check_compaction(pool_after, pool_before, tables, idx, S, n):
+    """Kept rows equal the source rows the indices name; slots past n are untouched."""
+    for plane in range(2):
+        before = dense_from_pool(pool_before[plane], tables, S)
+        after = dense_from_pool(pool_after[plane], tables, S)
+        want = torch.gather(before, 3, idx.long().unsqueeze(-1).expand(-1, -1, -1, -1, before.shape[-1]))
+        assert torch.equal(after[:, :, :, :n], want)
+        assert torch.equal(after[:, :, :, n:], before[:, :, :, n:])
+
+
+def test_config1_knorm_full(dev):
+    case = synth.knorm_case(seed=0)                              # CPU draw: bit-identical inputs on both sides
+    S, ratio = 1024, 0.5
+    ref_pool = case.kv_cache.clone()
+    ref_lens, ref_free, _ = opipe.compress_batch(ref_pool, case.block_tables, case.seq_lens,
+                                                 opipe.knorm_press_compressor(ratio))
+    pool = case.kv_cache.to(dev)
+    before = pool.clone()
+    tables = case.table_tensor(dev)
+    res = paged_press.knorm_compress_paged(pool, tables, case.lens_tensor(dev), S, ratio)
+    torch.cuda.synchronize()
+    assert res.n_kept == 512 == ref_lens[0] and ref_free[0] == case.block_tables[0][2:]
+    check_index_properties(res.indices, S, 512)
+    check_compaction(pool, before, tables, res.indices, S, 512)
+    ref_scores = torch.stack([opress.knorm_score(k)[0] for k, _ in opaged.extract_kv(case.kv_cache, case.block_tables[0], S)])
+    torch.testing.assert_close(res.scores[:, 0].cpu(), ref_scores, rtol=1e-3, atol=0)
+    tie = opress.near_tie_rows(ref_scores, 512)
+    ref_idx = opress.topk_lowest_index(ref_scores, 512)
+    assert torch.equal(res.indices[:, 0].cpu().long()[~tie], ref_idx[~tie])
+    assert int(tie.sum()) <= 0.02 * tie.numel()
+    if not tie.any():
+        assert torch.equal(pool.cpu().view(torch.uint8), ref_pool.view(torch.uint8))
+
+
+def test_config2_snapkv_full(dev):
+    L, B, Hq, Hkv, S, W, ksz, ratio = 36, 8, 32, 8, 4096, 64, 7, 0.75
+    case = synth.snapkv_case(seed=0, device=dev, device_draw=True)
+    pool, tables, lens = case.kv_cache, case.table_tensor(dev), case.lens_tensor(dev)
+    before = pool.clone()
+    res = paged_press.snapkv_compress_paged(pool, tables, lens, S, case.queries, ratio, W, ksz, True, "sum")
+    torch.cuda.synchronize()
+    n = 1024
+    assert res.n_kept == n
+    check_index_properties(res.indices, S, n)
+    assert bool((res.indices[..., -W:] == torch.arange(S - W, S, device=dev, dtype=torch.int32)).all())
+    check_compaction(pool, before, tables, res.indices, S, n)
+    # softmax mass: unpooled scores would sum to <= W*G per row; pooling keeps the sum within it
+    body = res.scores[..., :S - W]
+    assert bool((body >= 0).all()) and float(body.sum(-1).max()) <= W * (Hq // Hkv) * 1.001
+    # oracle on a sample of layers and sequences
+    for layer, b in ((0, 0), (17, 3), (35, 7)):
+        k = dense_from_pool(before[0, layer:layer + 1], tables[b:b + 1], S)[0].cpu()
+        ref = opress.snapkv_score(case.queries[layer, b:b + 1].cpu(), k, W, ksz, True, "sum")
+        got = res.scores[layer, b:b + 1].cpu()
+        torch.testing.assert_close(got[..., :S - W], ref[..., :S - W], rtol=1e-3, atol=1e-3 * float(ref.mean()))
+        # the window fill uses the maximum over the whole layer (all sequences and heads)
+        assert torch.equal(got[..., S - W:], res.scores[layer, :, :, :S - W].max().cpu().expand_as(got[..., S - W:]))
+        ref_full = ref.clone()
+        ref_full[..., S - W:] = got[..., S - W:]
+        tie = opress.near_tie_rows(ref[..., :S - W], n - W)
+        ridx = opress.topk_lowest_index(ref_full, n)
+        assert torch.equal(res.indices[layer, b:b + 1].cpu().long()[~tie], ridx[~tie])
+
+
+def test_config3_ccm_full(dev):
+    L, B, H, img, txt, cf = 32, 45, 32, 576, 64, 2
+    S = img + txt
+    case = synth.ccm_case(seed=0, device=dev, device_draw=True)
+    cfg = SimpleNamespace(text_config=SimpleNamespace(num_hidden_layers=L, num_key_value_heads=H, hidden_size=H * 128))
+    torch.manual_seed(0)
+    mod = KVCacheLinearDecoupleCompressor(cfg).to(dev).half().eval()        # constructor defaults
+    assert (mod.compression_factor, mod.min_seq_len) == (2, 1)
+    pool, tables, lens = case.kv_cache, case.table_tensor(dev), case.lens_tensor(dev)
+    before = pool.clone()
+    C = mod.paged_forward(pool, tables, lens, S, [img, txt])
+    torch.cuda.synchronize()
+    assert C == 320
+    # independent code path: dense, out of place, per layer -> must agree bit for bit with the paged in-place run
+    for layer in (0, 13, 31):
+        kd = dense_from_pool(before[0, layer:layer + 1], tables, S)[0]
+        vd = dense_from_pool(before[1, layer:layer + 1], tables, S)[0]
+        single = KVCacheLinearDecoupleCompressor(SimpleNamespace(text_config=SimpleNamespace(
+            num_hidden_layers=1, num_key_value_heads=H, hidden_size=H * 128))).to(dev).half().eval()
+        single.load_state_dict({k.replace(f".{layer}.", ".0.", 1): v for k, v in mod.state_dict().items()
+                                if k.split(".")[1] == str(layer)})
+        ok, ov = single([(kd, vd)], it_len=[img, txt])[0]
+        assert torch.equal(dense_from_pool(pool[0, layer:layer + 1], tables, C)[0], ok)
+        assert torch.equal(dense_from_pool(pool[1, layer:layer + 1], tables, C)[0], ov)
+        # oracle on two sequences of this layer
+        sd = {k: v.detach().cpu().float() for k, v in single.state_dict().items()}
+        ref = occm.linear_decouple_forward([(kd[:2].cpu(), vd[:2].cpu())], [img, txt], sd, cf, 1)
+        assert_mlp_close(ok[:2].cpu(), ref[0][0], torch.float16)
+        assert_mlp_close(ov[:2].cpu(), ref[0][1], torch.float16)
+    # bytes past the compressed length are untouched (third block of every table, tail of the second)
+    after_tail = dense_from_pool(pool[0], tables, S)[:, :, :, C:]
+    assert torch.equal(after_tail, dense_from_pool(before[0], tables, S)[:, :, :, C:])
+    # block accounting: 3 -> 2 blocks per sequence, 45 blocks back in table order
+    runner = PagedKVRunner(1, 1, 128, 1, torch.float16, dev)
+    bm = BlockManager(3 * B, 256)
+    seqs = [Sequence(list(range(i * S, (i + 1) * S))) for i in range(B)]
+    for s in seqs:
+        bm.allocate(s)
+        runner._compressed_lens[s.seq_id] = C
+    tails = [s.block_table[2] for s in seqs]
+    assert free_compressed_blocks(bm, runner, seqs) == B
+    assert list(bm.free_block_ids) == tails and all(len(s.block_table) == 2 for s in seqs)
+
+
+def test_config4_decode_full(dev):
+    L, B, Hq, Hkv, T = 32, 90, 32, 32, 128
+    case = synth.decode_case(seed=0, device=dev, device_draw=True, steps=T)
+    assert min(case.seq_lens) >= 128 and max(case.seq_lens) <= 2048
+    tables = case.table_tensor(dev)
+    lens0 = case.lens_tensor(dev)
+    g = torch.Generator(device=dev).manual_seed(1)
+    mk = lambda h: torch.randn((T, L, B, h, 128), generator=g, device=dev).half()
+    q, kn, vn = mk(Hq), mk(Hkv), mk(Hkv)
+    pool0 = case.kv_cache.clone()
+    lens = lens0.clone()
+    dg = DecodeGraph(case.kv_cache, tables, lens, q, kn, vn, 128 ** -0.5)
+    dg.capture()
+    out1 = dg.replay().clone()
+    torch.cuda.synchronize()
+    assert lens.tolist() == [n + T for n in case.seq_lens]
+    pool1 = case.kv_cache.clone()
+    # second replay from the same start reproduces pool and outputs bit for bit
+    case.kv_cache.copy_(pool0)
+    lens.copy_(lens0)
+    out2 = dg.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out2) and torch.equal(case.kv_cache, pool1)
+    # appended rows landed where the tables say
+    after = dense_from_pool(pool1[0, 5:6], tables, max(case.seq_lens) + T)[0]           # [B, H, S, D]
+    for b in (0, 44, 89):
+        n = case.seq_lens[b]
+        assert torch.equal(after[b, :, n:n + T].permute(1, 0, 2), kn[:, 5, b])
+    # oracle: last step of a sample of layers over a sample of sequences
+    sample = [0, 31, 89]
+    tab_c = tables[sample].cpu()
+    len_c = torch.tensor([case.seq_lens[b] + T for b in sample], dtype=torch.int32)
+    for layer in (0, 31):
+        ref = oattn.decode_attention(q[T - 1, layer, sample].cpu(), pool1[0, layer].cpu(), pool1[1, layer].cpu(), len_c,
+                                     tab_c, 128 ** -0.5)
+        torch.testing.assert_close(out1[T - 1, layer, sample].cpu().float(), ref.float(), atol=2e-2, rtol=0)
+    # and the first step
+    len_c0 = torch.tensor([case.seq_lens[b] + 1 for b in sample], dtype=torch.int32)
+    ref0 = oattn.decode_attention(q[0, 3, sample].cpu(), pool1[0, 3].cpu(), pool1[1, 3].cpu(), len_c0, tab_c, 128 ** -0.5)
+    torch.testing.assert_close(out1[0, 3, sample].cpu().float(), ref0.float(), atol=2e-2, rtol=0)
+
+
+def test_config5_hybrid_end_to_end(dev):
+    L, B, Hq, Hkv, S, cf, T = 28, 16, 28, 4, 16384, 5, 64
+    cfg = SimpleNamespace(architectures=["MiniCPMV"], num_hidden_layers=L, num_key_value_heads=Hkv,
+                          num_attention_heads=Hq, hidden_size=Hq * 128)
+    torch.manual_seed(0)
+    mod = KVCacheHybridCompressor(cfg, compression_factor=cf, min_seq_len=1).to(dev).bfloat16().eval()
+    nblk = B * 64 + 4
+    runner = PagedKVRunner(L, Hkv, 128, nblk, torch.bfloat16, dev, compressor=mod, image_token_len=0)
+    bm = BlockManager(nblk, 256)
+    seqs = [Sequence(list(range(i * S, (i + 1) * S))) for i in range(B)]
+    for s in seqs:
+        bm.allocate(s)
+    g = torch.Generator(device=dev).manual_seed(3)
+    for layer in range(L):
+        runner.kv_cache[:, layer].copy_(torch.randn(runner.kv_cache[:, layer].shape, generator=g, device=dev))
+    tables_before = [list(s.block_table) for s in seqs]
+    before = runner.kv_cache.clone()
+    # compress to 20 %: 16384 -> 3276 rows + 4 remainder tokens
+    sec, ratio = runner.compress_kv_cache_batch(seqs)
+    C = 3280
+    assert all(runner._compressed_lens[s.seq_id] == C for s in seqs) and abs(ratio - S / C) < 1e-9
+    free_before = list(bm.free_block_ids)
+    assert free_compressed_blocks(bm, runner, seqs) == 51 * B == 816
+    assert list(bm.free_block_ids) == free_before + [b for t in tables_before for b in t[13:]]
+    assert all(s.block_table == t[:13] and s.kv_cache_len == C for s, t in zip(seqs, tables_before))
+    # oracle on one sequence of two layers
+    sd = {k: v.detach().cpu().float() for k, v in mod.state_dict().items()}
+    tt = torch.tensor(tables_before, dtype=torch.int32, device=dev)
+    for layer in (0, 27):
+        kd = dense_from_pool(before[0, layer:layer + 1], tt[:1], S)[0].cpu()
+        vd = dense_from_pool(before[1, layer:layer + 1], tt[:1], S)[0].cpu()
+        lsd = {f"{k.split('.')[0]}.0.{k.split('.', 2)[2]}": v for k, v in sd.items() if k.split(".")[1] == str(layer)}
+        ref = occm.hybrid_forward([(kd, vd)], [0, S], lsd, cf, 1)
+        got_k = dense_from_pool(runner.kv_cache[0, layer:layer + 1], tt[:1], C)[0].cpu()
+        got_v = dense_from_pool(runner.kv_cache[1, layer:layer + 1], tt[:1], C)[0].cpu()
+        assert_mlp_close(got_k, ref[0][0], torch.bfloat16)
+        assert_mlp_close(got_v, ref[0][1], torch.bfloat16)
+        assert torch.equal(got_k[:, :, 3276:], kd[:, :, 16380:])            # remainder tokens copied through
+    # 64 decode steps over the compressed caches: freed blocks are handed out again as sequences grow
+    for s in seqs:
+        for _ in range(T):
+            s.append_token(1)
+            bm.may_append(s)
+        assert len(s.block_table) == 14 and s.kv_cache_len == C + T
+    assert len(bm.free_block_ids) + len(bm.used_block_ids) == nblk
+    tables = runner.preare_block_tables(seqs)
+    lens = torch.full((B,), C, dtype=torch.int32, device=dev)
+    mk = lambda h: torch.randn((T, L, B, h, 128), generator=g, device=dev).bfloat16()
+    q, kn, vn = mk(Hq), mk(Hkv), mk(Hkv)
+    dg = DecodeGraph(runner.kv_cache, tables, lens, q, kn, vn, 128 ** -0.5)
+    dg.capture()
+    out = dg.replay()
+    torch.cuda.synchronize()
+    assert lens.tolist() == [C + T] * B
+    tab_c = tables[:2].cpu()
+    for layer in (0, 27):
+        ref = oattn.decode_attention(q[T - 1, layer, :2].cpu(), runner.kv_cache[0, layer].cpu(),
+                                     runner.kv_cache[1, layer].cpu(), torch.tensor([C + T] * 2, dtype=torch.int32),
+                                     tab_c, 128 ** -0.5)
+        torch.testing.assert_close(out[T - 1, layer, :2].cpu().float(), ref.float(), atol=2e-2, rtol=0)
