@@ -35,7 +35,8 @@ def sources() -> list[Path]:
 
 def _compile_one(src: Path, verbose: bool) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
-    cmd = [HIPCC, *DEVICE_FLAGS, "-c", str(src), "-o", str(obj)]
+    extra = os.environ.get("FC_EXTRA_HIPCC_FLAGS", "").split()      # e.g. -DCP_R=16 for tuning runs
+    cmd = [HIPCC, *DEVICE_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -4,22 +4,35 @@
 // elements (256 or 512 bytes) and is moved by 16 or 32 lanes with 16-byte accesses.  The column is
 // walked in ascending chunks: all source rows of a chunk are loaded into registers, the
 // workgroup waits for the loads and synchronises, and only then are the chunk's destination
-// rows stored.  With ascending unique indices (dst j <= src idx[j]) this makes the in-place case
+// rows stored (while the next chunk's loads are already in flight).  With ascending unique indices (dst j <= src idx[j]) this makes the in-place case
 // (dst aliases src) safe: a chunk's stores can only hit rows whose reads have already completed,
 // and later chunks read rows that no earlier chunk writes.  Different heads, layers and K/V planes
 // touch disjoint bytes, so columns need no ordering between each other.
 #include "fc_common.h"
 
 #define CP_THREADS 256
-#define CP_R 8  // 16-byte loads in flight per lane
+#ifndef CP_R
+#define CP_R 8      // 16-byte loads in flight per lane and chunk
+#endif
+#define CP_TBL 1024 // block-table entries of one sequence cached in LDS (per view)
 
-__device__ __forceinline__ void cp_wait_loads_then_barrier() {
+__device__ __forceinline__ void cp_wait_then_barrier() {
   // the loaded registers are not consumed before the barrier, so wait for them explicitly
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 }
 
+__device__ __forceinline__ long long cp_offset(const KvView& v, const int* tbl, bool tbl_lds, int b, int s) {
+  if (tbl_lds) {
+    const int blk = tbl[s >> v.block_shift];
+    return blk < 0 ? -1 : (long long)blk * v.stride_block + (long long)(s & (v.block_size - 1)) * v.stride_token;
+  }
+  return fc_token_offset(v, b, s);
+}
+
 // GATHER: src token = indices[j]; otherwise src token = src_start + j.
+// The column is walked in chunks of CH rows with two register buffers: the loads of chunk c+1 are
+// issued right after the barrier that releases the stores of chunk c, so loads and stores overlap.
 template <int EB, bool GATHER>
 __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView sv, KvView dk, KvView dv,
                                                              const int* __restrict__ indices,
@@ -29,6 +42,7 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   constexpr int LPR = FC_HEAD_DIM * EB / 16;
   constexpr int RPP = CP_THREADS / LPR;
   constexpr int CH = RPP * CP_R;
+  __shared__ int stbl[CP_TBL], dtbl[CP_TBL];
   const int h = blockIdx.x, b = blockIdx.y;
   const int L = sk.num_layers;
   const int l = blockIdx.z % L;
@@ -40,39 +54,74 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   int n = n_kept ? n_kept[b] : k;
   if (!GATHER) n = min(n, S - src_start);
   if (n <= 0) return;
+
+  // block-table rows of this sequence (source and destination views may differ)
+  const bool s_lds = src.block_tables && src.block_shift >= 0 && S > 0 && ((S - 1) >> src.block_shift) < CP_TBL;
+  const int dlast = dst_start + n - 1;
+  const bool d_lds = dst.block_tables && dst.block_shift >= 0 && (dlast >> dst.block_shift) < CP_TBL;
+  if (s_lds)
+    for (int i = tid; i <= ((S - 1) >> src.block_shift); i += CP_THREADS)
+      stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
+  if (d_lds)
+    for (int i = tid; i <= (dlast >> dst.block_shift); i += CP_THREADS)
+      dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
+  __syncthreads();
+
   const int* idx = GATHER ? indices + (((long long)l * sk.batch + b) * heads_in_index + (h % heads_in_index)) *
                                           (long long)index_stride
                           : nullptr;
   const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * EB + sub * 16;
   char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * EB + sub * 16;
 
-  for (int j0 = 0; j0 < n; j0 += CH) {
-    uint4 buf[CP_R];
-    bool ok[CP_R];
+  auto load_idx = [&](int (&si)[CP_R], int j0) {
 #pragma unroll
     for (int u = 0; u < CP_R; ++u) {
       const int j = j0 + u * RPP + rg;
+      si[u] = j < n ? (GATHER ? idx[j] : src_start + j) : -1;
+    }
+  };
+  auto load_rows = [&](uint4 (&buf)[CP_R], bool (&ok)[CP_R], const int (&si)[CP_R]) {
+#pragma unroll
+    for (int u = 0; u < CP_R; ++u) {
       ok[u] = false;
-      if (j < n) {
-        const int s = GATHER ? idx[j] : src_start + j;
-        if (s >= 0 && s < S) {
-          const long long off = fc_token_offset(src, b, s);
-          if (off >= 0) {
-            buf[u] = *reinterpret_cast<const uint4*>(sbase + off * EB);
-            ok[u] = true;
-          }
+      const int s = si[u];
+      if (s >= 0 && s < S) {
+        const long long off = cp_offset(src, stbl, s_lds, b, s);
+        if (off >= 0) {
+          buf[u] = *reinterpret_cast<const uint4*>(sbase + off * EB);
+          ok[u] = true;
         }
       }
     }
-    cp_wait_loads_then_barrier();
+  };
+  auto store_rows = [&](const uint4 (&buf)[CP_R], const bool (&ok)[CP_R], int j0) {
 #pragma unroll
     for (int u = 0; u < CP_R; ++u) {
       const int j = j0 + u * RPP + rg;
       if (ok[u]) {
-        const long long off = fc_token_offset(dst, b, dst_start + j);
+        const long long off = cp_offset(dst, dtbl, d_lds, b, dst_start + j);
         if (off >= 0) *reinterpret_cast<uint4*>(dbase + off * EB) = buf[u];
       }
     }
+  };
+
+  uint4 bufa[CP_R], bufb[CP_R];
+  bool oka[CP_R], okb[CP_R];
+  int sia[CP_R], sib[CP_R];
+  load_idx(sia, 0);
+  load_rows(bufa, oka, sia);
+  load_idx(sib, CH);
+  for (int j0 = 0; j0 < n; j0 += 2 * CH) {
+    // chunk j0 is in flight in buffer a; the indices of chunk j0 + CH are in sib
+    cp_wait_then_barrier();
+    if (j0 + CH < n) load_rows(bufb, okb, sib);
+    load_idx(sia, j0 + 2 * CH);
+    store_rows(bufa, oka, j0);
+    if (j0 + CH >= n) break;
+    cp_wait_then_barrier();
+    if (j0 + 2 * CH < n) load_rows(bufa, oka, sia);
+    load_idx(sib, j0 + 3 * CH);
+    store_rows(bufb, okb, j0 + CH);
   }
 }
 

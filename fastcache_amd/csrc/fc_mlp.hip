@@ -25,6 +25,7 @@
 #include "fc_common.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -35,6 +36,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 #define ML_THREADS (ML_WAVES * 64)
 #define ML_ROWB 272                 // LDS bytes per weight row: 128 elements + 16 bytes of padding
 #define ML_WBYTES (128 * ML_ROWB)   // one 128 x 128 weight block in LDS
+#define ML_TBL 256                  // block-table entries cached per wavefront and view
 
 template <int DTYPE>
 __device__ __forceinline__ f32x16 ml_mfma(const uint4& a, const uint4& b, f32x16 c) {
@@ -61,27 +63,28 @@ __device__ __forceinline__ float ml_to_float(unsigned short h) {
   return DTYPE == FC_BF16 ? fc_bf16_to_float(h) : fc_half_to_float(h);
 }
 
-// relu(round(acc + bias)) for 8 consecutive accumulator registers -> one MFMA operand.
-// Registers i0..i0+7 of a block hold features fb + (i/4)*8 + lhalf*4 + i%4.
+// relu + round for 8 consecutive accumulator registers (the bias is already in the accumulator)
+// -> one MFMA operand.  ReLU before rounding equals rounding before ReLU.
 template <int DTYPE>
-__device__ __forceinline__ uint4 ml_act_operand(const f32x16& acc, int i0, const float* __restrict__ bias, int fb,
-                                                int lhalf) {
-  float v[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int i = i0 + e;
-    v[e] = acc[i] + bias[fb + (i >> 2) * 8 + lhalf * 4 + (i & 3)];
-  }
+__device__ __forceinline__ uint4 ml_act_operand(const f32x16& acc, int i0) {
   unsigned p[4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    // ReLU after rounding equals rounding after ReLU; a negative pair member is zeroed in the packed word
-    unsigned w = ml_pack2<DTYPE>(v[2 * e], v[2 * e + 1]);
-    if (w & 0x8000u) w &= 0xffff0000u;
-    if (w & 0x80000000u) w &= 0x0000ffffu;
-    p[e] = w;
-  }
+  for (int e = 0; e < 4; ++e)
+    p[e] = ml_pack2<DTYPE>(fmaxf(acc[i0 + 2 * e], 0.f), fmaxf(acc[i0 + 2 * e + 1], 0.f));
   return make_uint4(p[0], p[1], p[2], p[3]);
+}
+
+// accumulator block initialised with the bias of its 16 features: register i holds feature
+// fb + (i/4)*8 + lhalf*4 + i%4 (transposed layers: features run along the registers)
+__device__ __forceinline__ void ml_bias_init(f32x16& acc, const float* __restrict__ bias, int fb, int lhalf) {
+#pragma unroll
+  for (int i4 = 0; i4 < 4; ++i4) {
+    const float4 bv = *reinterpret_cast<const float4*>(bias + fb + i4 * 8 + lhalf * 4);
+    acc[i4 * 4 + 0] = bv.x;
+    acc[i4 * 4 + 1] = bv.y;
+    acc[i4 * 4 + 2] = bv.z;
+    acc[i4 * 4 + 3] = bv.w;
+  }
 }
 
 template <int DTYPE>
@@ -95,6 +98,7 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
   char* w2buf = lds + 2 * ML_WBYTES;       // permuted
   char* w3buf = lds + 3 * ML_WBYTES;       // permuted
   float* bias = reinterpret_cast<float*>(lds + 4 * ML_WBYTES);  // [3][128] fp32
+  int* tbls = reinterpret_cast<int*>(lds + 4 * ML_WBYTES + 3 * 128 * sizeof(float));  // [waves][2][ML_TBL]
 
   const int l = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -106,6 +110,24 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
   const int H = src.num_kv_heads;
   const int b = col_ok ? col / H : 0, h = col_ok ? col - (col / H) * H : 0;
   const int K1 = cf * 128;
+
+  // this wavefront's block-table rows (source and destination), so that no row address waits on a table read
+  int* stbl = tbls + (wave * 2) * ML_TBL;
+  int* dtbl = stbl + ML_TBL;
+  const int s_last = seg_start + c_rows * cf - 1, d_last = dst_start + c_rows - 1;
+  const bool s_lds = src.block_tables && src.block_shift >= 0 && (s_last >> src.block_shift) < ML_TBL;
+  const bool d_lds = dst.block_tables && dst.block_shift >= 0 && (d_last >> dst.block_shift) < ML_TBL;
+  if (col_ok && s_lds)
+    for (int i = lane; i <= (s_last >> src.block_shift); i += 64) stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
+  if (col_ok && d_lds)
+    for (int i = lane; i <= (d_last >> dst.block_shift); i += 64) dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
+  auto tok_off = [&](const KvView& v, const int* tbl, bool in_lds, int s) -> long long {
+    if (in_lds) {
+      const int blk = tbl[s >> v.block_shift];
+      return blk < 0 ? -1 : (long long)blk * v.stride_block + (long long)(s & (v.block_size - 1)) * v.stride_token;
+    }
+    return fc_token_offset(v, b, s);
+  };
 
   // ---- resident weights: W2, W3 with the k permutation, biases as fp32 ------------------------------
   {
@@ -130,19 +152,19 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
   // W1 chunk kc covers columns [kc*128, kc*128+128) of W1[l]: 2048 pieces of 16 bytes
   constexpr int WCH = 2048 / ML_THREADS;
   const char* w1l = w1 + (long long)l * 128 * K1 * 2;
-  uint4 wpre[WCH];
+  u32x4 wpre[WCH];
   auto w1_load = [&](int kc) {
 #pragma unroll
     for (int u = 0; u < WCH; ++u) {
       const int ch = tid + u * ML_THREADS;  // row n = ch / 16, part = ch % 16
-      wpre[u] = *reinterpret_cast<const uint4*>(w1l + ((long long)(ch >> 4) * K1 + kc * 128) * 2 + (ch & 15) * 16);
+      wpre[u] = *reinterpret_cast<const u32x4*>(w1l + ((long long)(ch >> 4) * K1 + kc * 128) * 2 + (ch & 15) * 16);
     }
   };
   auto w1_store = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < WCH; ++u) {
       const int ch = tid + u * ML_THREADS;
-      *reinterpret_cast<uint4*>(w1buf + buf * ML_WBYTES + (ch >> 4) * ML_ROWB + (ch & 15) * 16) = wpre[u];
+      *reinterpret_cast<u32x4*>(w1buf + buf * ML_WBYTES + (ch >> 4) * ML_ROWB + (ch & 15) * 16) = wpre[u];
     }
   };
 
@@ -160,7 +182,7 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     for (int tb = 0; tb < 2; ++tb) {
       const int r = row0 + tb * 32 + lrow;
       long long off = -1;
-      if (col_ok && r < c_rows) off = fc_token_offset(src, b, seg_start + cf * r + kc);
+      if (col_ok && r < c_rows) off = tok_off(src, stbl, s_lds, seg_start + cf * r + kc);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks)
         xf[tb][ks] = off >= 0 ? *reinterpret_cast<const uint4*>(sbase + off * 2 + ks * 32) : make_uint4(0, 0, 0, 0);
@@ -168,79 +190,101 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
   };
 
   f32x16 acc[4][2];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-    for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
 
   // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+1's rows load into `xnext`;
   // after the last chunk of an iteration, layers 2 and 3 and the stores.
   auto stage = [&](uint4 (&xcur)[2][8], uint4 (&xnext)[2][8], int q) {
     const int it = q / cf, kc = q - it * cf;
-    const bool more = q + 1 < q_total;
-    if (more) x_load(xnext, q + 1);
+    // The prefetches are unconditional (straight-line code keeps the staging registers out of
+    // scratch memory): past the last chunk the X rows are out of range and load nothing, and the
+    // extra W1 chunk lands in the buffer nobody reads again.
+    x_load(xnext, q + 1);
     __syncthreads();  // chunk q is in w1buf[q & 1]; every wavefront is done with chunk q - 1
-    if (more) w1_load((kc + 1 < cf) ? kc + 1 : 0);
+    w1_load((kc + 1 < cf) ? kc + 1 : 0);
     {
       const char* wa = w1buf + (q & 1) * ML_WBYTES + lrow * ML_ROWB + lhalf * 16;
+      uint4 af[2][4];      // weight fragments of k-step ks+1 are read while k-step ks multiplies
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) af[0][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
+        if (ks + 1 < 8) {
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+            af[(ks + 1) & 1][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + (ks + 1) * 32);
+        }
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
-          const uint4 a = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + ks * 32);
-          acc[mb][0] = ml_mfma<DTYPE>(a, xcur[0][ks], acc[mb][0]);
-          acc[mb][1] = ml_mfma<DTYPE>(a, xcur[1][ks], acc[mb][1]);
+          acc[mb][0] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[0][ks], acc[mb][0]);
+          acc[mb][1] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[1][ks], acc[mb][1]);
         }
       }
     }
-    if (more) w1_store((q + 1) & 1);
+    w1_store((q + 1) & 1);
     if (kc != cf - 1) return;
 
     // ---- layer 2: H2^T = W2 * H1^T, B operand taken from layer 1's accumulators -------------------
     uint4 hf[2][8];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb) {
-        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0, bias, mb * 32, lhalf);
-        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8, bias, mb * 32, lhalf);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0);
+        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8);
       }
+      ml_bias_init(acc[mb][0], bias + 128, mb * 32, lhalf);
+      acc[mb][1] = acc[mb][0];
+    }
     {
       const char* wa = w2buf + lrow * ML_ROWB + lhalf * 16;
+      uint4 af[2][4];
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) af[0][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB);
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
+        if (g + 1 < 8) {
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+            af[(g + 1) & 1][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + (g + 1) * 32);
+        }
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
-          const uint4 a = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + g * 32);
-          acc[mb][0] = ml_mfma<DTYPE>(a, hf[0][g], acc[mb][0]);
-          acc[mb][1] = ml_mfma<DTYPE>(a, hf[1][g], acc[mb][1]);
+          acc[mb][0] = ml_mfma<DTYPE>(af[g & 1][mb], hf[0][g], acc[mb][0]);
+          acc[mb][1] = ml_mfma<DTYPE>(af[g & 1][mb], hf[1][g], acc[mb][1]);
         }
       }
     }
     // ---- layer 3: Y = H2 * W3^T, A operand taken from layer 2's accumulators ---------------------
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb) {
-        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0, bias + 128, mb * 32, lhalf);
-        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8, bias + 128, mb * 32, lhalf);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0);
+        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8);
       }
+      // layer 3 is not transposed: register = token row, lane = feature -> one bias value per lane
+      const float b3v = bias[256 + mb * 32 + lrow];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mb][0][i] = b3v;
+      acc[mb][1] = acc[mb][0];
+    }
     {
       // acc[nb][tb] now accumulates Y[tb block rows][nb block features]
       const char* wb = w3buf + lrow * ML_ROWB + lhalf * 16;
+      uint4 bfr[2][4];
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) bfr[0][nb] = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB);
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
+        if (g + 1 < 8) {
+#pragma unroll
+          for (int nb = 0; nb < 4; ++nb)
+            bfr[(g + 1) & 1][nb] = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB + (g + 1) * 32);
+        }
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
-          const uint4 bw = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB + g * 32);
-          acc[nb][0] = ml_mfma<DTYPE>(hf[0][g], bw, acc[nb][0]);
-          acc[nb][1] = ml_mfma<DTYPE>(hf[1][g], bw, acc[nb][1]);
+          acc[nb][0] = ml_mfma<DTYPE>(hf[0][g], bfr[g & 1][nb], acc[nb][0]);
+          acc[nb][1] = ml_mfma<DTYPE>(hf[1][g], bfr[g & 1][nb], acc[nb][1]);
         }
       }
     }
@@ -253,16 +297,20 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
       for (int i4 = 0; i4 < 4; ++i4) {
         // registers 4*i4 .. 4*i4+3 are 4 consecutive rows
         const int r0 = row0 + tb * 32 + i4 * 8 + lhalf * 4;
+        const int t0 = dst_start + r0;
+        // the 4 rows share a block unless they straddle a block boundary (or the view is dense)
+        const bool together = !dst.block_tables || (dst.block_shift >= 0 && (t0 & (dst.block_size - 1)) + 3 < dst.block_size);
+        const long long off0 = (col_ok && r0 < c_rows) ? tok_off(dst, dtbl, d_lds, t0) : -1;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = r0 + e;
           long long off = -1;
-          if (col_ok && r < c_rows) off = fc_token_offset(dst, b, dst_start + r);
+          if (col_ok && r < c_rows)
+            off = together ? (off0 >= 0 ? off0 + (long long)e * dst.stride_token : -1) : tok_off(dst, dtbl, d_lds, t0 + e);
           if (off >= 0) {
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-              const float y = acc[nb][tb][i4 * 4 + e] + bias[256 + nb * 32 + lrow];
-              const unsigned w = ml_pack2<DTYPE>(y, 0.f);
+              const unsigned w = ml_pack2<DTYPE>(acc[nb][tb][i4 * 4 + e], 0.f);
               *reinterpret_cast<unsigned short*>(dbase + off * 2 + (nb * 32 + lrow) * 2) = (unsigned short)(w & 0xffff);
             }
           }
@@ -270,16 +318,21 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
       }
     }
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mb][tb][i] = 0.f;
+    for (int mb = 0; mb < 4; ++mb) {
+      ml_bias_init(acc[mb][0], bias, mb * 32, lhalf);
+      acc[mb][1] = acc[mb][0];
+    }
   };
 
   uint4 xa[2][8], xb[2][8];
   w1_load(0);
   w1_store(0);
+  __syncthreads();   // block tables, biases and the first weights are in LDS
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    ml_bias_init(acc[mb][0], bias, mb * 32, lhalf);
+    acc[mb][1] = acc[mb][0];
+  }
   x_load(xa, 0);
   for (int q = 0; q < q_total; q += 2) {
     stage(xa, xb, q);
@@ -317,7 +370,7 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && 64 * wpc * 2 <= c) wpc *= 2;
     const int cols_per_wg = ML_WAVES / wpc;
     dim3 grid((ncols + cols_per_wg - 1) / cols_per_wg, src->num_layers);
-    const size_t lds = 4 * ML_WBYTES + 3 * 128 * sizeof(float);
+    const size_t lds = 4 * ML_WBYTES + 3 * 128 * sizeof(float) + ML_WAVES * 2 * ML_TBL * sizeof(int);
     KvView s = fc_make_view(src), d = fc_make_view(dst);
     if (src->dtype == FC_BF16) {
       static bool attr_bf16 = false;
