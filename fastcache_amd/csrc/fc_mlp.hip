@@ -87,7 +87,9 @@ __device__ __forceinline__ void ml_bias_init(f32x16& acc, const float* __restric
   }
 }
 
-template <int DTYPE>
+// SRC_T / DST_T: 0 = dense view (no table), 1 = paged view whose table row fits the LDS cache,
+// 2 = paged view read through global memory.
+template <int DTYPE, int SRC_T, int DST_T>
 __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView dst, const char* __restrict__ w1,
                                                             const char* __restrict__ b1, const char* __restrict__ w2,
                                                             const char* __restrict__ b2, const char* __restrict__ w3,
@@ -115,18 +117,25 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
   int* stbl = tbls + (wave * 2) * ML_TBL;
   int* dtbl = stbl + ML_TBL;
   const int s_last = seg_start + c_rows * cf - 1, d_last = dst_start + c_rows - 1;
-  const bool s_lds = src.block_tables && src.block_shift >= 0 && (s_last >> src.block_shift) < ML_TBL;
-  const bool d_lds = dst.block_tables && dst.block_shift >= 0 && (d_last >> dst.block_shift) < ML_TBL;
-  if (col_ok && s_lds)
+  if (col_ok && SRC_T == 1)
     for (int i = lane; i <= (s_last >> src.block_shift); i += 64) stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
-  if (col_ok && d_lds)
+  if (col_ok && DST_T == 1)
     for (int i = lane; i <= (d_last >> dst.block_shift); i += 64) dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
-  auto tok_off = [&](const KvView& v, const int* tbl, bool in_lds, int s) -> long long {
-    if (in_lds) {
-      const int blk = tbl[s >> v.block_shift];
-      return blk < 0 ? -1 : (long long)blk * v.stride_block + (long long)(s & (v.block_size - 1)) * v.stride_token;
+  auto src_off = [&](int s) -> long long {
+    if (SRC_T == 0) return (long long)b * src.stride_batch + (long long)s * src.stride_token;
+    if (SRC_T == 1) {
+      const int blk = stbl[s >> src.block_shift];
+      return blk < 0 ? -1 : (long long)blk * src.stride_block + (long long)(s & (src.block_size - 1)) * src.stride_token;
     }
-    return fc_token_offset(v, b, s);
+    return fc_token_offset(src, b, s);
+  };
+  auto dst_off = [&](int s) -> long long {
+    if (DST_T == 0) return (long long)b * dst.stride_batch + (long long)s * dst.stride_token;
+    if (DST_T == 1) {
+      const int blk = dtbl[s >> dst.block_shift];
+      return blk < 0 ? -1 : (long long)blk * dst.stride_block + (long long)(s & (dst.block_size - 1)) * dst.stride_token;
+    }
+    return fc_token_offset(dst, b, s);
   };
 
   // ---- resident weights: W2, W3 with the k permutation, biases as fp32 ------------------------------
@@ -182,7 +191,7 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     for (int tb = 0; tb < 2; ++tb) {
       const int r = row0 + tb * 32 + lrow;
       long long off = -1;
-      if (col_ok && r < c_rows) off = tok_off(src, stbl, s_lds, seg_start + cf * r + kc);
+      if (col_ok && r < c_rows) off = src_off(seg_start + cf * r + kc);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks)
         xf[tb][ks] = off >= 0 ? *reinterpret_cast<const uint4*>(sbase + off * 2 + ks * 32) : make_uint4(0, 0, 0, 0);
@@ -298,20 +307,33 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
         // registers 4*i4 .. 4*i4+3 are 4 consecutive rows
         const int r0 = row0 + tb * 32 + i4 * 8 + lhalf * 4;
         const int t0 = dst_start + r0;
-        // the 4 rows share a block unless they straddle a block boundary (or the view is dense)
-        const bool together = !dst.block_tables || (dst.block_shift >= 0 && (t0 & (dst.block_size - 1)) + 3 < dst.block_size);
-        const long long off0 = (col_ok && r0 < c_rows) ? tok_off(dst, dtbl, d_lds, t0) : -1;
+        // common case: all 4 rows exist and sit in one block (always true for a dense view)
+        const bool together = DST_T == 0 || (dst.block_shift >= 0 && (t0 & (dst.block_size - 1)) + 3 < dst.block_size);
+        if (col_ok && r0 + 3 < c_rows && together) {
+          const long long off0 = dst_off(t0);
+          if (off0 >= 0) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = r0 + e;
-          long long off = -1;
-          if (col_ok && r < c_rows)
-            off = together ? (off0 >= 0 ? off0 + (long long)e * dst.stride_token : -1) : tok_off(dst, dtbl, d_lds, t0 + e);
-          if (off >= 0) {
+            for (int e = 0; e < 4; ++e) {
+              char* rowp = dbase + (off0 + (long long)e * dst.stride_token) * 2 + lrow * 2;
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-              const unsigned w = ml_pack2<DTYPE>(acc[nb][tb][i4 * 4 + e], 0.f);
-              *reinterpret_cast<unsigned short*>(dbase + off * 2 + (nb * 32 + lrow) * 2) = (unsigned short)(w & 0xffff);
+              for (int nb = 0; nb < 4; ++nb) {
+                const unsigned w = ml_pack2<DTYPE>(acc[nb][tb][i4 * 4 + e], 0.f);
+                *reinterpret_cast<unsigned short*>(rowp + nb * 64) = (unsigned short)(w & 0xffff);
+              }
+            }
+          }
+        } else if (col_ok && r0 < c_rows) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (r0 + e < c_rows) {
+              const long long off = dst_off(t0 + e);
+              if (off >= 0) {
+#pragma unroll
+                for (int nb = 0; nb < 4; ++nb) {
+                  const unsigned w = ml_pack2<DTYPE>(acc[nb][tb][i4 * 4 + e], 0.f);
+                  *reinterpret_cast<unsigned short*>(dbase + off * 2 + (nb * 32 + lrow) * 2) = (unsigned short)(w & 0xffff);
+                }
+              }
             }
           }
         }
@@ -372,25 +394,36 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     dim3 grid((ncols + cols_per_wg - 1) / cols_per_wg, src->num_layers);
     const size_t lds = 4 * ML_WBYTES + 3 * 128 * sizeof(float) + ML_WAVES * 2 * ML_TBL * sizeof(int);
     KvView s = fc_make_view(src), d = fc_make_view(dst);
-    if (src->dtype == FC_BF16) {
-      static bool attr_bf16 = false;
-      if (!attr_bf16) {
-        hipFuncSetAttribute((const void*)mlp_kernel<FC_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_bf16 = true;
-      }
-      hipLaunchKernelGGL((mlp_kernel<FC_BF16>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,
-                         (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,
-                         (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);
-    } else {
-      static bool attr_f16 = false;
-      if (!attr_f16) {
-        hipFuncSetAttribute((const void*)mlp_kernel<FC_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_f16 = true;
-      }
-      hipLaunchKernelGGL((mlp_kernel<FC_F16>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,
-                         (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,
-                         (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);
-    }
+    auto table_mode = [&](const KvView& v, int last_token) {
+      if (!v.block_tables) return 0;
+      return (v.block_shift >= 0 && (last_token >> v.block_shift) < ML_TBL) ? 1 : 2;
+    };
+    const int sm = table_mode(s, seg_start + c * cf - 1), dm = table_mode(d, dst_start + c - 1);
+    // dense/dense, LDS-cached tables, or the general path through global tables
+    const int mode = (sm == 0 && dm == 0) ? 0 : (sm == 1 && dm == 1) ? 1 : (sm == 0 && dm == 1) ? 2 : (sm == 1 && dm == 0) ? 3 : 4;
+#define ML_LAUNCH(DT, ST, DTT)                                                                                     \
+  do {                                                                                                             \
+    static bool attr_done = false;                                                                                 \
+    if (!attr_done) {                                                                                              \
+      hipFuncSetAttribute((const void*)mlp_kernel<DT, ST, DTT>, hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                          (int)lds);                                                                               \
+      attr_done = true;                                                                                            \
+    }                                                                                                              \
+    hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,       \
+                       (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,             \
+                       (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);                               \
+  } while (0)
+#define ML_DISPATCH(DT)                          \
+  switch (mode) {                                \
+    case 0: ML_LAUNCH(DT, 0, 0); break;          \
+    case 1: ML_LAUNCH(DT, 1, 1); break;          \
+    case 2: ML_LAUNCH(DT, 0, 1); break;          \
+    case 3: ML_LAUNCH(DT, 1, 0); break;          \
+    default: ML_LAUNCH(DT, 2, 2); break;         \
+  }
+    if (src->dtype == FC_BF16) { ML_DISPATCH(FC_BF16) } else { ML_DISPATCH(FC_F16) }
+#undef ML_DISPATCH
+#undef ML_LAUNCH
     FC_CHECK_LAUNCH(who);
   }
   if (rem > 0) return fc_copy_tokens(src, dst, seg_start + c * cf, rem, dst_start + c, stream);
