@@ -89,7 +89,9 @@ __device__ __forceinline__ void ml_bias_init(f32x16& acc, const float* __restric
 
 // SRC_T / DST_T: 0 = dense view (no table), 1 = paged view whose table row fits the LDS cache,
 // 2 = paged view read through global memory.
-template <int DTYPE, int SRC_T, int DST_T>
+// W1R: all of W1 fits the two LDS chunk buffers (cf <= 2) and is loaded once; otherwise W1 streams
+// through them one chunk per stage, which costs a workgroup barrier per chunk.
+template <int DTYPE, int SRC_T, int DST_T, bool W1R>
 __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView dst, const char* __restrict__ w1,
                                                             const char* __restrict__ b1, const char* __restrict__ w2,
                                                             const char* __restrict__ b2, const char* __restrict__ w3,
@@ -199,19 +201,24 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
   };
 
   f32x16 acc[4][2];
+  constexpr int XD = W1R ? 2 : 1;   // prefetch distance in chunks
 
-  // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+1's rows load into `xnext`;
+  // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+XD's rows load into `xnext`.
+  // With W1 resident three register buffers rotate (two chunks always in flight); the streaming
+  // variant needs registers for the W1 copy and keeps two buffers (one chunk in flight);
   // after the last chunk of an iteration, layers 2 and 3 and the stores.
   auto stage = [&](uint4 (&xcur)[2][8], uint4 (&xnext)[2][8], int q) {
     const int it = q / cf, kc = q - it * cf;
     // The prefetches are unconditional (straight-line code keeps the staging registers out of
     // scratch memory): past the last chunk the X rows are out of range and load nothing, and the
     // extra W1 chunk lands in the buffer nobody reads again.
-    x_load(xnext, q + 1);
-    __syncthreads();  // chunk q is in w1buf[q & 1]; every wavefront is done with chunk q - 1
-    w1_load((kc + 1 < cf) ? kc + 1 : 0);
+    x_load(xnext, q + XD);
+    if (!W1R) {
+      __syncthreads();  // chunk q is in w1buf[q & 1]; every wavefront is done with chunk q - 1
+      w1_load((kc + 1 < cf) ? kc + 1 : 0);
+    }
     {
-      const char* wa = w1buf + (q & 1) * ML_WBYTES + lrow * ML_ROWB + lhalf * 16;
+      const char* wa = w1buf + (W1R ? kc : (q & 1)) * ML_WBYTES + lrow * ML_ROWB + lhalf * 16;
       uint4 af[2][4];      // weight fragments of k-step ks+1 are read while k-step ks multiplies
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) af[0][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB);
@@ -229,7 +236,7 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
         }
       }
     }
-    w1_store((q + 1) & 1);
+    if (!W1R) w1_store((q + 1) & 1);
     if (kc != cf - 1) return;
 
     // ---- layer 2: H2^T = W2 * H1^T, B operand taken from layer 1's accumulators -------------------
@@ -297,8 +304,9 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
         }
       }
     }
-    // every wavefront of the group has consumed this iteration's source rows: stores may alias them
-    __syncthreads();
+    // every wavefront of the column has consumed this iteration's source rows: stores may alias them
+    // (a wavefront that owns its column alone is ordered by its own data dependences)
+    if (wpc > 1) __syncthreads();
     const int row0 = it * rows_per_iter + sub * 64;
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
@@ -346,9 +354,13 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     }
   };
 
-  uint4 xa[2][8], xb[2][8];
+  uint4 xa[2][8], xb[2][8], xc[2][8];
   w1_load(0);
   w1_store(0);
+  if (W1R && cf > 1) {
+    w1_load(1);
+    w1_store(1);
+  }
   __syncthreads();   // block tables, biases and the first weights are in LDS
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
@@ -356,9 +368,18 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     acc[mb][1] = acc[mb][0];
   }
   x_load(xa, 0);
-  for (int q = 0; q < q_total; q += 2) {
-    stage(xa, xb, q);
-    if (q + 1 < q_total) stage(xb, xa, q + 1);
+  if constexpr (W1R) {
+    x_load(xb, 1);
+    for (int q = 0; q < q_total; q += 3) {
+      stage(xa, xc, q);
+      if (q + 1 < q_total) stage(xb, xa, q + 1);
+      if (q + 2 < q_total) stage(xc, xb, q + 2);
+    }
+  } else {
+    for (int q = 0; q < q_total; q += 2) {
+      stage(xa, xb, q);
+      if (q + 1 < q_total) stage(xb, xa, q + 1);
+    }
   }
 }
 
@@ -401,27 +422,31 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     const int sm = table_mode(s, seg_start + c * cf - 1), dm = table_mode(d, dst_start + c - 1);
     // dense/dense, LDS-cached tables, or the general path through global tables
     const int mode = (sm == 0 && dm == 0) ? 0 : (sm == 1 && dm == 1) ? 1 : (sm == 0 && dm == 1) ? 2 : (sm == 1 && dm == 0) ? 3 : 4;
-#define ML_LAUNCH(DT, ST, DTT)                                                                                     \
+#define ML_LAUNCH(DT, ST, DTT, WR)                                                                                     \
   do {                                                                                                             \
     static bool attr_done = false;                                                                                 \
     if (!attr_done) {                                                                                              \
-      hipFuncSetAttribute((const void*)mlp_kernel<DT, ST, DTT>, hipFuncAttributeMaxDynamicSharedMemorySize,       \
+      hipFuncSetAttribute((const void*)mlp_kernel<DT, ST, DTT, WR>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
                           (int)lds);                                                                               \
       attr_done = true;                                                                                            \
     }                                                                                                              \
-    hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,       \
+    hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT, WR>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,   \
                        (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,             \
                        (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);                               \
   } while (0)
-#define ML_DISPATCH(DT)                          \
+#define ML_DISPATCH(DT, WR)                      \
   switch (mode) {                                \
-    case 0: ML_LAUNCH(DT, 0, 0); break;          \
-    case 1: ML_LAUNCH(DT, 1, 1); break;          \
-    case 2: ML_LAUNCH(DT, 0, 1); break;          \
-    case 3: ML_LAUNCH(DT, 1, 0); break;          \
-    default: ML_LAUNCH(DT, 2, 2); break;         \
+    case 0: ML_LAUNCH(DT, 0, 0, WR); break;      \
+    case 1: ML_LAUNCH(DT, 1, 1, WR); break;      \
+    case 2: ML_LAUNCH(DT, 0, 1, WR); break;      \
+    case 3: ML_LAUNCH(DT, 1, 0, WR); break;      \
+    default: ML_LAUNCH(DT, 2, 2, WR); break;     \
   }
-    if (src->dtype == FC_BF16) { ML_DISPATCH(FC_BF16) } else { ML_DISPATCH(FC_F16) }
+    if (src->dtype == FC_BF16) {
+      if (cf <= 2) { ML_DISPATCH(FC_BF16, true) } else { ML_DISPATCH(FC_BF16, false) }
+    } else {
+      if (cf <= 2) { ML_DISPATCH(FC_F16, true) } else { ML_DISPATCH(FC_F16, false) }
+    }
 #undef ML_DISPATCH
 #undef ML_LAUNCH
     FC_CHECK_LAUNCH(who);
