@@ -2,8 +2,9 @@
 // over rows made of `cf` consecutive tokens of one head, fp16/bf16 storage, fp32 accumulation,
 // each Linear's output rounded to the storage dtype.  Reads and writes the caches in place.
 //
-// Shape of the work: one workgroup of 4 wavefronts (one per SIMD, full register file) per group of (sequence, head) columns of one
-// layer; a wavefront owns 64 rows of one column per iteration.  The three GEMMs are chained
+// Shape of the work: one workgroup of 8 wavefronts (two per SIMD, so that one multiplies while
+// the other converts, loads or stores) per group of (sequence, head) columns of one
+// layer; a wavefront owns 32 rows of one column per iteration.  The three GEMMs are chained
 // through registers without any transposition:
 //   layer 1 (transposed)  H1^T = W1 * X^T   A = W1 rows from LDS, B = X token rows straight
 //                                           from HBM (16-byte loads, each element read once);
@@ -32,7 +33,13 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-#define ML_WAVES 4
+#ifndef ML_WAVES
+#define ML_WAVES 8       // wavefronts per workgroup (two per SIMD)
+#endif
+#ifndef ML_TB
+#define ML_TB 1          // 32-row token blocks per wavefront
+#endif
+#define ML_ROWS (32 * ML_TB)
 #define ML_THREADS (ML_WAVES * 64)
 #define ML_ROWB 272                 // LDS bytes per weight row: 128 elements + 16 bytes of padding
 #define ML_WBYTES (128 * ML_ROWB)   // one 128 x 128 weight block in LDS
@@ -92,7 +99,7 @@ __device__ __forceinline__ void ml_bias_init(f32x16& acc, const float* __restric
 // W1R: all of W1 fits the two LDS chunk buffers (cf <= 2) and is loaded once; otherwise W1 streams
 // through them one chunk per stage, which costs a workgroup barrier per chunk.
 template <int DTYPE, int SRC_T, int DST_T, bool W1R>
-__global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView dst, const char* __restrict__ w1,
+__global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView src, KvView dst, const char* __restrict__ w1,
                                                             const char* __restrict__ b1, const char* __restrict__ w2,
                                                             const char* __restrict__ b2, const char* __restrict__ w3,
                                                             const char* __restrict__ b3, int cf, int seg_start,
@@ -179,18 +186,18 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     }
   };
 
-  const int rows_per_iter = 64 * wpc;
+  const int rows_per_iter = ML_ROWS * wpc;
   const int n_iter = (c_rows + rows_per_iter - 1) / rows_per_iter;
   const int q_total = n_iter * cf;      // W1 chunk q = (iteration q / cf, token kc = q % cf) sits in buffer q & 1
   const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lhalf * 16;
   char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2;
 
   // X rows of chunk q for this lane: 2 token blocks x 8 k-steps of 16 bytes
-  auto x_load = [&](uint4 (&xf)[2][8], int q) {
+  auto x_load = [&](uint4 (&xf)[ML_TB][8], int q) {
     const int it = q / cf, kc = q - it * cf;
-    const int row0 = it * rows_per_iter + sub * 64;
+    const int row0 = it * rows_per_iter + sub * ML_ROWS;
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
+    for (int tb = 0; tb < ML_TB; ++tb) {
       const int r = row0 + tb * 32 + lrow;
       long long off = -1;
       if (col_ok && r < c_rows) off = src_off(seg_start + cf * r + kc);
@@ -200,14 +207,18 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     }
   };
 
-  f32x16 acc[4][2];
+  f32x16 acc[4][ML_TB];
+#ifdef ML_XD1
+  constexpr int XD = 1;
+#else
   constexpr int XD = W1R ? 2 : 1;   // prefetch distance in chunks
+#endif
 
   // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+XD's rows load into `xnext`.
   // With W1 resident three register buffers rotate (two chunks always in flight); the streaming
   // variant needs registers for the W1 copy and keeps two buffers (one chunk in flight);
   // after the last chunk of an iteration, layers 2 and 3 and the stores.
-  auto stage = [&](uint4 (&xcur)[2][8], uint4 (&xnext)[2][8], int q) {
+  auto stage = [&](uint4 (&xcur)[ML_TB][8], uint4 (&xnext)[ML_TB][8], int q) {
     const int it = q / cf, kc = q - it * cf;
     // The prefetches are unconditional (straight-line code keeps the staging registers out of
     // scratch memory): past the last chunk the X rows are out of range and load nothing, and the
@@ -231,8 +242,8 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
         }
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
-          acc[mb][0] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[0][ks], acc[mb][0]);
-          acc[mb][1] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[1][ks], acc[mb][1]);
+#pragma unroll
+          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[tb][ks], acc[mb][tb]);
         }
       }
     }
@@ -240,16 +251,17 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
     if (kc != cf - 1) return;
 
     // ---- layer 2: H2^T = W2 * H1^T, B operand taken from layer 1's accumulators -------------------
-    uint4 hf[2][8];
+    uint4 hf[ML_TB][8];
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-      for (int tb = 0; tb < 2; ++tb) {
+      for (int tb = 0; tb < ML_TB; ++tb) {
         hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0);
         hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8);
       }
       ml_bias_init(acc[mb][0], bias + 128, mb * 32, lhalf);
-      acc[mb][1] = acc[mb][0];
+#pragma unroll
+      for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
     }
     {
       const char* wa = w2buf + lrow * ML_ROWB + lhalf * 16;
@@ -265,8 +277,8 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
         }
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
-          acc[mb][0] = ml_mfma<DTYPE>(af[g & 1][mb], hf[0][g], acc[mb][0]);
-          acc[mb][1] = ml_mfma<DTYPE>(af[g & 1][mb], hf[1][g], acc[mb][1]);
+#pragma unroll
+          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = ml_mfma<DTYPE>(af[g & 1][mb], hf[tb][g], acc[mb][tb]);
         }
       }
     }
@@ -274,7 +286,7 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-      for (int tb = 0; tb < 2; ++tb) {
+      for (int tb = 0; tb < ML_TB; ++tb) {
         hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0);
         hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8);
       }
@@ -282,7 +294,8 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
       const float b3v = bias[256 + mb * 32 + lrow];
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][0][i] = b3v;
-      acc[mb][1] = acc[mb][0];
+#pragma unroll
+      for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
     }
     {
       // acc[nb][tb] now accumulates Y[tb block rows][nb block features]
@@ -299,17 +312,17 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
         }
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
-          acc[nb][0] = ml_mfma<DTYPE>(hf[0][g], bfr[g & 1][nb], acc[nb][0]);
-          acc[nb][1] = ml_mfma<DTYPE>(hf[1][g], bfr[g & 1][nb], acc[nb][1]);
+#pragma unroll
+          for (int tb = 0; tb < ML_TB; ++tb) acc[nb][tb] = ml_mfma<DTYPE>(hf[tb][g], bfr[g & 1][nb], acc[nb][tb]);
         }
       }
     }
     // every wavefront of the column has consumed this iteration's source rows: stores may alias them
     // (a wavefront that owns its column alone is ordered by its own data dependences)
     if (wpc > 1) __syncthreads();
-    const int row0 = it * rows_per_iter + sub * 64;
+    const int row0 = it * rows_per_iter + sub * ML_ROWS;
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
+    for (int tb = 0; tb < ML_TB; ++tb) {
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         // registers 4*i4 .. 4*i4+3 are 4 consecutive rows
@@ -350,11 +363,12 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
       ml_bias_init(acc[mb][0], bias, mb * 32, lhalf);
-      acc[mb][1] = acc[mb][0];
+#pragma unroll
+      for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
     }
   };
 
-  uint4 xa[2][8], xb[2][8], xc[2][8];
+  uint4 xa[ML_TB][8], xb[ML_TB][8], xc[ML_TB][8];
   w1_load(0);
   w1_store(0);
   if (W1R && cf > 1) {
@@ -365,10 +379,11 @@ __global__ __launch_bounds__(ML_THREADS, 1) void mlp_kernel(KvView src, KvView d
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
     ml_bias_init(acc[mb][0], bias, mb * 32, lhalf);
-    acc[mb][1] = acc[mb][0];
+#pragma unroll
+    for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
   }
   x_load(xa, 0);
-  if constexpr (W1R) {
+  if constexpr (XD == 2) {
     x_load(xb, 1);
     for (int q = 0; q < q_total; q += 3) {
       stage(xa, xc, q);
@@ -410,7 +425,7 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
   if (c > 0) {
     const int ncols = src->batch * src->num_kv_heads;
     int wpc = 1;
-    while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && 64 * wpc * 2 <= c) wpc *= 2;
+    while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && ML_ROWS * wpc * 2 <= c) wpc *= 2;
     const int cols_per_wg = ML_WAVES / wpc;
     dim3 grid((ncols + cols_per_wg - 1) / cols_per_wg, src->num_layers);
     const size_t lds = 4 * ML_WBYTES + 3 * 128 * sizeof(float) + ML_WAVES * 2 * ML_TBL * sizeof(int);
