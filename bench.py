@@ -125,13 +125,14 @@ class SnapKVWorkload(Workload):
         kview = _lib.paged_view(kv[0], self.tables, self.lens, S)
         vview = _lib.paged_view(kv[1], self.tables, self.lens, S)
         scores = torch.empty((L, B, Hkv, S), dtype=torch.float32, device=self.device)
+        row_max = torch.empty((L, B, Hkv), dtype=torch.float32, device=self.device)
         st = current_stream()
         with self.br:
             check(fn("fc_snapkv_score")(C.byref(kview), self.queries.data_ptr(), self.Hq, self.W, self.ksz, 1,
-                                        D ** -0.5, 1.0, scores.data_ptr(), S, st), "fc_snapkv_score")
-        # the window fill needs the whole layer's scores, so it is its own launch
-        check(fn("fc_snapkv_fill_window")(scores.data_ptr(), S, L, B, Hkv, self.lens.data_ptr(), S, self.W, st),
-              "fc_snapkv_fill_window")
+                                        D ** -0.5, 1.0, scores.data_ptr(), S, row_max.data_ptr(), st), "fc_snapkv_score")
+        # the window fill needs every row maximum of the layer, so it is its own (small) launch
+        check(fn("fc_snapkv_fill_window")(scores.data_ptr(), S, L, B, Hkv, self.lens.data_ptr(), S, self.W,
+                                          row_max.data_ptr(), st), "fc_snapkv_fill_window")
         idx = ops.topk_select(scores, self.n_kept)
         ops.compact(kview, vview, kview, vview, idx)
 

@@ -61,8 +61,8 @@ SIGNATURES = {
     "fc_last_error": (C.c_char_p, []),
     "fc_knorm_score": (C.c_int, [_V, _VP, _I, _VP]),
     "fc_knorm_mean_score": (C.c_int, [_V, _VP, _I, _VP]),
-    "fc_snapkv_score": (C.c_int, [_V, _VP, _I, _I, _I, _I, _F, _F, _VP, _I, _VP]),
-    "fc_snapkv_fill_window": (C.c_int, [_VP, _I, _I, _I, _I, _VP, _I, _I, _VP]),
+    "fc_snapkv_score": (C.c_int, [_V, _VP, _I, _I, _I, _I, _F, _F, _VP, _I, _VP, _VP]),
+    "fc_snapkv_fill_window": (C.c_int, [_VP, _I, _I, _I, _I, _VP, _I, _I, _VP, _VP]),
     "fc_topk_select": (C.c_int, [_VP, _I, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _VP]),
     "fc_compact": (C.c_int, [_V, _V, _V, _V, _VP, _I, _I, _I, _VP, _VP]),
     "fc_ccm_mlp": (C.c_int, [_V, _V, C.POINTER(FcMlpWeights), _I, _I, _I, _I, _VP]),

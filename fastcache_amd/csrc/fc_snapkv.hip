@@ -44,7 +44,7 @@ __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2
 template <int DTYPE, int NW>
 __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
     KvView kv, const char* __restrict__ q, int Hq, int W, int ksz, int causal, float c, float out_mul,
-    float* __restrict__ scores, int score_stride) {
+    float* __restrict__ scores, int score_stride, float* __restrict__ row_max) {
   constexpr int THREADS = NW * 64;
   constexpr int CHUNKS = SK_KT * 16;                        // 16-byte chunks per key tile
   constexpr int CH = (CHUNKS + THREADS - 1) / THREADS;      // chunks per thread
@@ -65,6 +65,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
 
   if (S <= W) {  // nothing outside the window to score
     for (int s = tid; s < score_stride; s += THREADS) out_row[s] = s < S ? 0.f : -INFINITY;
+    if (row_max && tid == 0) row_max[((long long)l * kv.batch + b) * Hkv + h] = -INFINITY;
     return;
   }
   const int SW = S - W;                       // scored keys
@@ -155,54 +156,70 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
   };
 
   // ================= sweep 1: per-lane softmax statistics ======================================
-  for (int t = 0; t < T; ++t) {
-    const int cur = t & 1;
-    load_tile(t + 1 < T ? t + 1 : 0);   // the tile after the last one is tile 0 of sweep 2
-    const int tile_end = (t + 1) * SK_KT;
-    const bool masked_tile = tile_end > S || (causal && tile_end > SW + 1);
+  // Tile 0 sets every lane-row's offset with the general (online-softmax) update.  Later tiles only
+  // add exp2(logit * c + nm): any fixed offset is mathematically valid, it merely has to keep the
+  // sums inside the fp32 range.  A sum that overflows (logits rising by more than ~2^7 in log2
+  // units above the first tile's) is detected afterwards and the sweep is redone with the general
+  // update on every tile.
+  int pb = 0;   // LDS buffer parity of tile 0 of the current sweep
+  auto sweep1 = [&](bool general) {
+    for (int t = 0; t < T; ++t) {
+      const int cur = (pb + t) & 1;
+      load_tile(t + 1 < T ? t + 1 : 0);   // the tile after the last one is tile 0 of the next sweep
+      const int tile_end = (t + 1) * SK_KT;
+      const bool masked_tile = tile_end > S || (causal && tile_end > SW + 1);
+      const bool slow = general || t == 0;
 #pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-      f32x16 acc[2];
-      logits(cur, cb, acc);
-      // keys past the sequence end, and (causal) window keys later than the query, are masked
-      if (masked_tile) {
-        const int s = t * SK_KT + cb * 32 + lrow;
+      for (int cb = 0; cb < 2; ++cb) {
+        f32x16 acc[2];
+        logits(cur, cb, acc);
+        // keys past the sequence end, and (causal) window keys later than the query, are masked
+        if (masked_tile) {
+          const int s = t * SK_KT + cb * 32 + lrow;
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-          // query index of register i is qi[rb] + lhalf*4 + (i/4)*8 + i%4: compare against constants
-          const int d = causal ? s - SW - qi[rb] - lhalf * 4 : -1;
+          for (int rb = 0; rb < 2; ++rb) {
+            // query index of register i is qi[rb] + lhalf*4 + (i/4)*8 + i%4: compare against constants
+            const int d = causal ? s - SW - qi[rb] - lhalf * 4 : -1;
 #pragma unroll
-          for (int i = 0; i < 16; ++i)
-            if (s >= S || d > ((i >> 2) * 8 + (i & 3))) acc[rb][i] = SK_NEG;
+            for (int i = 0; i < 16; ++i)
+              if (s >= S || d > ((i >> 2) * 8 + (i & 3))) acc[rb][i] = SK_NEG;
+          }
+        }
+        if (slow) {
+          // differences are formed before scaling: (-1e30) - (-1e30) = 0 exactly for still-masked rows
+#pragma unroll
+          for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const float tt = -acc[rb][i] * c;
+              const float mn = fminf(nm[rb][i], tt);
+              ls[rb][i] = ls[rb][i] * sk_exp2(mn - nm[rb][i]) + sk_exp2(mn - tt);
+              nm[rb][i] = mn;
+            }
+        } else {
+#pragma unroll
+          for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ls[rb][i] += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
         }
       }
-      // largest exponent argument relative to the lane's current offsets: does any offset have to move?
-      float worst = -1.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        worst = fmaxf(worst, fmaxf(fmaf(acc[0][i], c, nm[0][i]), fmaf(acc[1][i], c, nm[1][i])));
-      // A lane-row whose keys were all masked so far still has the SK_NEG offset, for which only
-      // exact differences are safe; shapes with fewer scored keys than one tile therefore always
-      // take the general update (after tile 0 every lane-row has a real offset otherwise).
-      if (always_general || __any(worst > SK_LAZY)) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float tt = -acc[rb][i] * c;
-            const float mn = fminf(nm[rb][i], tt);
-            ls[rb][i] = ls[rb][i] * sk_exp2(mn - nm[rb][i]) + sk_exp2(mn - tt);
-            nm[rb][i] = mn;
-          }
-      } else {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) ls[rb][i] += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
-      }
+      store_tile(cur ^ 1);
+      __syncthreads();
     }
-    store_tile(cur ^ 1);
-    __syncthreads();
+    pb += T;
+  };
+  for (int attempt = 0; attempt < 2; ++attempt) {   // one inlined copy of the sweep
+    sweep1(always_general || attempt == 1);
+    bool bad = false;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) bad |= !(ls[rb][i] <= 3.0e38f);   // inf or NaN
+    if (attempt == 1 || !__syncthreads_or(bad)) break;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { nm[rb][i] = -SK_NEG; ls[rb][i] = 0.f; }
   }
 
   // merge the per-lane states of each row across the 32 lanes of a half-wave and fold the
@@ -226,7 +243,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
 
   // ================= sweep 2: probabilities, per-key sums, moving average ======================
   for (int t = 0; t < T; ++t) {
-    const int cur = (T + t) & 1;
+    const int cur = (pb + t) & 1;
     if (t >= 1 && tid < SK_KT) {
       // fold the wavefronts' partial sums of tile t-1 (fixed order) into the ring
       float v = 0.f;
@@ -264,7 +281,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
     if (more) store_tile(cur ^ 1);
     __syncthreads();
   }
-  const int last_buf = (2 * T - 1) & 1;
+  const int last_buf = (pb + T - 1) & 1;
 
   // ---- drain: last tile's sums, then the moving average of the last three tiles ------------
   if (tid < SK_KT) {
@@ -287,9 +304,41 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
     }
     for (int s = S + tid; s < score_stride; s += THREADS) out_row[s] = -INFINITY;
   }
+  if (row_max) {   // maximum of this row's scores, for the window fill: re-read what this workgroup wrote
+    __syncthreads();
+    float rmax = -INFINITY;
+    for (int s = tid; s < SW; s += THREADS) rmax = fmaxf(rmax, out_row[s]);
+    rmax = fc_wave_max(rmax);
+    if (lane == 0) vpart[0][wave][0] = rmax;
+    __syncthreads();
+    if (tid == 0) {
+      float m = vpart[0][0][0];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) m = fmaxf(m, vpart[0][w][0]);
+      row_max[((long long)l * kv.batch + b) * Hkv + h] = m;
+    }
+  }
 }
 
-// One workgroup per layer: maximum over the scored part of every row, then the window fill.
+// Window fill.  With the per-row maxima from the scoring kernel: one small workgroup per row takes
+// the maximum over its layer's rows and writes its own window.  Without them: one workgroup per
+// layer scans the scored part of every row first.
+__global__ __launch_bounds__(64) void snapkv_fill_rows_kernel(float* __restrict__ scores, int score_stride, int batch,
+                                                              int Hkv, const int* __restrict__ seq_lens,
+                                                              int max_seq_len, int W,
+                                                              const float* __restrict__ row_max) {
+  const int r = blockIdx.x, l = blockIdx.y, lane = threadIdx.x;
+  const int rows = batch * Hkv;
+  float mx = -INFINITY;
+  for (int i = lane; i < rows; i += 64) mx = fmaxf(mx, row_max[(long long)l * rows + i]);
+  mx = fc_wave_max(mx);
+  int S = seq_lens ? seq_lens[r / Hkv] : max_seq_len;
+  S = min(S, max_seq_len);
+  float* row = scores + ((long long)l * rows + r) * score_stride;
+  for (int j = lane; j < W; j += 64)
+    if (S - W + j >= 0) row[S - W + j] = mx;
+}
+
 __global__ __launch_bounds__(1024) void snapkv_fill_kernel(float* __restrict__ scores, int score_stride, int batch,
                                                            int Hkv, const int* __restrict__ seq_lens, int max_seq_len,
                                                            int W) {
@@ -321,7 +370,7 @@ __global__ __launch_bounds__(1024) void snapkv_fill_kernel(float* __restrict__ s
 
 extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_heads, int32_t window,
                                int32_t kernel_size, int32_t causal_window, float scale, float out_scale,
-                               float* scores, int32_t score_stride, void* stream) {
+                               float* scores, int32_t score_stride, float* row_max, void* stream) {
   const char* who = "fc_snapkv_score";
   int rc = fc_check_view(keys, who);
   if (rc) return rc;
@@ -350,7 +399,7 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
   const char* q = (const char*)queries;
 #define SK_LAUNCH(DT, NWV)                                                                                   \
   hipLaunchKernelGGL((snapkv_kernel<DT, NWV>), grid, dim3(NWV * 64), 0, st, kv, q, num_q_heads, window,      \
-                     kernel_size, causal_window, c, out_mul, scores, score_stride)
+                     kernel_size, causal_window, c, out_mul, scores, score_stride, row_max)
 #define SK_DISPATCH(DT)                 \
   if (waves <= 1) SK_LAUNCH(DT, 1);     \
   else if (waves <= 2) SK_LAUNCH(DT, 2);\
@@ -365,14 +414,21 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
 
 extern "C" int fc_snapkv_fill_window(float* scores, int32_t score_stride, int32_t num_layers, int32_t batch,
                                      int32_t num_kv_heads, const int32_t* seq_lens, int32_t max_seq_len,
-                                     int32_t window, void* stream) {
+                                     int32_t window, const float* row_max, void* stream) {
   const char* who = "fc_snapkv_fill_window";
   FC_REQUIRE(scores, FC_EINVAL, "%s: null scores", who);
   FC_REQUIRE(num_layers > 0 && batch > 0 && num_kv_heads > 0 && window > 0 && max_seq_len >= 0 &&
                  score_stride >= max_seq_len,
              FC_EINVAL, "%s: bad sizes", who);
-  hipLaunchKernelGGL(snapkv_fill_kernel, dim3(num_layers), dim3(1024), 0, (hipStream_t)stream, scores, score_stride,
-                     batch, num_kv_heads, seq_lens, max_seq_len, window);
+  if (row_max) {
+    FC_REQUIRE(num_layers <= 65535, FC_EUNSUPPORTED, "%s: too many layers", who);
+    hipLaunchKernelGGL(snapkv_fill_rows_kernel, dim3(batch * num_kv_heads, num_layers), dim3(64), 0,
+                       (hipStream_t)stream, scores, score_stride, batch, num_kv_heads, seq_lens, max_seq_len, window,
+                       row_max);
+  } else {
+    hipLaunchKernelGGL(snapkv_fill_kernel, dim3(num_layers), dim3(1024), 0, (hipStream_t)stream, scores, score_stride,
+                       batch, num_kv_heads, seq_lens, max_seq_len, window);
+  }
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }

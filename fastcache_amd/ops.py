@@ -74,11 +74,12 @@ def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size
     dev = queries.device
     out = torch.empty((L, B, keys.num_kv_heads, stride), dtype=torch.float32, device=dev)
     st = current_stream()
+    row_max = torch.empty((L, B, keys.num_kv_heads), dtype=torch.float32, device=dev)
     check(fn("fc_snapkv_score")(C.byref(keys), queries.data_ptr(), Hq, window, kernel_size,
-                                int(causal_window), scale, out_scale, out.data_ptr(), stride, st),
+                                int(causal_window), scale, out_scale, out.data_ptr(), stride, row_max.data_ptr(), st),
           "fc_snapkv_score")
     check(fn("fc_snapkv_fill_window")(out.data_ptr(), stride, L, B, keys.num_kv_heads, ptr(seq_lens),
-                                      keys.max_seq_len, window, st), "fc_snapkv_fill_window")
+                                      keys.max_seq_len, window, row_max.data_ptr(), st), "fc_snapkv_fill_window")
     return out
 
 

@@ -101,6 +101,7 @@ int fc_knorm_mean_score(const fc_kv_view* keys, float* out, int32_t score_stride
  *   v[hq][s] = sum_i A[hq][i][s] for s < S-W;  pooled = avg_pool1d(v, kernel, stride 1,
  *   pad kernel/2, zeros counted);  scores[l][b][hkv][s] = out_scale * sum_{hq in group} pooled.
  *   Entries S-W <= s < S are left for fc_snapkv_fill_window; entries s >= S are -inf.
+ *   row_max (optional, float[num_layers][batch][num_kv_heads]) receives each row's largest score.
  * Replaces kvpress.SnapKVPress.score / compute_window_attention (third-party; reference
  * call sites utils_ccm/utils_compress.py:310-312, 335-337; bench_kvpress_native.py:137-147;
  * nanovllm/kernels/kvpress_compressor.py:139-143).
@@ -109,16 +110,17 @@ int fc_knorm_mean_score(const fc_kv_view* keys, float* out, int32_t score_stride
 int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_heads,
                     int32_t window, int32_t kernel_size, int32_t causal_window,
                     float scale, float out_scale,
-                    float* scores, int32_t score_stride, void* stream);
+                    float* scores, int32_t score_stride, float* row_max, void* stream);
 
 /*
  * Sets the window entries scores[l][b][h][S_b-W .. S_b) to the maximum over
  * scores[l][:, :, :S_b-W] of the same layer, the way kvpress pads the observation window
  * back in (F.pad(value=scores.max())) so that it always survives selection.
+ * row_max (optional): the per-row maxima written by fc_snapkv_score, which save the scan.
  */
 int fc_snapkv_fill_window(float* scores, int32_t score_stride, int32_t num_layers, int32_t batch,
                           int32_t num_kv_heads, const int32_t* seq_lens, int32_t max_seq_len,
-                          int32_t window, void* stream);
+                          int32_t window, const float* row_max, void* stream);
 
 /*
  * Row-wise top-k with a defined order.  Row r of `rows` score rows has

@@ -119,3 +119,20 @@ def test_snapkv_scores_and_selection(dev, cfg, causal, reduction):
         assert torch.equal(idx[~tie], ref_idx[~tie])
         # the observation window always survives
         assert (idx[..., -W:] == torch.arange(S - W, S)).all()
+
+
+@pytest.mark.parametrize("boost,where", [(18.0, 130), (30.0, 200), (60.0, 70), (30.0, 10)])
+def test_snapkv_extreme_logits(dev, boost, where):
+    """Logits that jump far above the running offset: the lazy-offset sweep must rescale (moderate
+    jump) or fall back to the general update (jump that overflows fp32) and still match the oracle."""
+    L, B, Hq, Hkv, S, W, ksz = 1, 2, 8, 2, 400, 64, 5
+    case = synth.snapkv_case(seed=19, num_layers=L, batch=B, num_q_heads=Hq, num_kv_heads=Hkv, seq_len=S,
+                             window=W, keep_dense=True)
+    case.dense_k[:, :, :, where:where + 10] *= boost
+    q = case.queries
+    ref = torch.stack([opress.snapkv_score(q[l], case.dense_k[l], W, ksz, True, "sum") for l in range(L)])
+    assert torch.isfinite(ref).all()
+    dk = case.dense_k.to(dev)
+    got = ops.snapkv_score(_lib.dense_view(dk), q.to(dev), W, ksz, causal_window=True, reduction="sum").cpu()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-4 * float(ref.max()))
