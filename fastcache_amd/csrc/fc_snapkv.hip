@@ -23,6 +23,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+#ifndef SK_RB
+#define SK_RB 1          // 32-row query blocks per wavefront
+#endif
 #define SK_KT 64          // keys per tile
 #define SK_ROWB 272       // LDS bytes per key row (256 + 16 pad)
 #define SK_NEG (-1.0e30f) // "minus infinity" that stays finite under subtraction
@@ -42,7 +45,7 @@ __device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16
 __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int DTYPE, int NW>
-__global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
+__global__ __launch_bounds__(NW * 64, (SK_RB == 2 ? (NW <= 4 ? 2 : 1) : (NW <= 4 ? 4 : NW <= 8 ? 4 : 2))) void snapkv_kernel(
     KvView kv, const char* __restrict__ q, int Hq, int W, int ksz, int causal, float c, float out_mul,
     float* __restrict__ scores, int score_stride, float* __restrict__ row_max) {
   constexpr int THREADS = NW * 64;
@@ -72,12 +75,12 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
   const int T = (S + SK_KT - 1) / SK_KT;      // key tiles
 
   // ---- query fragments ------------------------------------------------------------------
-  uint4 qf[2][8];
-  int qi[2];          // query index (within the window) of this lane's A row
-  bool rb_valid[2];
+  uint4 qf[SK_RB][8];
+  int qi[SK_RB];      // query index (within the window) of this lane's A row
+  bool rb_valid[SK_RB];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
-    const int blk = wave * 2 + rb;
+  for (int rb = 0; rb < SK_RB; ++rb) {
+    const int blk = wave * SK_RB + rb;
     rb_valid[rb] = blk < RBT;
     const int g = rb_valid[rb] ? blk / WB : 0;
     const int wb = rb_valid[rb] ? blk - g * WB : 0;
@@ -128,9 +131,9 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
 
   // per-lane softmax state for the lane's 2 x 16 query rows: nm = -(offset * c), ls = sum of
   // exp2(logit * c + nm) over the keys this lane has seen
-  float nm[2][16], ls[2][16];
+  float nm[SK_RB][16], ls[SK_RB][16];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb)
+  for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) { nm[rb][i] = -SK_NEG; ls[rb][i] = 0.f; }
 
@@ -141,17 +144,17 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
 
   const bool always_general = SW < SK_KT;
 
-  auto logits = [&](int cur, int cb, f32x16 (&acc)[2]) {
+  auto logits = [&](int cur, int cb, f32x16 (&acc)[SK_RB]) {
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[rb][i] = 0.f;
     const char* kb = &kbuf[cur][(cb * 32 + lrow) * SK_ROWB + lhalf * 16];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       const uint4 bf = *reinterpret_cast<const uint4*>(kb + ks * 32);
-      acc[0] = sk_mfma<DTYPE>(qf[0][ks], bf, acc[0]);
-      acc[1] = sk_mfma<DTYPE>(qf[1][ks], bf, acc[1]);
+#pragma unroll
+      for (int rb = 0; rb < SK_RB; ++rb) acc[rb] = sk_mfma<DTYPE>(qf[rb][ks], bf, acc[rb]);
     }
   };
 
@@ -171,13 +174,13 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
       const bool slow = general || t == 0;
 #pragma unroll
       for (int cb = 0; cb < 2; ++cb) {
-        f32x16 acc[2];
+        f32x16 acc[SK_RB];
         logits(cur, cb, acc);
         // keys past the sequence end, and (causal) window keys later than the query, are masked
         if (masked_tile) {
           const int s = t * SK_KT + cb * 32 + lrow;
 #pragma unroll
-          for (int rb = 0; rb < 2; ++rb) {
+          for (int rb = 0; rb < SK_RB; ++rb) {
             // query index of register i is qi[rb] + lhalf*4 + (i/4)*8 + i%4: compare against constants
             const int d = causal ? s - SW - qi[rb] - lhalf * 4 : -1;
 #pragma unroll
@@ -188,7 +191,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
         if (slow) {
           // differences are formed before scaling: (-1e30) - (-1e30) = 0 exactly for still-masked rows
 #pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
+          for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
               const float tt = -acc[rb][i] * c;
@@ -198,7 +201,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
             }
         } else {
 #pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
+          for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) ls[rb][i] += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
         }
@@ -212,12 +215,12 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
     sweep1(always_general || attempt == 1);
     bool bad = false;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) bad |= !(ls[rb][i] <= 3.0e38f);   // inf or NaN
     if (attempt == 1 || !__syncthreads_or(bad)) break;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) { nm[rb][i] = -SK_NEG; ls[rb][i] = 0.f; }
   }
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
   // merge the per-lane states of each row across the 32 lanes of a half-wave and fold the
   // normaliser into the offset: p = exp2(logit * c + nm), nm = -(max * c) - log2(sum)
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb)
+  for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       float mm = nm[rb][i], ll = ls[rb][i];
@@ -268,11 +271,11 @@ __global__ __launch_bounds__(NW * 64, (NW <= 4 ? 2 : 1)) void snapkv_kernel(
     if (more) load_tile(t + 1);
 #pragma unroll
     for (int cb = 0; cb < 2; ++cb) {
-      f32x16 acc[2];
+      f32x16 acc[SK_RB];
       logits(cur, cb, acc);
       float vs = 0.f;
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+      for (int rb = 0; rb < SK_RB; ++rb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) vs += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
       vs += __shfl_xor(vs, 32, 64);
@@ -387,8 +390,8 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
              score_stride, keys->max_seq_len);
   const int G = num_q_heads / keys->num_kv_heads;
   const int rbt = G * ((window + 31) / 32);
-  const int waves = (rbt + 1) / 2;
-  FC_REQUIRE(waves <= 8, FC_EUNSUPPORTED, "%s: group of %d heads x window %d needs %d wavefronts (max 8)", who, G,
+  const int waves = (rbt + SK_RB - 1) / SK_RB;
+  FC_REQUIRE(waves <= 16, FC_EUNSUPPORTED, "%s: group of %d heads x window %d needs %d wavefronts (max 16)", who, G,
              window, waves);
   if (keys->max_seq_len == 0) return FC_OK;
   KvView kv = fc_make_view(keys);
@@ -404,7 +407,8 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
   if (waves <= 1) SK_LAUNCH(DT, 1);     \
   else if (waves <= 2) SK_LAUNCH(DT, 2);\
   else if (waves <= 4) SK_LAUNCH(DT, 4);\
-  else SK_LAUNCH(DT, 8)
+  else if (waves <= 8) SK_LAUNCH(DT, 8);\
+  else SK_LAUNCH(DT, 16)
   if (keys->dtype == FC_BF16) { SK_DISPATCH(FC_BF16); } else { SK_DISPATCH(FC_F16); }
 #undef SK_DISPATCH
 #undef SK_LAUNCH
