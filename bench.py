@@ -363,8 +363,66 @@ class DecodeWorkload(Workload):
                           "scaled by cached tokens and layers to one decode step"}
 
 
-WORKLOADS = {"snapkv": SnapKVWorkload, "knorm": KnormWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
+# ---------------------------------------------------------------------------------------------------
+# calibration: a plain copy of known size through fc_copy_tokens (for scaling FETCH_SIZE / WRITE_SIZE)
+# ---------------------------------------------------------------------------------------------------
+class CopyWorkload(Workload):
+    name = "copy-calibration-1GiB"
+    dtype_name = "bf16"
+    kernel_name = "compact_kernel"
+    metric = "tokens copied/sec"
+    unit = "tokens/s"
+
+    def __init__(self, seed, device):
+        super().__init__()
+        self.device = device
+        L, B, H, S = 1, 4, 8, 65536                       # 4 * 8 * 65536 * 256 B = 512 MiB per tensor
+        self.src = torch.randn((L, B, H, S, D), device=device, dtype=torch.float32).to(torch.bfloat16)
+        self.dst = torch.empty_like(self.src)
+        self.S = S
+        self.tokens_per_step = B * S
+        self.kernel_bytes = 2 * self.src.numel() * 2      # read once + written once
+        self.pass_bytes = self.kernel_bytes
+
+    def config(self):
+        return {"workload": self.name, "bytes_read": self.kernel_bytes // 2, "bytes_written": self.kernel_bytes // 2}
+
+    def step(self):
+        from fastcache_amd import _lib, ops
+        with self.br:
+            ops.copy_tokens(_lib.dense_view(self.src), _lib.dense_view(self.dst), 0, self.S, 0)
+
+    def cpu_baseline(self, budget_s=0):
+        threads = _cpu_threads()
+        a = self.src[0, :1].cpu()
+        t0 = time.perf_counter()
+        b = a.clone()
+        dt = time.perf_counter() - t0
+        return {"value": round(a.shape[0] * a.shape[2] / dt, 1), "unit": self.unit, "cores": threads, "kind": "port",
+                "sample": "torch clone of 1 of 4 sequences on the host"}
+
+
+WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
              "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True)}
+
+
+# HBM-side bytes per launch of a workload's dominant kernel, from two rocprofv3 counter runs
+# (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter reads for the
+# copy workload below, whose traffic is known (512 MiB read, 512 MiB written):
+#   copy:   FETCH_SIZE 2.634e5 KiB -> scale 1.990;  WRITE_SIZE 5.269e5 KiB -> scale 0.995
+# The commands and raw readings are in profiles/*_hbm_traffic.txt.
+_FETCH_SCALE = 524288 / 2.634e5
+_WRITE_SCALE = 524288 / 5.269e5
+_COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
+    "cfg2-snapkv-qwen3-8b": (2.491e6, 1.423e5),
+}
+
+
+def _measured_traffic(workload_name):
+    kib = _COUNTER_KIB.get(workload_name)
+    if kib is None:
+        return None
+    return int(round((kib[0] * _FETCH_SCALE + kib[1] * _WRITE_SCALE) * 1024))
 
 
 def main():
@@ -405,7 +463,7 @@ def main():
     k_ms = w.br.mean_ms() / w.launches_per_bracket
     achieved = w.kernel_bytes / w.launches_per_bracket / (k_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": w.kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _measured_traffic(w.name),
                 "kernel_ms": round(k_ms, 4), "launches_per_step": w.launches_per_bracket,
                 "algorithmic_bytes_per_launch": w.kernel_bytes // w.launches_per_bracket,
                 "pass_gbs": round(w.pass_bytes / (ms_per_step * 1e-3) / 1e9, 1),

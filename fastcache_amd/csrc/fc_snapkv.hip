@@ -1,22 +1,26 @@
 // SnapKV observation-window scoring for fp16/bf16 caches.
 //
-// One workgroup per (layer, sequence, kv head).  Each wavefront keeps 64 query rows (two 32-row
-// blocks of one or two query heads of the group) as MFMA A-operands in registers for the whole
-// kernel.  Keys stream through LDS in tiles of 64 (double buffered, rows padded to 272 bytes so
-// that the 16-byte B-operand reads of a half-wave fall on distinct banks) and are multiplied
-// with v_mfma_f32_32x32x16, giving each lane 16 logits per 32x32 block: 16 query rows of one
-// key column.
+// One workgroup per (layer, sequence, kv head) with one wavefront per 32-row block of window
+// queries (group of G query heads x ceil(W/32) blocks, up to 16 wavefronts).  A wavefront keeps
+// its 32 query rows as MFMA A-operands in registers for the whole kernel.  Keys stream through
+// LDS in tiles of 64 (double buffered, rows padded to 272 bytes so that the 16-byte B-operand
+// reads of a half-wave fall on distinct banks) and are multiplied with v_mfma_f32_32x32x16,
+// giving each lane 16 logits per 32x32 block: 16 query rows of one key column.
 //
 // The softmax needs every key of a row before any probability is final, and the [G*W, S] logit
 // matrix does not fit on chip, so the keys are swept twice:
-//   sweep 1  per-lane running (offset, sum of exp2) for each of the lane's 32 query rows, with a
-//            lazily moved offset (it only has to stay within 2^40 of the running maximum), then
-//            one cross-lane merge per row at the end;
+//   sweep 1  per-lane (offset, sum of exp2) for each of the lane's 16 query rows.  The first tile
+//            fixes the offset with the online-softmax update; later tiles only add
+//            exp2(logit - offset).  Should a sum overflow, the sweep is redone with the online
+//            update on every tile.  One cross-lane merge per row at the end;
 //   sweep 2  logits recomputed, p = exp2(x - m) / l summed over the lane's rows, the two
 //            half-waves and the group's wavefronts (fixed order, no atomics) into a 4-tile ring
 //            of per-key sums, from which the zero-padded moving average of width `kernel_size`
 //            is written two tiles later.
-// All arithmetic after the MFMA is fp32.  Sweep 2 mostly hits L2 / Infinity Cache for K.
+// All arithmetic after the MFMA is fp32.  The second sweep reads K again (a workgroup's column
+// does not stay in L2 between the sweeps), so the kernel's memory traffic is about twice the
+// algorithmic figure; its run time is set by the exponentials, not by that traffic.
+// Optionally the kernel also emits the maximum of each score row for the window fill.
 #include "fc_common.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -29,7 +33,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 #define SK_KT 64          // keys per tile
 #define SK_ROWB 272       // LDS bytes per key row (256 + 16 pad)
 #define SK_NEG (-1.0e30f) // "minus infinity" that stays finite under subtraction
-#define SK_LAZY 40.0f     // allowed excess (log2 units) of a logit over the lane's offset
 #define SK_TBL 1024       // block-table entries of one sequence cached in LDS
 
 template <int DTYPE>
