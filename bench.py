@@ -270,7 +270,7 @@ class CCMWorkload(Workload):
         threads = _cpu_threads()
         sd = {k: v.detach().cpu().float() for k, v in self.module.state_dict().items()}
         fwd = occm.hybrid_forward if self.hybrid else occm.linear_decouple_forward
-        nb = 1 if self.hybrid else 4
+        nb = self.B
         tables, lens = self.case.block_tables[:nb], [self.S] * nb
         t_total, done = 0.0, 0
         for layer in range(self.L):
