@@ -2,38 +2,42 @@
 //
 // One workgroup per (layer, sequence, kv head) with one wavefront per 32-row block of window
 // queries (group of G query heads x ceil(W/32) blocks, up to 16 wavefronts).  A wavefront keeps
-// its 32 query rows as MFMA A-operands in registers for the whole kernel.  Keys stream through
-// LDS in tiles of 64 (double buffered, rows padded to 272 bytes so that the 16-byte B-operand
-// reads of a half-wave fall on distinct banks) and are multiplied with v_mfma_f32_32x32x16,
-// giving each lane 16 logits per 32x32 block: 16 query rows of one key column.
+// its 32 query rows as MFMA operands in registers for the whole kernel.  Keys stream through LDS
+// in tiles of 64 rows: global memory -> LDS directly (global_load_lds_dwordx4, no register
+// staging), three or four tiles resident or in flight per workgroup, one barrier per tile.  Rows
+// are unpadded; their 16-byte chunks are XOR-swizzled with the row number so that the operand
+// reads of a half-wave (32 rows, same chunk) fall on distinct banks.  Logits come from
+// v_mfma_f32_32x32x16, 16 per lane and 32x32 block.
 //
 // The softmax needs every key of a row before any probability is final, and the [G*W, S] logit
 // matrix does not fit on chip, so the keys are swept twice:
-//   sweep 1  per-lane (offset, sum of exp2) for each of the lane's 16 query rows.  The first tile
-//            fixes the offset with the online-softmax update; later tiles only add
-//            exp2(logit - offset).  Should a sum overflow, the sweep is redone with the online
-//            update on every tile.  One cross-lane merge per row at the end;
-//   sweep 2  logits recomputed, p = exp2(x - m) / l summed over the lane's rows, the two
-//            half-waves and the group's wavefronts (fixed order, no atomics) into a 4-tile ring
-//            of per-key sums, from which the zero-padded moving average of width `kernel_size`
-//            is written two tiles later.
-// All arithmetic after the MFMA is fp32.  The second sweep reads K again (a workgroup's column
-// does not stay in L2 between the sweeps), so the kernel's memory traffic is about twice the
-// algorithmic figure; its run time is set by the exponentials, not by that traffic.
+//   sweep 1  C[key][query] orientation: a lane owns ONE query and 16 keys per block, so its
+//            softmax state is two scalars (largest logit, sum of exp2).  The first tile fixes the
+//            offset with the online-softmax update; later tiles only add exp2(logit - offset).
+//            Should a sum overflow, the sweep is redone with the online update on every tile;
+//   sweep 2  C[query][key] orientation, tiles in descending order (the tiles read last are the
+//            likeliest to still be cached): logits recomputed, p = exp2(x - m) / l summed over the
+//            lane's 16 queries, the two half-waves and the group's wavefronts (fixed order, no
+//            atomics) into a 4-tile ring of per-key sums, from which the zero-padded moving
+//            average of width `kernel_size` is written one tile later.
+// In both sweeps the MFMAs of a block are issued together with the exponentials of the block
+// before it (two accumulator sets, sched_group_barrier hints).  All arithmetic after the MFMA is
+// fp32.  The second sweep reads K again (a workgroup's column does not stay in L2 between the
+// sweeps), so the kernel's memory traffic is about twice the algorithmic figure.
 // Optionally the kernel also emits the maximum of each score row for the window fill.
+//
+// Table entries of a live sequence must be allocated blocks: a negative entry inside the sequence
+// reads block 0 instead of faulting.
 #include "fc_common.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-#ifndef SK_RB
-#define SK_RB 1          // 32-row query blocks per wavefront
-#endif
-#define SK_KT 64          // keys per tile
-#define SK_ROWB 272       // LDS bytes per key row (256 + 16 pad)
-#define SK_NEG (-1.0e30f) // "minus infinity" that stays finite under subtraction
-#define SK_TBL 1024       // block-table entries of one sequence cached in LDS
+#define SK_KT 64           // keys per tile
+#define SK_TILEB (SK_KT * 256)  // LDS bytes per key tile (rows unpadded, 16-byte chunks XOR-swizzled)
+#define SK_NEG (-1.0e30f)  // "minus infinity" that stays finite under subtraction
+#define SK_TBL 1024        // block-table entries of one sequence cached in LDS
 
 template <int DTYPE>
 __device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16 c) {
@@ -47,26 +51,65 @@ __device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16
 
 __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int DTYPE, int NW>
-__global__ __launch_bounds__(NW * 64, (SK_RB == 2 ? (NW <= 4 ? 2 : 1) : (NW <= 4 ? 4 : NW <= 8 ? 4 : 2))) void snapkv_kernel(
+__device__ __forceinline__ unsigned sk_lds_addr(const void* p) {
+  return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16 (lds_base is
+// wave-uniform).  The load is counted in vmcnt; the compiler does not know it writes LDS, so
+// every consumer sits behind sk_wait_barrier.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void sk_load_lds(const char* g, unsigned lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
+               : "memory", "m0");
+}
+// same with a wave-uniform 64-bit base and a 32-bit per-lane byte offset
+__device__ __forceinline__ void sk_load_lds(const char* g_uniform, unsigned lane_off, unsigned lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_off),
+               "s"(g_uniform)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+// Wait until at most N vector-memory operations of this wave are outstanding and all its LDS
+// operations are done, then synchronise the workgroup.
+template <int N>
+__device__ __forceinline__ void sk_wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int NW>
+struct SkCfg {
+  static constexpr int ST = NW >= 8 ? 4 : 3;   // key tiles resident or in flight per workgroup
+  static constexpr int LDS = ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4 + SK_TBL * 4;
+};
+
+template <int DTYPE, int NW, bool FAST>
+__global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     KvView kv, const char* __restrict__ q, int Hq, int W, int ksz, int causal, float c, float out_mul,
     float* __restrict__ scores, int score_stride, float* __restrict__ row_max) {
   constexpr int THREADS = NW * 64;
-  constexpr int CHUNKS = SK_KT * 16;                        // 16-byte chunks per key tile
-  constexpr int CH = (CHUNKS + THREADS - 1) / THREADS;      // chunks per thread
-  __shared__ __align__(16) char kbuf[2][SK_KT * SK_ROWB];
-  __shared__ float vpart[2][NW][SK_KT];
-  __shared__ float vraw[4][SK_KT];
-  __shared__ int tbl[SK_TBL];
+  constexpr int ST = SkCfg<NW>::ST;
+  constexpr int LPW = 16 / NW;   // 1 KB wave-loads (4 key rows) per wavefront and tile
+  static_assert(LPW * NW == 16, "NW must divide 16");
+  extern __shared__ __align__(16) char smem[];
+  char* kbuf = smem;
+  float(*vpart)[NW][SK_KT] = reinterpret_cast<float(*)[NW][SK_KT]>(smem + ST * SK_TILEB);
+  float(*vraw)[SK_KT] = reinterpret_cast<float(*)[SK_KT]>(smem + ST * SK_TILEB + 4 * NW * SK_KT * 4);
+  int* tbl = reinterpret_cast<int*>(smem + ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4);
 
   const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
   const int Hkv = kv.num_kv_heads;
   const int G = Hq / Hkv;
   const int WB = (W + 31) / 32;        // 32-row blocks per query head
   const int RBT = G * WB;              // row blocks of the group
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane & 31, lhalf = lane >> 5;
-  const int S = fc_seq_len(kv, b);
+  const int S = __builtin_amdgcn_readfirstlane(fc_seq_len(kv, b));
   float* out_row = scores + (((long long)l * kv.batch + b) * Hkv + h) * (long long)score_stride;
 
   if (S <= W) {  // nothing outside the window to score
@@ -77,23 +120,18 @@ __global__ __launch_bounds__(NW * 64, (SK_RB == 2 ? (NW <= 4 ? 2 : 1) : (NW <= 4
   const int SW = S - W;                       // scored keys
   const int T = (S + SK_KT - 1) / SK_KT;      // key tiles
 
-  // ---- query fragments ------------------------------------------------------------------
-  uint4 qf[SK_RB][8];
-  int qi[SK_RB];      // query index (within the window) of this lane's A row
-  bool rb_valid[SK_RB];
-#pragma unroll
-  for (int rb = 0; rb < SK_RB; ++rb) {
-    const int blk = wave * SK_RB + rb;
-    rb_valid[rb] = blk < RBT;
-    const int g = rb_valid[rb] ? blk / WB : 0;
-    const int wb = rb_valid[rb] ? blk - g * WB : 0;
-    qi[rb] = wb * 32;
-    const int qa = wb * 32 + lrow;
-    const bool ok = rb_valid[rb] && qa < W;
-    const char* qp = q + (((((long long)l * kv.batch + b) * Hq + (h * G + g)) * W + qa) * FC_HEAD_DIM + lhalf * 8) * 2;
+  // ---- query fragment: this wavefront's 32 query rows as MFMA A-operands ------------------
+  uint4 qf[8];
+  const bool rb_valid = wave < RBT;
+  const int qg = rb_valid ? wave / WB : 0;
+  const int qi = (rb_valid ? wave - qg * WB : 0) * 32;   // first query index of the block
+  {
+    const int qa = qi + lrow;
+    const bool ok = rb_valid && qa < W;
+    const char* qp = q + (((((long long)l * kv.batch + b) * Hq + (h * G + qg)) * W + qa) * FC_HEAD_DIM + lhalf * 8) * 2;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
-      qf[rb][ks] = ok ? *reinterpret_cast<const uint4*>(qp + ks * 32) : make_uint4(0, 0, 0, 0);
+      qf[ks] = ok ? *reinterpret_cast<const uint4*>(qp + ks * 32) : make_uint4(0, 0, 0, 0);
   }
 
   // this sequence's block-table row, so that the tile loads do not wait on a table read each
@@ -103,211 +141,278 @@ __global__ __launch_bounds__(NW * 64, (SK_RB == 2 ? (NW <= 4 ? 2 : 1) : (NW <= 4
     const int nblk = ((S - 1) >> kv.block_shift) + 1;
     for (int i = tid; i < nblk; i += THREADS) tbl[i] = kv.block_tables[(long long)b * kv.table_stride + i];
   }
-  const char* kbase = kv.base + ((long long)l * kv.stride_layer + (long long)h * kv.stride_head) * 2;
-  uint4 pre[CH];
-  auto load_tile = [&](int t) {
-#pragma unroll
-    for (int u = 0; u < CH; ++u) {
-      const int ch = tid + u * THREADS;
-      const int key = ch >> 4, part = ch & 15;
-      const int s = t * SK_KT + key;
-      pre[u] = make_uint4(0, 0, 0, 0);
-      if (ch < CHUNKS && s < S) {
-        long long off;
-        if (tbl_lds) {
-          const int blk = tbl[s >> kv.block_shift];
-          off = blk < 0 ? -1 : (long long)blk * kv.stride_block + (long long)(s & (kv.block_size - 1)) * kv.stride_token;
-        } else {
-          off = fc_token_offset(kv, b, s);
-        }
-        if (off >= 0) pre[u] = *reinterpret_cast<const uint4*>(kbase + off * 2 + part * 16);
-      }
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < CH; ++u) {
-      const int ch = tid + u * THREADS;
-      if (ch < CHUNKS) *reinterpret_cast<uint4*>(&kbuf[buf][(ch >> 4) * SK_ROWB + (ch & 15) * 16]) = pre[u];
-    }
-  };
-
-  // per-lane softmax state for the lane's 2 x 16 query rows: nm = -(offset * c), ls = sum of
-  // exp2(logit * c + nm) over the keys this lane has seen
-  float nm[SK_RB][16], ls[SK_RB][16];
-#pragma unroll
-  for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) { nm[rb][i] = -SK_NEG; ls[rb][i] = 0.f; }
-
-  __syncthreads();  // tbl
-  load_tile(0);
-  store_tile(0);
   __syncthreads();
 
-  const bool always_general = SW < SK_KT;
+  // ---- key tiles: global -> LDS, ST stages ---------------------------------------------------
+  // A wave-load moves 4 key rows (1 KB).  Lane i writes LDS chunk i of those 64 chunks and fetches
+  // the global chunk (i & 15) ^ (row & 15) of row i / 16, which is the XOR swizzle that keeps the
+  // B-operand reads (32 rows, same chunk) free of bank conflicts.  Rows past the sequence end are
+  // clamped to its last row (every lane always loads, so the outstanding-load count is exact);
+  // those keys are masked in sweep 1 and never emitted in sweep 2.
+  const char* kbase = kv.base + ((long long)l * kv.stride_layer + (long long)h * kv.stride_head) * 2;
+  const unsigned kbuf_lds = __builtin_amdgcn_readfirstlane(sk_lds_addr(kbuf));
+  // FAST: a tile lies inside one page (or the view is dense), so a load is a wave-uniform tile base
+  // plus a per-lane byte offset; the offset is recomputed per load rather than kept in registers.
+  const unsigned tok_bytes = (unsigned)kv.stride_token * 2;
+  auto issue = [&](int tile, int stage) {
+    if constexpr (FAST) {
+      const int s0 = tile * SK_KT;
+      long long tb;
+      if (paged) {
+        const int blk = max(__builtin_amdgcn_readfirstlane(tbl[s0 >> kv.block_shift]), 0);
+        tb = (long long)blk * kv.stride_block + (long long)(s0 & (kv.block_size - 1)) * kv.stride_token;
+      } else {
+        tb = (long long)b * kv.stride_batch + (long long)s0 * kv.stride_token;
+      }
+      const char* g = kbase + tb * 2;
+      const int rmax = S - 1 - s0;   // rows past the end re-read the last row
+#pragma unroll
+      for (int u = 0; u < LPW; ++u) {
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int r = 4 * (wave * LPW + u) + (ln >> 4);
+        const unsigned lo = (unsigned)min(r, rmax) * tok_bytes + (((ln & 15) ^ (r & 15)) << 4);
+        sk_load_lds(g, lo, kbuf_lds + stage * SK_TILEB + (wave * LPW + u) * 1024);
+      }
+    } else {
+#pragma unroll 1
+    for (int u = 0; u < LPW; ++u) {
+      const int j = wave * LPW + u;
+      const int r = 4 * j + (lane >> 4);
+      const int ch = (lane & 15) ^ (r & 15);
+      const int s = min(tile * SK_KT + r, S - 1);
+      long long off = fc_token_offset(kv, b, s);
+      if (off < 0) off = 0;
+      sk_load_lds(kbase + off * 2 + ch * 16, kbuf_lds + stage * SK_TILEB + j * 1024);
+    }
+    }
+  };
+  // One plan = sweep 1 over the tiles in ascending order, then sweep 2 in descending order (the
+  // tiles read last are the likeliest to still be cached).  m is the position in the plan, kc the
+  // number of tiles consumed so far; tile position m lives in stage (kc % ST) when it is consumed
+  // and positions m+1 .. m+ST-2 are in flight meanwhile.
+  auto plan_tile = [&](int pos) { return pos < T ? pos : 2 * T - 1 - pos; };
+  int kc = 0, m = 0;
+  auto prologue = [&]() {
+    m = 0;
+    for (int i = 0; i < ST - 1 && i < 2 * T; ++i) issue(plan_tile(i), (kc + i) % ST);
+  };
+  // top of a tile iteration: tile position m has landed for every wave, the stage consumed by the
+  // previous iteration is free and receives position m+ST-1; returns the stage to read
+  auto acquire = [&]() {
+    if (m + ST - 2 < 2 * T) sk_wait_barrier<LPW*(ST - 2)>(); else sk_wait_barrier<0>();
+    const int nx = m + ST - 1;
+    if (nx < 2 * T) issue(plan_tile(nx), (kc + ST - 1) % ST);
+    return kc % ST;
+  };
 
-  auto logits = [&](int cur, int cb, f32x16 (&acc)[SK_RB]) {
+  const bool always_general = SW < SK_KT;
+  const int swz = lrow & 15;
+
+  // LDS address of the lane's fragment of k-slice ks of a 32-key block: the row base plus the
+  // swizzled chunk ((ks*2 + lhalf) ^ swz) * 16.  ks*32, lhalf*16 and the row base occupy disjoint
+  // bits, so this is (row base + xs) ^ (ks*32).
+  const unsigned xs = (unsigned)((lhalf ^ swz) << 4) + lrow * 256;
+  // 32 keys x 32 queries of logits.  KEYS_ROWS: C[key][query] (the lane owns one query and 16
+  // keys), otherwise C[query][key] (the lane owns one key and 16 queries).
+  auto mfma_block = [&](bool keys_rows, int stage, int cb, f32x16& acc) {
 #pragma unroll
-    for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[rb][i] = 0.f;
-    const char* kb = &kbuf[cur][(cb * 32 + lrow) * SK_ROWB + lhalf * 16];
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    const unsigned a0 = (unsigned)(stage * SK_TILEB + cb * 8192) + xs;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      const uint4 bf = *reinterpret_cast<const uint4*>(kb + ks * 32);
+      const uint4 kf = *reinterpret_cast<const uint4*>(kbuf + (a0 ^ (unsigned)(ks * 32)));
+      acc = keys_rows ? sk_mfma<DTYPE>(kf, qf[ks], acc) : sk_mfma<DTYPE>(qf[ks], kf, acc);
+    }
+  };
+  // ask the scheduler to spread the VALU work of one block between the MFMAs of the next
+  auto interleave = [&]() {
 #pragma unroll
-      for (int rb = 0; rb < SK_RB; ++rb) acc[rb] = sk_mfma<DTYPE>(qf[rb][ks], bf, acc[rb]);
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);   // seven VALU
     }
   };
 
-  // ================= sweep 1: per-lane softmax statistics ======================================
-  // Tile 0 sets every lane-row's offset with the general (online-softmax) update.  Later tiles only
-  // add exp2(logit * c + nm): any fixed offset is mathematically valid, it merely has to keep the
+  // ================= sweep 1: softmax statistics ==============================================
+  // C[key][query]: lane (lrow, lhalf) owns query qi + lrow and, per 32-key block, the 16 keys
+  // (i/4)*8 + lhalf*4 + i%4.  Its state is (mref, lsq): the largest raw logit seen and the sum of
+  // exp2((logit - mref) * c).  The first tile uses the online update; later tiles only add
+  // exp2(logit * c - mref * c): any fixed offset is mathematically valid, it merely has to keep the
   // sums inside the fp32 range.  A sum that overflows (logits rising by more than ~2^7 in log2
-  // units above the first tile's) is detected afterwards and the sweep is redone with the general
-  // update on every tile.
-  int pb = 0;   // LDS buffer parity of tile 0 of the current sweep
-  auto sweep1 = [&](bool general) {
-    for (int t = 0; t < T; ++t) {
-      const int cur = (pb + t) & 1;
-      load_tile(t + 1 < T ? t + 1 : 0);   // the tile after the last one is tile 0 of the next sweep
-      const int tile_end = (t + 1) * SK_KT;
-      const bool masked_tile = tile_end > S || (causal && tile_end > SW + 1);
-      const bool slow = general || t == 0;
+  // units above the first tile's) is detected afterwards and the sweep is redone with the online
+  // update on every tile.  Masked logits are SK_NEG; differences are formed before scaling so that
+  // SK_NEG - SK_NEG is exactly 0 and nothing overflows.
+  float mref = SK_NEG, lsq = 0.f, nmq = 0.f;
+  const int klim = causal ? min(S, SW + qi + lrow + 1) : S;   // first masked key of this lane's query
+  auto stats_general = [&](f32x16& acc, int t, int cb) {
+    const int sb = t * SK_KT + cb * 32 + lhalf * 4;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (sb + (i >> 2) * 8 + (i & 3) >= klim) acc[i] = SK_NEG;
+    float mx = acc[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, acc[i]);
+    float bs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) bs += sk_exp2((acc[i] - mx) * c);
+    const float mnew = fmaxf(mref, mx);
+    lsq = lsq * sk_exp2((mref - mnew) * c) + bs * sk_exp2((mx - mnew) * c);
+    mref = mnew;
+  };
+  auto stats_fast = [&](const f32x16& acc) {
+    float bs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) bs += sk_exp2(fmaf(acc[i], c, nmq));
+    lsq += bs;
+  };
+  // tiles [t0, t1) one block at a time, with masking; fixed offset unless `general`
+  auto sweep1_plain = [&](int t0, int t1, bool general) {
+    for (int t = t0; t < t1; ++t) {
+      const int stage = acquire();
 #pragma unroll
       for (int cb = 0; cb < 2; ++cb) {
-        f32x16 acc[SK_RB];
-        logits(cur, cb, acc);
-        // keys past the sequence end, and (causal) window keys later than the query, are masked
-        if (masked_tile) {
-          const int s = t * SK_KT + cb * 32 + lrow;
-#pragma unroll
-          for (int rb = 0; rb < SK_RB; ++rb) {
-            // query index of register i is qi[rb] + lhalf*4 + (i/4)*8 + i%4: compare against constants
-            const int d = causal ? s - SW - qi[rb] - lhalf * 4 : -1;
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-              if (s >= S || d > ((i >> 2) * 8 + (i & 3))) acc[rb][i] = SK_NEG;
-          }
-        }
-        if (slow) {
-          // differences are formed before scaling: (-1e30) - (-1e30) = 0 exactly for still-masked rows
-#pragma unroll
-          for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const float tt = -acc[rb][i] * c;
-              const float mn = fminf(nm[rb][i], tt);
-              ls[rb][i] = ls[rb][i] * sk_exp2(mn - nm[rb][i]) + sk_exp2(mn - tt);
-              nm[rb][i] = mn;
-            }
+        f32x16 acc;
+        mfma_block(true, stage, cb, acc);
+        if (general) {
+          stats_general(acc, t, cb);
         } else {
+          const int sb = t * SK_KT + cb * 32 + lhalf * 4;
 #pragma unroll
-          for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) ls[rb][i] += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
+          for (int i = 0; i < 16; ++i)
+            if (sb + (i >> 2) * 8 + (i & 3) >= klim) acc[i] = SK_NEG;
+          stats_fast(acc);
         }
       }
-      store_tile(cur ^ 1);
-      __syncthreads();
+      ++m;
+      ++kc;
     }
-    pb += T;
   };
-  for (int attempt = 0; attempt < 2; ++attempt) {   // one inlined copy of the sweep
-    sweep1(always_general || attempt == 1);
-    bool bad = false;
-#pragma unroll
-    for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) bad |= !(ls[rb][i] <= 3.0e38f);   // inf or NaN
-    if (attempt == 1 || !__syncthreads_or(bad)) break;
-#pragma unroll
-    for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) { nm[rb][i] = -SK_NEG; ls[rb][i] = 0.f; }
+  // unmasked tiles [t0, t1), t1 > t0, fixed offset: the MFMAs of each block are issued together
+  // with the exponentials of the block before it
+  auto sweep1_piped = [&](int t0, int t1) {
+    f32x16 acc_a, acc_b;
+    int stage = acquire();
+    mfma_block(true, stage, 0, acc_a);
+    for (int t = t0; t < t1 - 1; ++t) {
+      mfma_block(true, stage, 1, acc_b);
+      stats_fast(acc_a);
+      interleave();
+      ++m;
+      ++kc;
+      stage = acquire();
+      mfma_block(true, stage, 0, acc_a);
+      stats_fast(acc_b);
+      interleave();
+    }
+    mfma_block(true, stage, 1, acc_b);
+    stats_fast(acc_a);
+    interleave();
+    stats_fast(acc_b);
+    ++m;
+    ++kc;
+  };
+  // leading tiles without any masked key
+  const int TF = causal ? min(S, SW + 1) / SK_KT : S / SK_KT;
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    prologue();
+    if (always_general || attempt == 1) {
+      sweep1_plain(0, T, true);
+    } else {
+      sweep1_plain(0, 1, true);
+      nmq = -mref * c;
+      if (TF > 1) sweep1_piped(1, TF);
+      sweep1_plain(max(TF, 1), T, false);
+    }
+    const bool bad = !(lsq <= 3.0e38f);   // inf or NaN
+    if (attempt == 1 || !__builtin_amdgcn_readfirstlane(__syncthreads_or(bad))) break;
+    sk_wait_barrier<0>();   // the tiles prefetched for sweep 2 land before their stages are reused
+    mref = SK_NEG;
+    lsq = 0.f;
   }
 
-  // merge the per-lane states of each row across the 32 lanes of a half-wave and fold the
-  // normaliser into the offset: p = exp2(logit * c + nm), nm = -(max * c) - log2(sum)
+  // merge the two half-waves' states of each query and fold the normaliser into the offset:
+  // p = exp2(logit * c + nmfin), nmfin = -(max * c) - log2(sum).  Then hand every lane the offsets
+  // of the 16 queries it owns in the C[query][key] orientation of sweep 2.
+  float nm[16];
+  {
+    const float m2 = __shfl_xor(mref, 32, 64), l2 = __shfl_xor(lsq, 32, 64);
+    const float mnew = fmaxf(mref, m2);
+    const float ll = lsq * sk_exp2((mref - mnew) * c) + l2 * sk_exp2((m2 - mnew) * c);
+    const bool ok = rb_valid && qi + lrow < W;
+    const float nmfin = ok ? -mnew * c - __builtin_amdgcn_logf(ll) : SK_NEG;   // v_log_f32 is log2
 #pragma unroll
-  for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float mm = nm[rb][i], ll = ls[rb][i];
-#pragma unroll
-      for (int o = 1; o < 32; o <<= 1) {
-        const float m2 = __shfl_xor(mm, o, 64), l2 = __shfl_xor(ll, o, 64);
-        const float mn = fminf(mm, m2);
-        ll = ll * sk_exp2(mn - mm) + l2 * sk_exp2(mn - m2);
-        mm = mn;
-      }
-      const int qa = qi[rb] + (i >> 2) * 8 + lhalf * 4 + (i & 3);
-      const bool ok = rb_valid[rb] && qa < W;
-      nm[rb][i] = ok ? mm - __builtin_amdgcn_logf(ll) : SK_NEG;   // v_log_f32 is log2
-    }
+    for (int i = 0; i < 16; ++i) nm[i] = __shfl(nmfin, (i >> 2) * 8 + lhalf * 4 + (i & 3), 64);
+  }
 
   // ================= sweep 2: probabilities, per-key sums, moving average ======================
-  for (int t = 0; t < T; ++t) {
-    const int cur = (pb + t) & 1;
-    if (t >= 1 && tid < SK_KT) {
-      // fold the wavefronts' partial sums of tile t-1 (fixed order) into the ring
-      float v = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) v += vpart[cur ^ 1][w][tid];
-      vraw[(t - 1) & 3][tid] = v;
-      // moving average for tile t-3: its neighbours t-4 .. t-2 are complete
-      if (t >= 3) {
-        const int s = (t - 3) * SK_KT + tid;
-        if (s < SW) {
-          float acc = 0.f;
-          const int hw = ksz >> 1;
-          for (int j = -hw; j <= hw; ++j) {
-            const int x = s + j;
-            if (x >= 0 && x < SW) acc += vraw[(x / SK_KT) & 3][x % SK_KT];
-          }
-          out_row[s] = acc * out_mul;
-        }
-      }
+  // C[query][key], tiles in descending order.  Every wavefront leaves its per-key sums of a tile in
+  // vpart (four tiles deep); wave 0 folds them (fixed order) into vraw, a ring of four tiles, and
+  // writes the moving average of a tile once both neighbours are folded.
+  const int hw = ksz >> 1;
+  auto emit = [&](int s) {   // scored key s: zero-padded moving average over [s-hw, s+hw]
+    float acc = 0.f;
+    for (int j = -hw; j <= hw; ++j) {
+      const int x = s + j;
+      if (x >= 0 && x < SW) acc += vraw[(x / SK_KT) & 3][x % SK_KT];
     }
-    const bool more = t + 1 < T;
-    if (more) load_tile(t + 1);
-#pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-      f32x16 acc[SK_RB];
-      logits(cur, cb, acc);
-      float vs = 0.f;
-#pragma unroll
-      for (int rb = 0; rb < SK_RB; ++rb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) vs += sk_exp2(fmaf(acc[rb][i], c, nm[rb][i]));
-      vs += __shfl_xor(vs, 32, 64);
-      if (lane < 32) vpart[cur][wave][cb * 32 + lane] = vs;
-    }
-    if (more) store_tile(cur ^ 1);
-    __syncthreads();
-  }
-  const int last_buf = (pb + T - 1) & 1;
-
-  // ---- drain: last tile's sums, then the moving average of the last three tiles ------------
-  if (tid < SK_KT) {
+    out_row[s] = acc * out_mul;
+  };
+  auto fold = [&](int u) {   // tile processed u-th (tile T-1-u): sum the wavefronts' partial sums
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) v += vpart[last_buf][w][tid];
-    vraw[(T - 1) & 3][tid] = v;
+    for (int w = 0; w < NW; ++w) v += vpart[u & 3][w][lane];
+    vraw[(T - 1 - u) & 3][lane] = v;
+  };
+  auto probs = [&](const f32x16& acc, int u, int cb) {
+    float vs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) vs += sk_exp2(fmaf(acc[i], c, nm[i]));
+    vs += __shfl_xor(vs, 32, 64);
+    if (lane < 32) vpart[u & 3][wave][cb * 32 + lane] = vs;
+  };
+  {
+    f32x16 acc_a, acc_b;
+    int stage = acquire();
+    mfma_block(false, stage, 0, acc_a);
+    for (int u = 0; u < T - 1; ++u) {
+      mfma_block(false, stage, 1, acc_b);
+      probs(acc_a, u, 0);
+      interleave();
+      ++m;
+      ++kc;
+      stage = acquire();
+      if (u >= 1 && wave == (u & (NW - 1))) {
+        // the sums of the tile processed before this one are complete: fold them (the wavefronts
+        // take turns), then the tile before that (T-u+1) has both neighbours
+        fold(u - 1);
+        if (u >= 2) {
+          const int s = (T - u + 1) * SK_KT + lane;
+          if (s < SW) emit(s);
+        }
+      }
+      mfma_block(false, stage, 0, acc_a);
+      probs(acc_b, u, 1);
+      interleave();
+    }
+    mfma_block(false, stage, 1, acc_b);
+    probs(acc_a, T - 1, 0);
+    interleave();
+    probs(acc_b, T - 1, 1);
+    ++m;
+    ++kc;
+  }
+
+  // ---- drain: the last two tiles' sums, then the moving average of tiles 2, 1, 0 ---------------
+  __syncthreads();
+  if (wave == 0) {
+    if (T >= 2) fold(T - 2);
+    fold(T - 1);
   }
   __syncthreads();
   {
-    const int first = T >= 3 ? (T - 3) * SK_KT : 0;
-    const int hw = ksz >> 1;
-    for (int s = first + tid; s < SW; s += THREADS) {
-      float acc = 0.f;
-      for (int j = -hw; j <= hw; ++j) {
-        const int x = s + j;
-        if (x >= 0 && x < SW) acc += vraw[(x / SK_KT) & 3][x % SK_KT];
-      }
-      out_row[s] = acc * out_mul;
-    }
+    const int last = min(3 * SK_KT, SW);
+    for (int s = tid; s < last; s += THREADS) emit(s);
     for (int s = S + tid; s < score_stride; s += THREADS) out_row[s] = -INFINITY;
   }
   if (row_max) {   // maximum of this row's scores, for the window fill: re-read what this workgroup wrote
@@ -318,10 +423,10 @@ __global__ __launch_bounds__(NW * 64, (SK_RB == 2 ? (NW <= 4 ? 2 : 1) : (NW <= 4
     if (lane == 0) vpart[0][wave][0] = rmax;
     __syncthreads();
     if (tid == 0) {
-      float m = vpart[0][0][0];
+      float mx = vpart[0][0][0];
 #pragma unroll
-      for (int w = 1; w < NW; ++w) m = fmaxf(m, vpart[0][w][0]);
-      row_max[((long long)l * kv.batch + b) * Hkv + h] = m;
+      for (int w = 1; w < NW; ++w) mx = fmaxf(mx, vpart[0][w][0]);
+      row_max[((long long)l * kv.batch + b) * Hkv + h] = mx;
     }
   }
 }
@@ -393,7 +498,7 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
              score_stride, keys->max_seq_len);
   const int G = num_q_heads / keys->num_kv_heads;
   const int rbt = G * ((window + 31) / 32);
-  const int waves = (rbt + SK_RB - 1) / SK_RB;
+  const int waves = rbt;
   FC_REQUIRE(waves <= 16, FC_EUNSUPPORTED, "%s: group of %d heads x window %d needs %d wavefronts (max 16)", who, G,
              window, waves);
   if (keys->max_seq_len == 0) return FC_OK;
@@ -403,16 +508,31 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
   const float c = scale * 1.4426950408889634f;
   const float out_mul = out_scale / (float)kernel_size;
   const char* q = (const char*)queries;
-#define SK_LAUNCH(DT, NWV)                                                                                   \
-  hipLaunchKernelGGL((snapkv_kernel<DT, NWV>), grid, dim3(NWV * 64), 0, st, kv, q, num_q_heads, window,      \
-                     kernel_size, causal_window, c, out_mul, scores, score_stride, row_max)
-#define SK_DISPATCH(DT)                 \
-  if (waves <= 1) SK_LAUNCH(DT, 1);     \
-  else if (waves <= 2) SK_LAUNCH(DT, 2);\
-  else if (waves <= 4) SK_LAUNCH(DT, 4);\
-  else if (waves <= 8) SK_LAUNCH(DT, 8);\
-  else SK_LAUNCH(DT, 16)
+#define SK_LAUNCH(DT, NWV, FA)                                                                                  \
+  do {                                                                                                       \
+    static bool attr_done = false;                                                                           \
+    if (!attr_done) {                                                                                        \
+      hipFuncSetAttribute((const void*)snapkv_kernel<DT, NWV, FA>,                                           \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, SkCfg<NWV>::LDS);                      \
+      attr_done = true;                                                                                      \
+    }                                                                                                        \
+    hipLaunchKernelGGL((snapkv_kernel<DT, NWV, FA>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,       \
+                       num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,    \
+                       row_max);                                                                             \
+  } while (0)
+#define SK_DISPATCH2(DT, FA)                 \
+  if (waves <= 1) SK_LAUNCH(DT, 1, FA);      \
+  else if (waves <= 2) SK_LAUNCH(DT, 2, FA); \
+  else if (waves <= 4) SK_LAUNCH(DT, 4, FA); \
+  else if (waves <= 8) SK_LAUNCH(DT, 8, FA); \
+  else SK_LAUNCH(DT, 16, FA)
+#define SK_DISPATCH(DT) \
+  if (fast) { SK_DISPATCH2(DT, true); } else { SK_DISPATCH2(DT, false); }
+  // a key tile lies inside one page (whose table row fits the LDS copy), or the view is dense
+  const bool fast = !keys->block_tables ||
+                    (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL);
   if (keys->dtype == FC_BF16) { SK_DISPATCH(FC_BF16); } else { SK_DISPATCH(FC_F16); }
+#undef SK_DISPATCH2
 #undef SK_DISPATCH
 #undef SK_LAUNCH
   FC_CHECK_LAUNCH(who);
