@@ -1,0 +1,113 @@
+// Symmetric per-row quantisation of KV rows to int8 storage (4- or 8-bit range) and back.
+//
+// One wavefront per row of `d` elements.  The arithmetic follows what a tensor library does on a
+// tensor of the row's dtype, step by step: every intermediate (row maximum, scale, quotient) is
+// computed in fp32 and rounded to the storage dtype before the next step, so that the integers
+// and scales are bit-identical to the eager expression
+//   scale = clamp(max|x| / qmax, min=1e-8);  q = clamp(round(x / scale), -qmax-1, qmax).
+#include "fc_common.h"
+
+template <int DTYPE>
+__device__ __forceinline__ float qz_load(const char* p, long long i) {
+  if constexpr (DTYPE == FC_F32) return reinterpret_cast<const float*>(p)[i];
+  const unsigned short r = reinterpret_cast<const unsigned short*>(p)[i];
+  return DTYPE == FC_BF16 ? fc_bf16_to_float(r) : fc_half_to_float(r);
+}
+template <int DTYPE>
+__device__ __forceinline__ float qz_round(float v) {   // round to the storage dtype, back to fp32
+  if constexpr (DTYPE == FC_F32) return v;
+  return DTYPE == FC_BF16 ? fc_bf16_to_float(fc_float_to_bf16(v)) : fc_half_to_float(fc_float_to_half(v));
+}
+template <int DTYPE>
+__device__ __forceinline__ void qz_store(char* p, long long i, float v) {
+  if constexpr (DTYPE == FC_F32) reinterpret_cast<float*>(p)[i] = v;
+  else reinterpret_cast<unsigned short*>(p)[i] = DTYPE == FC_BF16 ? fc_float_to_bf16(v) : fc_float_to_half(v);
+}
+
+template <int DTYPE>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const char* __restrict__ x, long long rows, int d,
+                                                            float qmax, signed char* __restrict__ q,
+                                                            char* __restrict__ scale) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows) return;
+  const long long base = r * d;
+  float mx = 0.f;
+  bool has_nan = false;
+  for (int j = lane; j < d; j += 64) {
+    const float v = qz_load<DTYPE>(x, base + j);
+    has_nan |= v != v;
+    mx = fmaxf(mx, fabsf(v));
+  }
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mx = __builtin_nanf("");   // a NaN in the row makes the maximum NaN
+  // scale = max / qmax, rounded; clamp(min=1e-8) in fp32, rounded again (1e-8 underflows to 0 in fp16)
+  float sc = qz_round<DTYPE>(mx / qmax);
+  sc = qz_round<DTYPE>(sc != sc ? sc : fmaxf(sc, 1e-8f));
+  if (lane == 0) qz_store<DTYPE>(scale, r, sc);
+  for (int j = lane; j < d; j += 64) {
+    const float v = qz_load<DTYPE>(x, base + j);
+    float t = qz_round<DTYPE>(v / sc);
+    t = rintf(t);                                   // round half to even
+    t = fminf(fmaxf(t, -qmax - 1.f), qmax);         // NaN falls through fmaxf/fminf to the bound
+    q[base + j] = (t != t) ? (signed char)0 : (signed char)(int)t;
+  }
+}
+
+// out = float(q) * scale, rounded to the output dtype.  SDT = dtype of scale, ODT = dtype of out.
+template <int SDT, int ODT>
+__global__ __launch_bounds__(256) void dequantize_rows_kernel(const signed char* __restrict__ q,
+                                                              const char* __restrict__ scale, long long rows, int d,
+                                                              char* __restrict__ out) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows) return;
+  const float sc = qz_load<SDT>(scale, r);
+  const long long base = r * d;
+  for (int j = lane; j < d; j += 64) qz_store<ODT>(out, base + j, (float)q[base + j] * sc);
+}
+
+extern "C" int fc_quantize_rows(const void* x, int64_t rows, int32_t d, int32_t dtype, int32_t bits, int8_t* q,
+                                void* scale, void* stream) {
+  const char* who = "fc_quantize_rows";
+  FC_REQUIRE(x && q && scale, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(rows >= 0 && d > 0, FC_EINVAL, "%s: bad sizes rows=%lld d=%d", who, (long long)rows, d);
+  FC_REQUIRE(bits >= 2 && bits <= 8, FC_EINVAL, "%s: bits must be in [2, 8] (got %d)", who, bits);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (rows == 0) return FC_OK;
+  const long long blocks = (rows + 3) / 4;
+  FC_REQUIRE(blocks <= 2147483647LL, FC_EUNSUPPORTED, "%s: too many rows", who);
+  const float qmax = (float)((1 << (bits - 1)) - 1);
+  hipStream_t st = (hipStream_t)stream;
+#define QZ(DT) hipLaunchKernelGGL((quantize_rows_kernel<DT>), dim3((unsigned)blocks), dim3(256), 0, st, (const char*)x, \
+                                  (long long)rows, d, qmax, (signed char*)q, (char*)scale)
+  if (dtype == FC_F32) QZ(FC_F32); else if (dtype == FC_F16) QZ(FC_F16); else QZ(FC_BF16);
+#undef QZ
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_dequantize_rows(const int8_t* q, const void* scale, int64_t rows, int32_t d, int32_t scale_dtype,
+                                  int32_t out_dtype, void* out, void* stream) {
+  const char* who = "fc_dequantize_rows";
+  FC_REQUIRE(q && scale && out, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(rows >= 0 && d > 0, FC_EINVAL, "%s: bad sizes rows=%lld d=%d", who, (long long)rows, d);
+  if (rows == 0) return FC_OK;
+  const long long blocks = (rows + 3) / 4;
+  FC_REQUIRE(blocks <= 2147483647LL, FC_EUNSUPPORTED, "%s: too many rows", who);
+  hipStream_t st = (hipStream_t)stream;
+#define DQ(S, O) hipLaunchKernelGGL((dequantize_rows_kernel<S, O>), dim3((unsigned)blocks), dim3(256), 0, st,        \
+                                    (const signed char*)q, (const char*)scale, (long long)rows, d, (char*)out)
+  // the output dtype is the promotion of the two: equal dtypes, or fp32 when either side is fp32
+  if (scale_dtype == out_dtype) {
+    if (out_dtype == FC_F32) DQ(FC_F32, FC_F32);
+    else if (out_dtype == FC_F16) DQ(FC_F16, FC_F16);
+    else if (out_dtype == FC_BF16) DQ(FC_BF16, FC_BF16);
+    else { fc_set_error("%s: dtype %d", who, out_dtype); return FC_EUNSUPPORTED; }
+  } else if (out_dtype == FC_F32 && scale_dtype == FC_F16) DQ(FC_F16, FC_F32);
+  else if (out_dtype == FC_F32 && scale_dtype == FC_BF16) DQ(FC_BF16, FC_F32);
+  else { fc_set_error("%s: scale dtype %d with output dtype %d", who, scale_dtype, out_dtype); return FC_EUNSUPPORTED; }
+#undef DQ
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}

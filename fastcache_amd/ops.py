@@ -162,6 +162,63 @@ def ccm_mlp(src: FcKvView, dst: FcKvView, weights: Tuple[torch.Tensor, ...], cf:
                            current_stream()), "fc_ccm_mlp")
 
 
+def quantize_rows(x: torch.Tensor, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row (last dimension) symmetric quantisation: ``(q int8 like x, scale x.dtype [..., 1])``."""
+    _lib.require_gpu(x, "x")
+    if x.dim() < 1 or x.numel() == 0:
+        raise FastcacheError("quantize_rows: empty input")
+    xc = x.contiguous()
+    d = xc.shape[-1]
+    rows = xc.numel() // d
+    q = torch.empty(xc.shape, dtype=torch.int8, device=x.device)
+    scale = torch.empty(xc.shape[:-1] + (1,), dtype=x.dtype, device=x.device)
+    check(fn("fc_quantize_rows")(xc.data_ptr(), rows, d, _lib.dtype_code(x.dtype), bits, q.data_ptr(),
+                                 scale.data_ptr(), current_stream()), "fc_quantize_rows")
+    return q, scale
+
+
+def dequantize_rows(q: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """``q.to(dtype) * scale`` with the dtype promotion of that expression."""
+    _lib.require_gpu(q, "q")
+    _lib.require_gpu(scale, "scale")
+    if q.dtype != torch.int8:
+        raise FastcacheError(f"dequantize_rows: int8 codes expected, got {q.dtype}")
+    d = q.shape[-1]
+    rows = q.numel() // d
+    if scale.numel() != rows:
+        raise FastcacheError("dequantize_rows: one scale per row expected")
+    out_dtype = torch.promote_types(dtype, scale.dtype)
+    qc, sc = q.contiguous(), scale.contiguous()
+    out = torch.empty(qc.shape, dtype=out_dtype, device=q.device)
+    check(fn("fc_dequantize_rows")(qc.data_ptr(), sc.data_ptr(), rows, d, _lib.dtype_code(sc.dtype),
+                                   _lib.dtype_code(out_dtype), out.data_ptr(), current_stream()), "fc_dequantize_rows")
+    return out
+
+
+def linear_act(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], apply_relu: bool) -> torch.Tensor:
+    """``act(x @ weight.T + bias)`` for ``x [M, K]`` (unit stride along K) and ``weight [N, K]`` contiguous,
+    fp16/bf16, fp32 accumulation, rounded once to the input dtype."""
+    _lib.require_gpu(x, "x")
+    _lib.require_gpu(weight, "weight")
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise FastcacheError(f"linear_act: x {tuple(x.shape)} and weight {tuple(weight.shape)} do not match")
+    if x.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != x.dtype:
+        raise FastcacheError(f"linear_act: fp16/bf16 operands of one dtype expected, got {x.dtype} and {weight.dtype}")
+    if x.stride(1) != 1 or not weight.is_contiguous():
+        raise FastcacheError("linear_act: x needs unit stride along K and weight must be contiguous [N, K]")
+    if bias is not None:
+        _lib.require_gpu(bias, "bias")
+        if bias.dtype != x.dtype or tuple(bias.shape) != (weight.shape[0],) or not bias.is_contiguous():
+            raise FastcacheError("linear_act: bias must be contiguous [N] in the input dtype")
+    M, K = x.shape
+    N = weight.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    check(fn("fc_linear_act")(x.data_ptr(), x.stride(0) if M > 1 else K, weight.data_ptr(), _lib.ptr(bias),
+                              y.data_ptr(), N, M, N, K, _lib.dtype_code(x.dtype), int(bool(apply_relu)),
+                              current_stream()), "fc_linear_act")
+    return y
+
+
 # ---------------------------------------------------------------------------------------------
 # decode
 # ---------------------------------------------------------------------------------------------

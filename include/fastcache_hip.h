@@ -175,6 +175,31 @@ int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weight
                int32_t cf, int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream);
 
 /*
+ * One Linear layer on dense row-major matrices: y[m][n] = act(x[m][k] * weight^T + bias), weight
+ * in nn.Linear layout [n][k], fp16 or bf16 throughout, fp32 accumulation, one rounding to the
+ * storage dtype.  bias may be NULL; apply_relu != 0 clamps at zero.  k must be a multiple of 16,
+ * n of 32, ldx (row stride of x in elements) of 8; x and weight 16-byte aligned.
+ * Replaces fused_linear_relu_dropout in inference mode (nanovllm/kernels/fused_compress.py:21-178)
+ * and the generated per-layer kernel mlp_layer_kernel (nanovllm/autocompress/kernels.py:177-222).
+ */
+int fc_linear_act(const void* x, int64_t ldx, const void* weight, const void* bias, void* y,
+                  int64_t ldy, int64_t m, int32_t n, int32_t k, int32_t dtype, int32_t apply_relu,
+                  void* stream);
+
+/*
+ * Symmetric per-row quantisation: for each of `rows` rows of `d` elements,
+ *   scale = clamp(max|x| / qmax, min=1e-8), q = clamp(round_half_even(x / scale), -qmax-1, qmax),
+ * qmax = 2^(bits-1) - 1, q stored as int8 (also for bits = 4), scale in the dtype of x; every
+ * intermediate is rounded to that dtype as an eager tensor expression would.  And the inverse,
+ * out = q * scale rounded to out_dtype (= scale_dtype, or fp32 for an fp16/bf16 scale).
+ * Replaces the quantize / dequantize pair of nanovllm/autocompress/kernels.py:387-421.
+ */
+int fc_quantize_rows(const void* x, int64_t rows, int32_t d, int32_t dtype, int32_t bits,
+                     int8_t* q, void* scale, void* stream);
+int fc_dequantize_rows(const int8_t* q, const void* scale, int64_t rows, int32_t d,
+                       int32_t scale_dtype, int32_t out_dtype, void* out, void* stream);
+
+/*
  * Plain ordered token copy src[seg_start + i] -> dst[dst_start + i], i < count, per
  * (layer, b, head); the pass-through branch of compress_layer when seg_len/cf < min_seq_len
  * (module_ccm_v11.py:674-675).  dst may alias src when dst_start <= seg_start.

@@ -1,0 +1,65 @@
+"""Oracle (test infrastructure): the single-layer fused Linear, the bias-free generated MLP, the
+sparse gather and the per-row quantiser of the reference's kernel factories.
+
+Restates ``fused_linear_relu_dropout`` in inference mode (nanovllm/kernels/fused_compress.py:21-178),
+``FusedCompressor.compress_layer_fused`` (:307-377), and the eager variants of
+``nanovllm/autocompress/kernels.py``: ``mlp_compress`` (:268-288), ``sparse_gather`` (:348-353),
+``quantize`` / ``dequantize`` (:387-421).
+"""
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+
+def linear_act(x: torch.Tensor, weight_kn: torch.Tensor, bias, apply_relu: bool) -> torch.Tensor:
+    """``act(x @ W + b)`` with ``W [K, N]``: operands in the storage dtype, fp32 accumulation, bias and
+    ReLU applied on the fp32 accumulator, one rounding to the storage dtype (the Triton kernel's
+    ``acc + b`` -> ``maximum`` -> ``tl.store(acc.to(dtype))``, fused_compress.py:93-118)."""
+    acc = x.float() @ weight_kn.float()
+    if bias is not None:
+        acc = acc + bias.float()[None, :]
+    if apply_relu:
+        acc = torch.clamp_min(acc, 0.0)
+    return acc.to(x.dtype)
+
+
+def mlp_nobias(X: torch.Tensor, W1: torch.Tensor, W2: torch.Tensor, W3: torch.Tensor) -> torch.Tensor:
+    """kernels.py:268-288: ``relu(X @ W1)``, ``relu(. @ W2)``, ``. @ W3`` with every product rounded to the dtype of X."""
+    y = linear_act(X, W1, None, True)
+    y = linear_act(y, W2, None, True)
+    return linear_act(y, W3, None, False)
+
+
+def fused_compress_layer(k: torch.Tensor, w, cf: int) -> torch.Tensor:
+    """fused_compress.py:307-377 for one tensor ``[B, H, S, D]``; ``w = (w1 [cf*D, D], b1, w2, b2, w3, b3)``."""
+    B, H, S, D = k.shape
+    c = S // cf
+    if c < 1:
+        return k
+    flat = k[:, :, :c * cf, :].reshape(B * H * c, cf * D)
+    y = linear_act(flat, w[0], w[1], True)
+    y = linear_act(y, w[2], w[3], True)
+    y = linear_act(y, w[4], w[5], False).reshape(B, H, c, D)
+    return torch.cat([y, k[:, :, c * cf:, :]], dim=2) if S > c * cf else y
+
+
+def sparse_gather(X: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    return X[indices.long()]
+
+
+def quantize(X: torch.Tensor, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """kernels.py:399-416, the same tensor expression evaluated by torch on the CPU."""
+    x_max = X.abs().max(dim=-1, keepdim=True).values
+    scale = x_max / (2 ** (bits - 1) - 1)
+    scale = scale.clamp(min=1e-8)
+    x_quant = (X / scale).round().clamp(-(2 ** (bits - 1)), 2 ** (bits - 1) - 1)
+    return x_quant.to(torch.int8), scale
+
+
+def dequantize(X_quant: torch.Tensor, scale: torch.Tensor, dtype=None) -> torch.Tensor:
+    """kernels.py:418-421."""
+    if dtype is None:
+        dtype = torch.float16
+    return X_quant.to(dtype) * scale

@@ -312,3 +312,57 @@ def test_decode_slot_rule():
     k = torch.zeros(2, 4, 1, 2)
     oattn.store_kv(k, k.clone(), torch.ones(1, 1, 2), torch.ones(1, 1, 2), torch.tensor([5]))
     assert k.view(8, 1, 2)[5].sum() == 2 and k.sum() == 2
+
+
+def test_linear_act_float64_and_single_rounding():
+    """oracle.autocompress.linear_act: float64 loops; bias and ReLU act on the unrounded accumulator."""
+    from oracle import autocompress as oa
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(7, 32, generator=g).half()
+    w = (torch.randn(32, 16, generator=g) * 0.3).half()
+    b = torch.randn(16, generator=g).half()
+    ref = np.zeros((7, 16))
+    for i in range(7):
+        for j in range(16):
+            acc = sum(float(x[i, t]) * float(w[t, j]) for t in range(32)) + float(b[j])
+            ref[i, j] = max(acc, 0.0)
+    got = oa.linear_act(x, w, b, True)
+    assert got.dtype == torch.float16
+    assert np.array_equal(got.numpy(), ref.astype(np.float32).astype(np.float16))
+    # one rounding only: an accumulator of 0.3 ulp below a half-way point plus the bias must not round twice
+    x1 = torch.tensor([[1.0, 2.0 ** -11]], dtype=torch.float16)
+    w1 = torch.tensor([[1.0], [1.0]], dtype=torch.float16)
+    b1 = torch.tensor([2.0 ** -12], dtype=torch.float16)
+    # exact sum 1 + 2^-11 + 2^-12 rounds up to 1 + 2^-10; rounding x@w first (to 1.0, ties-to-even) would give 1.0
+    assert float(oa.linear_act(x1, w1, b1, False)[0, 0]) == 1.0 + 2.0 ** -10
+    # the bias-free chain rounds after every product
+    W1, W2, W3 = (torch.randn(32, 16, generator=g) * 0.3).half(), (torch.randn(16, 16, generator=g) * 0.3).half(), \
+        (torch.randn(16, 16, generator=g) * 0.3).half()
+    y1 = torch.clamp_min(x.double() @ W1.double(), 0).half()
+    y2 = torch.clamp_min(y1.double() @ W2.double(), 0).half()
+    y3 = (y2.double() @ W3.double()).half()
+    assert torch.equal(oa.mlp_nobias(x, W1, W2, W3), y3)
+
+
+def test_quantize_numpy_float16_steps_and_hand_rows():
+    """oracle.autocompress.quantize / dequantize against step-by-step numpy float16 arithmetic and hand-worked rows."""
+    from oracle import autocompress as oa
+    g = torch.Generator().manual_seed(9)
+    X = (torch.randn(6, 40, generator=g) * 3).half()
+    for bits in (4, 8):
+        qmax = 2 ** (bits - 1) - 1
+        q, sc = oa.quantize(X, bits)
+        xn = X.numpy()
+        mx = np.abs(xn).max(axis=-1, keepdims=True)                              # float16
+        scn = (mx.astype(np.float32) / np.float32(qmax)).astype(np.float16)      # one rounding per step
+        quo = (xn.astype(np.float32) / scn.astype(np.float32)).astype(np.float16)
+        qn = np.clip(np.rint(quo.astype(np.float32)), -qmax - 1, qmax).astype(np.int8)
+        assert np.array_equal(sc.numpy(), scn) and np.array_equal(q.numpy(), qn)
+        deq = oa.dequantize(q, sc, torch.float16)
+        assert np.array_equal(deq.numpy(), (qn.astype(np.float16).astype(np.float32) * scn.astype(np.float32)).astype(np.float16))
+    # by hand, fp32: row [7, -3.5, 0.5] at 4 bits: scale 1, codes [7, -4 (round half to even of -3.5), 0 (0.5 -> 0)]
+    q, sc = oa.quantize(torch.tensor([[7.0, -3.5, 0.5]]), 4)
+    assert sc.item() == 1.0 and q.tolist() == [[7, -4, 0]]
+    # range: the most negative code -qmax-1 is reachable only through clamping; 8 bits keeps [-128, 127]
+    q, sc = oa.quantize(torch.tensor([[127.0, -127.0, 63.5]]), 8)
+    assert sc.item() == 1.0 and q.tolist() == [[127, -127, 64]]
