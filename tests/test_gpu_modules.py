@@ -320,3 +320,67 @@ def test_background_compression_event_protocol(dev):
     assert PagedKVRunner(L, H, 128, 2, dtype, dev).start_background_compression(seqs) is None
     runner.clear_compressed_lens([seqs[0].seq_id])
     assert seqs[0].seq_id not in runner._compressed_lens and seqs[1].seq_id in runner._compressed_lens
+
+
+def test_async_compression_manager_states_and_effective_len(dev):
+    """Per-sequence states, events and the effective KV length of the asynchronous manager; the pages end up
+    identical to the synchronous path's."""
+    from fastcache_amd.engine.async_compress import AsyncCompressionManager, CompressionState
+    dtype, L, H, S = torch.float16, 2, 2, 700
+    case = synth.make_paged_case(seed=8, num_layers=L, batch=2, num_kv_heads=H, seq_lens=[S, S], dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0)
+    mk = lambda: PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0,
+                               compressor=KVPressCompressor("knorm", 0.5))
+    runner, sync_runner = mk(), mk()
+    bm = BlockManager(8, 256)
+    seqs = [Sequence(list(range(i * 1000, i * 1000 + S))) for i in range(2)]
+    for s in seqs:
+        bm.allocate(s)
+    _fill_pool_from_case(runner, case, seqs)
+    sync_runner.kv_cache.copy_(runner.kv_cache)
+    sync_runner.compress_kv_cache_batch(seqs)
+
+    mgr = AsyncCompressionManager(runner)
+    assert mgr.get_effective_kv_len(seqs[0]) == S and not mgr.is_compression_complete(seqs[0].seq_id)
+    mgr.start_async_compression(seqs, image_len=0)
+    mgr.wait_for_compression(seqs[0].seq_id)
+    mgr.wait_all_compressions()
+    for s in seqs:
+        assert mgr.seq_states[s.seq_id] == CompressionState.COMPLETED and mgr.is_compression_complete(s.seq_id)
+        assert mgr.get_effective_kv_len(s) == 350 == runner._compressed_lens[s.seq_id]
+        assert mgr.seq_original_lens[s.seq_id] == S
+    assert torch.equal(runner.kv_cache, sync_runner.kv_cache)
+    mgr.cleanup_seq(seqs[0].seq_id)
+    assert seqs[0].seq_id not in mgr.seq_states and mgr.get_effective_kv_len(seqs[0]) == S
+    # a failing compressor leaves the sequence uncompressed instead of raising (the reference's fallback)
+    bad = PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0,
+                        compressor=lambda kv, it_len=None: (_ for _ in ()).throw(RuntimeError("boom")))
+    bmgr = AsyncCompressionManager(bad)
+    bmgr.start_async_compression(seqs[:1], image_len=0)
+    bmgr.wait_all_compressions()
+    assert bmgr.seq_states[seqs[0].seq_id] == CompressionState.NONE and bmgr.get_effective_kv_len(seqs[0]) == S
+    assert AsyncCompressionManager(PagedKVRunner(L, H, 128, 2, dtype, dev)).start_async_compression(seqs) is None
+
+
+def test_pipeline_async_compressor_round_robin(dev):
+    from fastcache_amd.engine.async_compress import CompressionState, PipelineAsyncCompressor
+    dtype, L = torch.float16, 2
+    comp = KVPressCompressor("streaming_llm", 0.5)
+    pipe = PipelineAsyncCompressor(comp, num_streams=2)
+    written = {}
+    events = []
+    kvs = [to_dev(rand_kv(L, 1, 2, 300 + 20 * i, dtype, seed=i), dev) for i in range(3)]
+    for i, kv in enumerate(kvs):
+        events.append(pipe.submit_compression(i, kv, [i], kv[0][0].shape[2], [0, kv[0][0].shape[2]],
+                                              lambda out, table, i=i: written.__setitem__(i, (out, table))))
+    assert pipe.current_stream_idx == 1            # three submissions over two streams
+    for i, ev in enumerate(events):
+        pipe.wait_compression(i)
+        assert ev.query() and pipe.is_compression_ready(i)
+        assert pipe.seq_states[i] == CompressionState.COMPLETED
+        n = (300 + 20 * i) // 2
+        assert pipe.get_compressed_len(i) == n and written[i][1] == [i]
+        ref = comp(kvs[i], it_len=[0, 300 + 20 * i])
+        assert all(torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) for a, b in zip(written[i][0], ref))
+    pipe.cleanup(0)
+    assert pipe.get_compressed_len(0) is None and not pipe.is_compression_ready(0)
