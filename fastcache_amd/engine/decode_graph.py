@@ -13,11 +13,12 @@ token less: it writes the new row at ``len`` but passes ``len`` as the attended 
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
 from .. import _lib, ops
+from ..utils.context import get_context, reset_context, set_context
 
 
 class DecodeGraph:
@@ -63,3 +64,86 @@ class DecodeGraph:
             raise RuntimeError("capture() first")
         self.graph.replay()
         return self.out
+
+
+class BucketedDecodeGraphs:
+    """One captured decode step per batch bucket, replayed with host-patched static buffers: the
+    protocol of ``capture_cudagraph`` / ``reset_graph_vars`` / the decode branch of ``run_model``
+    (nanovllm/engine/llava_model_runner.py:1109-1169, 914-921, 697-710), with the attention layers
+    standing in for the model.
+
+    ``layers`` are ``fastcache_amd.layers.Attention`` modules whose ``k_cache`` / ``v_cache`` are set.
+    A step takes q ``[L, bs, Hq*D]`` and k, v ``[L, bs, Hkv*D]`` and the decode context
+    (``set_context(False, slot_mapping=, context_lens=, block_tables=)``) and returns ``[L, bs, Hq*D]``.
+    Padded rows of a bucket get ``context_len = 0`` and ``slot = -1`` (skipped by the append kernel); the
+    reference zeroes the slot instead, which makes every padded row overwrite slot 0 of block 0.
+    """
+
+    def __init__(self, layers: Sequence, max_bs: int, max_num_blocks: int, dtype: torch.dtype, device):
+        self.layers = list(layers)
+        self.max_bs, self.max_num_blocks = min(max_bs, 256), max_num_blocks
+        self.dtype, self.device = dtype, torch.device(device)
+        self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
+        self.graph_bs: List[int] = []
+        self.graph_vars: Dict[str, torch.Tensor] = {}
+        self.graph_pool = None
+
+    def _model(self, q, k, v, out):
+        for i, layer in enumerate(self.layers):
+            out[i] = layer(q[i], k[i], v[i])
+
+    @torch.inference_mode()
+    def capture_cudagraph(self):
+        a = self.layers[0]
+        L, bsz, dev = len(self.layers), self.max_bs, self.device
+        block_size = a.k_cache.shape[1]
+        slot_mapping = torch.full((bsz,), -1, dtype=torch.int32, device=dev)
+        context_lens = torch.zeros(bsz, dtype=torch.int32, device=dev)
+        block_tables = torch.zeros(bsz, self.max_num_blocks, dtype=torch.int32, device=dev)
+        q = torch.zeros(L, bsz, a.num_heads * a.head_dim, dtype=self.dtype, device=dev)
+        k = torch.zeros(L, bsz, a.num_kv_heads * a.head_dim, dtype=self.dtype, device=dev)
+        v = torch.zeros_like(k)
+        outputs = torch.zeros_like(q)
+        workspace = ops.decode_attn_workspace(bsz, a.num_heads, self.max_num_blocks * block_size, dev)
+        for layer in self.layers:
+            layer.workspace = workspace
+        self.graph_bs = [b for b in [1, 2, 4, 8] + list(range(16, bsz + 1, 16)) if b <= bsz]
+        if self.graph_bs[-1] != bsz:
+            self.graph_bs.append(bsz)
+        for bs in reversed(self.graph_bs):
+            graph = torch.cuda.CUDAGraph()
+            set_context(False, slot_mapping=slot_mapping[:bs], context_lens=context_lens[:bs],
+                        block_tables=block_tables[:bs])
+            self._model(q[:, :bs], k[:, :bs], v[:, :bs], outputs[:, :bs])       # warm-up outside the graph
+            with torch.cuda.graph(graph, self.graph_pool):
+                self._model(q[:, :bs], k[:, :bs], v[:, :bs], outputs[:, :bs])
+            if self.graph_pool is None:
+                self.graph_pool = graph.pool()
+            self.graphs[bs] = graph
+            torch.cuda.synchronize()
+            reset_context()
+        self.graph_vars = dict(slot_mapping=slot_mapping, context_lens=context_lens, block_tables=block_tables,
+                               q=q, k=k, v=v, outputs=outputs)
+
+    def reset_graph_vars(self):
+        gv = self.graph_vars
+        gv["slot_mapping"].fill_(-1)
+        gv["context_lens"].zero_()
+        gv["block_tables"].zero_()
+
+    @torch.inference_mode()
+    def run(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        """Replay the graph of the smallest bucket that holds the batch, with the current decode context."""
+        bs = q.shape[1]
+        context = get_context()
+        self.reset_graph_vars()
+        graph = self.graphs[next(x for x in self.graph_bs if x >= bs)]
+        gv = self.graph_vars
+        gv["q"][:, :bs] = q
+        gv["k"][:, :bs] = k
+        gv["v"][:, :bs] = v
+        gv["slot_mapping"][:bs] = context.slot_mapping
+        gv["context_lens"][:bs] = context.context_lens
+        gv["block_tables"][:bs, :context.block_tables.size(1)] = context.block_tables
+        graph.replay()
+        return gv["outputs"][:, :bs]

@@ -66,6 +66,7 @@ class Attention(nn.Module):
         super().__init__()
         self.num_heads, self.head_dim, self.scale, self.num_kv_heads = num_heads, head_dim, scale, num_kv_heads
         self.k_cache = self.v_cache = torch.tensor([])
+        self.workspace: Optional[torch.Tensor] = None   # set by a graph runner that owns the scratch memory
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
         q = q.view(-1, self.num_heads, self.head_dim)
@@ -75,5 +76,6 @@ class Attention(nn.Module):
         store_kvcache(k, v, self.k_cache, self.v_cache, ctx.slot_mapping)
         if ctx.is_prefill:
             raise NotImplementedError("prefill attention is outside the KV-cache compression path built here")
-        o = decode_attention(q.unsqueeze(1), self.k_cache, self.v_cache, ctx.context_lens, ctx.block_tables, self.scale)
+        o = decode_attention(q.unsqueeze(1), self.k_cache, self.v_cache, ctx.context_lens, ctx.block_tables, self.scale,
+                             workspace=self.workspace)
         return o.view(-1, self.num_heads * self.head_dim)

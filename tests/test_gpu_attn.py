@@ -147,3 +147,55 @@ def test_multi_step_decode_graph_matches_eager_and_oracle(dev):
         assert lens2.tolist() == [n + T for n in lens]
         _ = (pool2.float().sum()).item()          # unrelated eager work between replays
     assert torch.equal(pool2, pool)
+
+
+def test_bucketed_decode_graphs_match_eager_layers(dev):
+    """One captured step per batch bucket, static buffers patched per step: every replay equals the eager
+    Attention layers bit for bit (outputs and pool), for batches that fill a bucket exactly and that do not."""
+    from fastcache_amd.engine.decode_graph import BucketedDecodeGraphs
+    from fastcache_amd.layers import Attention
+    from fastcache_amd.utils.context import reset_context, set_context
+    dtype, L, Hq, Hkv, D, steps = torch.float16, 2, 8, 2, 128, 3
+    max_bs, scale = 40, 128 ** -0.5
+    all_lens = [100 + 37 * i for i in range(21)]
+    all_lens[4] = 255                                            # crosses a block boundary during the steps
+    case = synth.make_paged_case(seed=21, num_layers=L, batch=21, num_kv_heads=Hkv, seq_lens=all_lens, dtype=dtype,
+                                 reserve_tokens=steps + 1)
+    tables_all = case.table_tensor("cpu")
+
+    def make_layers(pool):
+        layers = []
+        for l in range(L):
+            a = Attention(Hq, D, scale, Hkv)
+            a.k_cache, a.v_cache = pool[0, l], pool[1, l]
+            layers.append(a)
+        return layers
+
+    pool_g, pool_e = case.kv_cache.to(dev), case.kv_cache.to(dev)
+    graphs = BucketedDecodeGraphs(make_layers(pool_g), max_bs, tables_all.shape[1], dtype, dev)
+    graphs.capture_cudagraph()
+    assert graphs.graph_bs == [1, 2, 4, 8, 16, 32, 40]
+    pool_g.copy_(case.kv_cache)                                  # capture warm-ups wrote nothing (slots are -1)
+    eager_layers = make_layers(pool_e)
+    g = torch.Generator().manual_seed(6)
+    for bs in (3, 21, 16):
+        lens = list(all_lens[:bs])
+        tables = tables_all[:bs].to(dev)
+        for t in range(steps):
+            q = torch.randn(L, bs, Hq * D, generator=g).to(dtype).to(dev)
+            k = torch.randn(L, bs, Hkv * D, generator=g).to(dtype).to(dev)
+            v = torch.randn(L, bs, Hkv * D, generator=g).to(dtype).to(dev)
+            slots = torch.tensor([oattn.decode_slot(case.block_tables[b], lens[b]) for b in range(bs)],
+                                 dtype=torch.int32, device=dev)
+            lens = [n + 1 for n in lens]
+            ctx_lens = torch.tensor(lens, dtype=torch.int32, device=dev)
+            set_context(False, slot_mapping=slots, context_lens=ctx_lens, block_tables=tables)
+            out_g = graphs.run(q, k, v).clone()
+            out_e = torch.stack([eager_layers[l](q[l], k[l], v[l]) for l in range(L)])
+            reset_context()
+            torch.cuda.synchronize()
+            assert torch.equal(out_g, out_e), f"bs={bs} step={t}"
+            assert torch.equal(pool_g, pool_e)
+        # restore the prefixes for the next batch size
+        pool_g.copy_(case.kv_cache)
+        pool_e.copy_(case.kv_cache)
