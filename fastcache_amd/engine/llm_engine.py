@@ -1,0 +1,140 @@
+"""The engine loop around the compression hooks, and the lazy (threshold-triggered) compression policy.
+
+``CompressionEngine.step`` follows ``LlavaLLMEngine.step`` (nanovllm/engine/llava_engine.py:187-272):
+schedule, run the model, compress after prefill (synchronously, or on the side stream with the wait moved
+in front of the first decode of those sequences), release the freed blocks, post-process.  The model
+forward is not part of this build: ``model_step(seqs, is_prefill) -> token ids`` is supplied by the caller
+(a real model writing its KV through the runner's pool, or a synthetic stand-in).
+
+``LazyCompressionEngine`` follows nanovllm_fastapi_server.py:54-153: no compression after prefill; when the
+free blocks fall under a fraction of the pool, every running sequence not yet compressed is compressed
+in one batch and its tail blocks are released.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Tuple
+
+from .kv_runner import PagedKVRunner
+from .llm_hooks import free_compressed_blocks
+from .scheduler import LlavaScheduler
+from .sequence import Sequence, SequenceStatus
+
+
+@dataclass
+class SamplingParams:
+    temperature: float = 1.0
+    max_tokens: int = 64
+    ignore_eos: bool = False
+
+
+class CompressionEngine:
+    def __init__(self, scheduler: LlavaScheduler, model_runner: PagedKVRunner,
+                 model_step: Callable[[List[Sequence], bool], List[int]], enable_compression: bool = True,
+                 async_compression: bool = False):
+        self.scheduler = scheduler
+        self.model_runner = model_runner
+        self.model_step = model_step
+        self.enable_compression = enable_compression
+        self.async_compression = async_compression
+        self._pending_compression_events: Dict[int, object] = {}
+        self.total_compression_time = 0.0
+        self.total_freed_blocks = 0
+
+    def add_request(self, prompt: List[int], sampling_params: Optional[SamplingParams] = None) -> Sequence:
+        seq = Sequence(prompt, sampling_params or SamplingParams())
+        self.scheduler.add(seq)
+        return seq
+
+    def is_finished(self) -> bool:
+        return self.scheduler.is_finished()
+
+    def step(self, apply_compression: bool = False) -> Tuple[list, int]:
+        seqs, is_prefill = self.scheduler.schedule()
+        if not is_prefill and self.async_compression and self.enable_compression:
+            self._wait_pending_compressions(seqs)
+            self._free_compressed_blocks(seqs)
+        token_ids = self.model_step(seqs, is_prefill)
+        compress_now = apply_compression and is_prefill and self.enable_compression
+        if compress_now and not self.async_compression:
+            sec, _ = self.model_runner.compress_kv_cache_batch(seqs)
+            self.total_compression_time += sec
+            self._free_compressed_blocks(seqs)
+        if compress_now and self.async_compression:
+            self._start_pipeline_compression(seqs)
+        self.scheduler.postprocess(seqs, token_ids)
+        outputs = [(seq.seq_id, seq[seq.num_prompt_tokens:]) for seq in seqs if seq.status == SequenceStatus.FINISHED]
+        for seq_id, _ in outputs:
+            self.model_runner.clear_compressed_lens([seq_id])
+        num_tokens = sum(len(seq) for seq in seqs) if is_prefill else -len(seqs)
+        return outputs, num_tokens
+
+    def _start_pipeline_compression(self, seqs: List[Sequence]) -> None:
+        event = self.model_runner.start_background_compression(seqs)
+        if event is not None:
+            for seq in seqs:
+                self._pending_compression_events[seq.seq_id] = event
+
+    def _wait_pending_compressions(self, seqs: List[Sequence]) -> None:
+        for seq in seqs:
+            event = self._pending_compression_events.pop(seq.seq_id, None)
+            if event is not None:
+                event.synchronize()
+
+    def _free_compressed_blocks(self, seqs: List[Sequence]) -> None:
+        todo = [s for s in seqs if not s.is_compressed]      # a sequence is shortened once
+        self.total_freed_blocks += free_compressed_blocks(self.scheduler.block_manager, self.model_runner, todo)
+
+
+class LazyCompressionEngine:
+    def __init__(self, llm: CompressionEngine, compression_threshold: float = 0.3,
+                 compression_backend: str = "kvpress"):
+        self.llm = llm
+        self.compression_threshold = compression_threshold
+        self.compression_backend = compression_backend
+        self.total_blocks = len(llm.scheduler.block_manager.blocks)
+        self.threshold_blocks = int(self.total_blocks * compression_threshold)
+        self.uncompressed_seqs = set()
+        self.compression_count = 0
+        self.total_compression_time = 0.0
+
+    def add_request(self, prompt, sampling_params=None):
+        return self.llm.add_request(prompt, sampling_params)
+
+    def is_finished(self) -> bool:
+        return self.llm.is_finished()
+
+    def step(self):
+        free_blocks = len(self.llm.scheduler.block_manager.free_block_ids)
+        if free_blocks < self.threshold_blocks and self.uncompressed_seqs:
+            self._do_batch_compression()
+        outputs, num_tokens = self.llm.step(apply_compression=False)
+        if num_tokens > 0:
+            for seq in self.llm.scheduler.running:
+                if not seq.is_compressed:
+                    self.uncompressed_seqs.add(seq.seq_id)
+        for seq_id, _ in outputs:
+            self.uncompressed_seqs.discard(seq_id)
+        return outputs, num_tokens
+
+    def _do_batch_compression(self) -> None:
+        """One batched launch for every running sequence that still has its full cache.  A sequence that has
+        decoded since its prefill holds ``len(seq) - 1`` KV rows (the last token's row is written by the next
+        step); the reference compresses ``len(seq)`` rows there, one of them never written."""
+        seqs = [s for s in self.llm.scheduler.running if s.seq_id in self.uncompressed_seqs and not s.is_compressed]
+        if not seqs:
+            self.uncompressed_seqs.clear()
+            return
+        start = time.time()
+        self.llm.model_runner.compress_kv_cache_batch(seqs)
+        for seq in seqs:
+            self.llm._free_compressed_blocks([seq])
+            self.uncompressed_seqs.discard(seq.seq_id)
+        self.compression_count += 1
+        self.total_compression_time += time.time() - start
+
+    def get_stats(self) -> dict:
+        n = self.compression_count
+        return {"compression_count": n, "total_compression_time_ms": self.total_compression_time * 1000,
+                "avg_compression_time_ms": self.total_compression_time / n * 1000 if n > 0 else 0}

@@ -384,3 +384,55 @@ def test_pipeline_async_compressor_round_robin(dev):
         assert all(torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) for a, b in zip(written[i][0], ref))
     pipe.cleanup(0)
     assert pipe.get_compressed_len(0) is None and not pipe.is_compression_ready(0)
+
+
+def test_lazy_compression_engine_on_the_pool(dev):
+    """Threshold-triggered batch compression over a real pool: when the free blocks run out the three running
+    sequences are compressed in ONE batched pass, their pages equal the oracle's per-sequence loop, the freed
+    blocks admit the waiting request, and every block is back in the pool at the end."""
+    from fastcache_amd.engine.llm_engine import CompressionEngine, LazyCompressionEngine, SamplingParams
+    from fastcache_amd.engine.scheduler import LlavaScheduler
+    dtype, L, H, S = torch.float16, 2, 2, 600
+    case = synth.make_paged_case(seed=17, num_layers=L, batch=4, num_kv_heads=H, seq_lens=[S] * 4, dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0)
+    ratio = 1.0 - 1.0 / 3
+    runner = PagedKVRunner(L, H, 128, num_blocks=9, dtype=dtype, device=dev, image_token_len=0,
+                           compressor=KVPressCompressor("streaming_llm", ratio))
+    sched = LlavaScheduler(max_num_seqs=8, max_num_batched_tokens=600, eos=-1, num_kvcache_blocks=9)
+    order = {}
+
+    def model_step(seqs, is_prefill):
+        if is_prefill:                         # "prefill": the sequence's KV rows appear in its pages
+            for s in seqs:
+                b = order.setdefault(s.seq_id, len(order))
+                for i, blk in enumerate(s.block_table):
+                    runner.kv_cache[:, :, blk] = case.kv_cache[:, :, case.block_tables[b][i]].to(dev)
+        return [3] * len(seqs)
+
+    llm = CompressionEngine(sched, runner, model_step)
+    eng = LazyCompressionEngine(llm, compression_threshold=0.4)
+    seqs = [eng.add_request(list(range(i * 1000, i * 1000 + S)), SamplingParams(max_tokens=4, ignore_eos=True))
+            for i in range(4)]
+    for _ in range(3):                         # one prefill per step (600 batched tokens)
+        eng.step()
+    assert len(sched.block_manager.free_block_ids) == 0 and len(sched.waiting) == 1
+    tables_before = [list(s.block_table) for s in seqs[:3]]
+    ref_pool = runner.kv_cache.cpu()
+    lens = [len(s) for s in seqs[:3]]          # 601: the lazy path compresses len(seq) rows, like the reference
+    ref_lens, _, _ = opipe.compress_batch(
+        ref_pool, tables_before, lens,
+        lambda hf, i, n: [opress.adapter_compress_layer("streaming_llm", k, v, ratio) for k, v in hf])
+    eng.step()                                 # trigger: compress the three, then prefill the fourth
+    assert eng.compression_count == 1 and len(sched.running) == 4 and not sched.waiting
+    for s, c, tab in zip(seqs[:3], ref_lens.values(), tables_before):
+        assert s.is_compressed and len(s.block_table) == 1 and s.block_table == tab[:1]
+        assert s.kv_cache_len == c
+        got = runner.kv_cache[:, :, s.block_table[0], :c].cpu()
+        assert torch.equal(got, ref_pool[:, :, tab[0], :c])
+    steps = 0
+    while not eng.is_finished():
+        eng.step()
+        steps += 1
+        assert steps < 50
+    bm = sched.block_manager
+    assert len(bm.free_block_ids) == 9 and not bm.used_block_ids and llm.total_freed_blocks == 6

@@ -189,3 +189,96 @@ def test_hybrid_image_branch_raises_like_reference():
     with pytest.raises(TypeError):
         h._paged_segments(16, [8, 8])
     assert h._paged_segments(16, [0, 16]) == [("compress_tk", "compress_tv", 0, 16)]
+
+
+class _FakeRunner:
+    """Host-side stand-in for PagedKVRunner's bookkeeping (no device work): compression keeps len // cf rows."""
+
+    def __init__(self, cf=4, block_size=256):
+        self.cf, self.block_size = cf, block_size
+        self._compressed_lens, self._blocks_to_free = {}, {}
+        self.batches = []
+
+    def compress_kv_cache_batch(self, seqs, image_len=None):
+        self.batches.append([s.seq_id for s in seqs])
+        for s in seqs:
+            self._compressed_lens[s.seq_id] = len(s) // self.cf
+        return 0.0, float(self.cf)
+
+    def get_compressed_block_count(self, seq_id):
+        c = self._compressed_lens.get(seq_id)
+        return -1 if c is None else -(-c // self.block_size)
+
+    def clear_compressed_lens(self, seq_ids=None):
+        for i in (seq_ids or list(self._compressed_lens)):
+            self._compressed_lens.pop(i, None)
+
+
+def _drive(engine, max_steps=200):
+    peak, steps, done = 0, 0, {}
+    while not engine.is_finished():
+        outputs, _ = engine.step()
+        llm = getattr(engine, "llm", engine)
+        peak = max(peak, len(llm.scheduler.running) + len(outputs))
+        bm = llm.scheduler.block_manager
+        assert len(bm.free_block_ids) + len(bm.used_block_ids) == len(bm.blocks)
+        done.update(dict(outputs))
+        steps += 1
+        assert steps < max_steps
+    return peak, steps, done
+
+
+def test_scheduler_engine_and_lazy_compression_admit_more_requests():
+    """Freed pages turn into admitted requests: with threshold-triggered batch compression all five requests
+    run together, without it the pool holds three; every block returns to the pool at the end."""
+    from fastcache_amd.engine.llm_engine import CompressionEngine, LazyCompressionEngine, SamplingParams
+    from fastcache_amd.engine.scheduler import LlavaScheduler
+
+    def build(lazy):
+        sched = LlavaScheduler(max_num_seqs=8, max_num_batched_tokens=4096, eos=-1, num_kvcache_blocks=12)
+        runner = _FakeRunner(cf=4)
+        llm = CompressionEngine(sched, runner, lambda seqs, is_prefill: [7] * len(seqs))
+        eng = LazyCompressionEngine(llm, compression_threshold=0.3) if lazy else llm
+        for i in range(5):
+            eng.add_request(list(range(i * 5000, i * 5000 + 1000)), SamplingParams(max_tokens=6, ignore_eos=True))
+        return eng, llm, runner
+
+    eng, llm, runner = build(lazy=False)
+    peak, steps_plain, done = _drive(eng)
+    assert peak == 3 and len(done) == 5 and all(len(v) == 6 for v in done.values())
+    assert len(llm.scheduler.block_manager.free_block_ids) == 12 and not runner.batches
+
+    eng, llm, runner = build(lazy=True)
+    assert eng.threshold_blocks == 3
+    peak, steps_lazy, done = _drive(eng)
+    assert len(done) == 5 and all(len(v) == 6 for v in done.values())
+    assert peak == 5 and steps_lazy < steps_plain
+    # the first three prefills exhaust the pool (12 blocks), the next step compresses exactly those three in one batch
+    assert len(runner.batches[0]) == 3 and eng.get_stats()["compression_count"] == len(runner.batches) >= 1
+    assert llm.total_freed_blocks >= 9
+    assert len(llm.scheduler.block_manager.free_block_ids) == 12
+    assert not runner._compressed_lens                       # cleared as sequences finish
+
+
+def test_engine_sync_compression_after_prefill_and_preemption():
+    """apply_compression=True shortens every sequence right after its prefill (kv_cache_len, table, freed tail);
+    a sequence is shortened once; pre-emption puts a sequence back with its cache dropped."""
+    from fastcache_amd.engine.llm_engine import CompressionEngine, SamplingParams
+    from fastcache_amd.engine.scheduler import LlavaScheduler
+    from fastcache_amd.engine.sequence import SequenceStatus
+    sched = LlavaScheduler(max_num_seqs=4, max_num_batched_tokens=8192, eos=-1, num_kvcache_blocks=9)
+    runner = _FakeRunner(cf=4)
+    llm = CompressionEngine(sched, runner, lambda seqs, is_prefill: [1] * len(seqs))
+    a = llm.add_request(list(range(1024)), SamplingParams(max_tokens=3, ignore_eos=True))
+    b = llm.add_request(list(range(9000, 9000 + 1100)), SamplingParams(max_tokens=3, ignore_eos=True))
+    outputs, n = llm.step(apply_compression=True)             # prefill of both: 4 + 5 blocks
+    assert n == 1025 + 1101 and outputs == []                 # counted after the sampled token is appended
+    assert a.is_compressed and a.kv_cache_len == 256 + 1 and len(a.block_table) == 1   # 256 rows kept, +1 appended
+    assert b.kv_cache_len == 275 + 1 and len(b.block_table) == 2
+    assert len(sched.block_manager.free_block_ids) == 9 - 3
+    llm.step(apply_compression=True)                          # decode: a crosses into a new block (257 % 256 == 1)
+    assert len(a.block_table) == 2 and a.kv_cache_len == 258 and b.kv_cache_len == 277
+    # pre-emption drops the cache and the compressed length
+    sched.preempt(b)
+    sched.running.remove(b)
+    assert b.status == SequenceStatus.WAITING and not b.is_compressed and b.block_table == [] and sched.waiting[0] is b
