@@ -81,6 +81,21 @@ __device__ __forceinline__ void sk_wait_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// Sum over aligned groups of N consecutive lanes (N a power of two up to 16) with DPP adds in a
+// fixed order; every lane of a group ends up with the group's sum.
+template <int CTRL>
+__device__ __forceinline__ float sk_dpp_get(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int N>
+__device__ __forceinline__ float sk_group_sum(float v) {
+  if constexpr (N >= 2) v += sk_dpp_get<0xB1>(v);    // quad_perm [1,0,3,2]
+  if constexpr (N >= 4) v += sk_dpp_get<0x4E>(v);    // quad_perm [2,3,0,1]
+  if constexpr (N >= 8) v += sk_dpp_get<0x141>(v);   // row_half_mirror
+  if constexpr (N >= 16) v += sk_dpp_get<0x140>(v);  // row_mirror
+  return v;
+}
+
 template <int NW>
 struct SkCfg {
   static constexpr int ST = NW >= 8 ? 4 : 3;   // key tiles resident or in flight per workgroup
@@ -347,22 +362,26 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
 
   // ================= sweep 2: probabilities, per-key sums, moving average ======================
   // C[query][key], tiles in descending order.  Every wavefront leaves its per-key sums of a tile in
-  // vpart (four tiles deep); wave 0 folds them (fixed order) into vraw, a ring of four tiles, and
-  // writes the moving average of a tile once both neighbours are folded.
+  // vpart (four tiles deep); one iteration later the sums are folded (fixed order) into vraw, a ring
+  // of four tiles, each wavefront taking 64/NW keys; the moving average of a tile is written two
+  // iterations after its own fold, when both neighbours are in the ring.
   const int hw = ksz >> 1;
-  auto emit = [&](int s) {   // scored key s: zero-padded moving average over [s-hw, s+hw]
-    float acc = 0.f;
-    for (int j = -hw; j <= hw; ++j) {
-      const int x = s + j;
-      if (x >= 0 && x < SW) acc += vraw[(x / SK_KT) & 3][x % SK_KT];
-    }
-    out_row[s] = acc * out_mul;
+  // Every wavefront folds and emits 64/NW keys of a tile with NW lanes per key.
+  constexpr int KPW = SK_KT / NW;
+  const int fkey = wave * KPW + lane / NW, fp = lane % NW;
+  auto fold = [&](int u) {   // tile processed u-th (tile T-1-u): sum the wavefronts' partial sums per key
+    const float v = sk_group_sum<NW>(vpart[u & 3][fp][fkey]);
+    if (fp == 0) vraw[(T - 1 - u) & 3][fkey] = v;
   };
-  auto fold = [&](int u) {   // tile processed u-th (tile T-1-u): sum the wavefronts' partial sums
-    float v = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) v += vpart[u & 3][w][lane];
-    vraw[(T - 1 - u) & 3][lane] = v;
+  auto emit_tile = [&](int e) {   // moving average of tile e, whose neighbours are folded
+    const int s = e * SK_KT + fkey;
+    float a = 0.f;
+    for (int j = fp; j < ksz; j += NW) {
+      const int x = s + j - hw;
+      if (x >= 0 && x < SW) a += vraw[(x / SK_KT) & 3][x % SK_KT];
+    }
+    a = sk_group_sum<NW>(a);
+    if (fp == 0 && s < SW) out_row[s] = a * out_mul;
   };
   auto probs = [&](const f32x16& acc, int u, int cb) {
     float vs = 0.f;
@@ -382,15 +401,10 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       ++m;
       ++kc;
       stage = acquire();
-      if (u >= 1 && wave == (u & (NW - 1))) {
-        // the sums of the tile processed before this one are complete: fold them (the wavefronts
-        // take turns), then the tile before that (T-u+1) has both neighbours
-        fold(u - 1);
-        if (u >= 2) {
-          const int s = (T - u + 1) * SK_KT + lane;
-          if (s < SW) emit(s);
-        }
-      }
+      // the sums of the tile processed before this one are complete: fold them; tile T-u+2 had
+      // both neighbours folded (by other wavefronts) before the barrier just passed
+      if (u >= 1) fold(u - 1);
+      if (u >= 3) emit_tile(T - u + 2);
       mfma_block(false, stage, 0, acc_a);
       probs(acc_b, u, 1);
       interleave();
@@ -403,18 +417,19 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     ++kc;
   }
 
-  // ---- drain: the last two tiles' sums, then the moving average of tiles 2, 1, 0 ---------------
+  // ---- drain: fold the last two tiles processed (tiles 1 and 0) and write tiles 3, 2, 1, 0.  Tile 3 needs
+  // tile 4, whose ring slot tile 0 takes over, so tile 0 is folded after tiles 3 and 2 are written.
   __syncthreads();
-  if (wave == 0) {
-    if (T >= 2) fold(T - 2);
-    fold(T - 1);
-  }
+  if (T >= 2) fold(T - 2);
   __syncthreads();
-  {
-    const int last = min(3 * SK_KT, SW);
-    for (int s = tid; s < last; s += THREADS) emit(s);
-    for (int s = S + tid; s < score_stride; s += THREADS) out_row[s] = -INFINITY;
-  }
+  emit_tile(3);
+  emit_tile(2);
+  __syncthreads();
+  fold(T - 1);
+  __syncthreads();
+  emit_tile(1);
+  emit_tile(0);
+  for (int s = S + tid; s < score_stride; s += THREADS) out_row[s] = -INFINITY;
   if (row_max) {   // maximum of this row's scores, for the window fill: re-read what this workgroup wrote
     __syncthreads();
     float rmax = -INFINITY;
