@@ -32,12 +32,13 @@ class SamplingParams:
 class CompressionEngine:
     def __init__(self, scheduler: LlavaScheduler, model_runner: PagedKVRunner,
                  model_step: Callable[[List[Sequence], bool], List[int]], enable_compression: bool = True,
-                 async_compression: bool = False):
+                 async_compression: bool = False, decode_overlap=None):
         self.scheduler = scheduler
         self.model_runner = model_runner
         self.model_step = model_step
         self.enable_compression = enable_compression
         self.async_compression = async_compression
+        self.decode_overlap = decode_overlap          # a DecodeOverlapCompressor: compress a few layers per decode step
         self._pending_compression_events: Dict[int, object] = {}
         self.total_compression_time = 0.0
         self.total_freed_blocks = 0
@@ -57,6 +58,13 @@ class CompressionEngine:
             self._free_compressed_blocks(seqs)
         token_ids = self.model_step(seqs, is_prefill)
         compress_now = apply_compression and is_prefill and self.enable_compression
+        if self.decode_overlap is not None and self.enable_compression:
+            # kv-cache pipeline/nanovllm/engine/llava_engine.py: start after prefill, advance after every decode step
+            if compress_now:
+                self.decode_overlap.start_decode_overlap_compression(seqs)
+            elif not is_prefill:
+                self._free_compressed_blocks(self.decode_overlap.step_decode_overlap_compression(seqs))
+            compress_now = False
         if compress_now and not self.async_compression:
             sec, _ = self.model_runner.compress_kv_cache_batch(seqs)
             self.total_compression_time += sec

@@ -105,24 +105,33 @@ class BatchedGEMMCompressor(nn.Module):
                 dst += self._seg_len(n)
         return [(out[0][i], out[1][i]) for i in range(L)]
 
+    def paged_compressed_len(self, seq_len: int, it_len: Sequence[int]) -> int:
+        img = min(int(it_len[0]), seq_len) if it_len[0] > 0 else 0
+        return (self._seg_len(img) if img else 0) + (self._seg_len(seq_len - img) if seq_len > img else 0)
+
     @torch.no_grad()
     def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
-                      seq_len: int, it_len: Sequence[int]) -> int:
-        """In place on a paged pool ``[2, L, blocks, block_size, Hkv, D]`` for sequences that all hold
-        ``seq_len`` tokens; returns the compressed length."""
+                      seq_len: int, it_len: Sequence[int], layers: Optional[Tuple[int, int]] = None,
+                      out: Optional[torch.Tensor] = None) -> int:
+        """On a paged pool ``[2, L, blocks, block_size, Hkv, D]`` for sequences that all hold ``seq_len``
+        tokens: in place, or for the layers ``layers=(l0, l1)`` only, or into ``out [2, L, B, Hkv, C, D]``
+        leaving the pages untouched; returns the compressed length."""
         cf = self.compression_factor
         img = min(int(it_len[0]), seq_len) if it_len[0] > 0 else 0
+        l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
         dst = 0
-        views = [_lib.paged_view(kv_cache[p], block_tables, seq_lens, seq_len) for p in range(2)]
+        views = [_lib.paged_view(kv_cache[p][l0:l1], block_tables, seq_lens, seq_len) for p in range(2)]
+        dviews = views if out is None else [_lib.dense_view(out[p][l0:l1]) for p in range(2)]
         for s0, n, seg in ((0, img, "i"), (img, seq_len - img, "t")):
             if n == 0:
                 continue
-            for view, kind in ((views[0], "k"), (views[1], "v")):
+            for view, dview, kind in ((views[0], dviews[0], "k"), (views[1], dviews[1], "v")):
                 if n // cf < self.min_seq_len:
-                    if dst != s0:
-                        ops.copy_tokens(view, view, s0, n, dst)
+                    if out is not None or dst != s0:
+                        ops.copy_tokens(view, dview, s0, n, dst)
                 else:
-                    ops.ccm_mlp(view, view, self._weights(seg + kind, kv_cache.dtype, kv_cache.device), cf, s0, n, dst)
+                    ops.ccm_mlp(view, dview, self._weights(seg + kind, kv_cache.dtype, kv_cache.device, (l0, l1)), cf,
+                                s0, n, dst)
             dst += self._seg_len(n)
         return dst
 

@@ -101,19 +101,33 @@ class KVPressCompressor(nn.Module):
         ops.compact(kview, vview, _lib.dense_view(out_k), _lib.dense_view(out_v), idx)
         return out_k, out_v
 
+    def paged_compressed_len(self, seq_len: int, it_len=None) -> int:
+        n = self.get_compressed_length(seq_len)
+        if n >= seq_len:
+            return seq_len
+        if self.method_name in ("knorm", "random"):
+            return n
+        return int(self._static_indices(seq_len, n, torch.device("cpu")).numel())
+
     @torch.no_grad()
     def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
-                      seq_len: int, it_len=None) -> int:
-        """The same selection and gather in place on a paged pool ``[2, L, blocks, block_size, Hkv, D]``
-        for sequences that all hold ``seq_len`` tokens; returns the kept length."""
+                      seq_len: int, it_len=None, layers: Optional[Tuple[int, int]] = None,
+                      out: Optional[torch.Tensor] = None) -> int:
+        """The same selection and gather on a paged pool ``[2, L, blocks, block_size, Hkv, D]`` for
+        sequences that all hold ``seq_len`` tokens: in place, or for the layers ``layers=(l0, l1)`` only, or
+        into ``out [2, L, B, Hkv, C, D]`` leaving the pages untouched; returns the kept length."""
         S = seq_len
         n = self.get_compressed_length(S)
-        if n >= S:
-            return S
         dev = kv_cache.device
-        L, B = kv_cache.shape[1], block_tables.shape[0]
-        kview = _lib.paged_view(kv_cache[0], block_tables, seq_lens, S)
-        vview = _lib.paged_view(kv_cache[1], block_tables, seq_lens, S)
+        l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
+        L, B = l1 - l0, block_tables.shape[0]
+        kview = _lib.paged_view(kv_cache[0][l0:l1], block_tables, seq_lens, S)
+        vview = _lib.paged_view(kv_cache[1][l0:l1], block_tables, seq_lens, S)
+        if n >= S:
+            if out is not None:
+                ops.copy_tokens(kview, _lib.dense_view(out[0][l0:l1]), 0, S, 0)
+                ops.copy_tokens(vview, _lib.dense_view(out[1][l0:l1]), 0, S, 0)
+            return S
         if self.method_name == "knorm":
             idx = ops.topk_select(ops.knorm_mean_score(kview, dev), n).view(L, B, 1, n)
         elif self.method_name == "random":
@@ -123,7 +137,10 @@ class KVPressCompressor(nn.Module):
             t = self._static_indices(S, n, dev)
             n = t.numel()
             idx = t.view(1, 1, 1, n).expand(L, B, 1, n).contiguous()
-        ops.compact(kview, vview, kview, vview, idx)
+        if out is None:
+            ops.compact(kview, vview, kview, vview, idx)
+        else:
+            ops.compact(kview, vview, _lib.dense_view(out[0][l0:l1]), _lib.dense_view(out[1][l0:l1]), idx)
         return n
 
     @torch.no_grad()

@@ -105,25 +105,34 @@ class _CCMBase(nn.Module):
         img = min(int(it_len[0]), seq_len)
         return [("compress_ik", "compress_iv", 0, img), ("compress_tk", "compress_tv", img, seq_len - img)]
 
+    def paged_compressed_len(self, seq_len: int, it_len: Sequence[int]) -> int:
+        """Length ``paged_forward`` leaves for a sequence of ``seq_len`` tokens."""
+        return sum(self._segment_len(n) for _, _, _, n in self._paged_segments(seq_len, it_len))
+
     @torch.no_grad()
     def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
-                      seq_len: int, it_len: Sequence[int]) -> int:
-        """Compress, in place, sequences that all hold ``seq_len`` tokens in the pool
-        ``kv_cache [2, L, blocks, block_size, Hkv, D]``; the result occupies the leading slots of the
-        same block tables (what extract -> forward -> write-back leaves there).  Returns the
-        compressed length."""
+                      seq_len: int, it_len: Sequence[int], layers: Optional[Tuple[int, int]] = None,
+                      out: Optional[torch.Tensor] = None) -> int:
+        """Compress sequences that all hold ``seq_len`` tokens in the pool
+        ``kv_cache [2, L, blocks, block_size, Hkv, D]``.  By default in place: the result occupies the
+        leading slots of the same block tables (what extract -> forward -> write-back leaves there).
+        ``layers=(l0, l1)`` restricts the work to those layers; ``out [2, L, B, Hkv, C, D]`` receives the
+        result instead of the pages (which then stay untouched).  Returns the compressed length."""
         cf = self.compression_factor
-        views = [_lib.paged_view(kv_cache[p], block_tables, seq_lens, seq_len) for p in range(2)]
+        l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
+        views = [_lib.paged_view(kv_cache[p][l0:l1], block_tables, seq_lens, seq_len) for p in range(2)]
+        dviews = views if out is None else [_lib.dense_view(out[p][l0:l1]) for p in range(2)]
         dst = 0
         for gk, gv, s0, n in self._paged_segments(seq_len, it_len):
             if n == 0:
                 continue
-            for view, g in ((views[0], gk), (views[1], gv)):
+            for view, dview, g in ((views[0], dviews[0], gk), (views[1], dviews[1], gv)):
                 if n // cf < self.min_seq_len:
-                    if dst != s0:
-                        ops.copy_tokens(view, view, s0, n, dst)
+                    if out is not None or dst != s0:
+                        ops.copy_tokens(view, dview, s0, n, dst)
                 else:
-                    ops.ccm_mlp(view, view, self._weights(g, kv_cache.dtype, kv_cache.device), cf, s0, n, dst)
+                    w = tuple(t[l0:l1] for t in self._weights(g, kv_cache.dtype, kv_cache.device))
+                    ops.ccm_mlp(view, dview, w, cf, s0, n, dst)
             dst += self._segment_len(n)
         return dst
 

@@ -436,3 +436,73 @@ def test_lazy_compression_engine_on_the_pool(dev):
         assert steps < 50
     bm = sched.block_manager
     assert len(bm.free_block_ids) == 9 and not bm.used_block_ids and llm.total_freed_blocks == 6
+
+
+@pytest.mark.parametrize("backend", ["mlp", "kvpress"])
+def test_decode_overlap_compression_splices_generated_rows(dev, backend):
+    """A few layers per decode step on a side stream; at the end the pages hold compress(prefill rows) followed by
+    the rows generated meanwhile, and the untouched pages served the steps in between."""
+    from fastcache_amd.engine.decode_overlap import DecodeOverlapCompressor
+    dtype, L, H, img = torch.float16, 5, 2, 100
+    lens = [600, 600, 520]
+    case = synth.make_paged_case(seed=41, num_layers=L, batch=3, num_kv_heads=H, seq_lens=lens, dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0, reserve_tokens=8)
+    if backend == "mlp":
+        torch.manual_seed(2)
+        comp = KVCacheLinearDecoupleCompressor(llava_cfg(L, H), compression_factor=2).to(dev).to(dtype).eval()
+        sd = {k: v.detach().cpu().float() for k, v in comp.state_dict().items()}
+        oracle = lambda hf, n: occm.linear_decouple_forward(hf, [img, max(1, n - img)], sd, 2, 1)
+    else:
+        comp = KVPressCompressor("knorm", 0.5)
+        oracle = lambda hf, n: [opress.adapter_compress_layer("knorm", k, v, 0.5) for k, v in hf]
+    runner = PagedKVRunner(L, H, 128, num_blocks=16, dtype=dtype, device=dev, image_token_len=img, compressor=comp)
+    bm = BlockManager(16, 256)
+    seqs = [Sequence(list(range(1000 * i, 1000 * i + n))) for i, n in enumerate(lens)]
+    for s in seqs:
+        bm.allocate(s)
+    _fill_pool_from_case(runner, case, seqs)
+    before = runner.kv_cache.cpu()
+
+    ov = DecodeOverlapCompressor(runner, layers_per_step=2)
+    ov.start_decode_overlap_compression(seqs)
+    assert all(ov.pending(s.seq_id) for s in seqs)
+    g = torch.Generator().manual_seed(77)
+    appended = {s.seq_id: [] for s in seqs}
+    steps = 0
+    done = []
+    while len(done) < 3:
+        # a decode step: one new KV row per sequence at position len(seq), then the sampled token is appended
+        for s in seqs:
+            row = torch.randn(2, L, H, 128, generator=g).to(dtype)
+            pos = len(s)
+            blk = s.block_table[pos // 256]
+            runner.kv_cache[:, :, blk, pos % 256] = row.to(dev)
+            appended[s.seq_id].append(row)
+            s.append_token(5)
+        steps += 1
+        finished = ov.step_decode_overlap_compression(seqs)
+        if steps < 3:
+            assert finished == []                                   # 5 layers, 2 per step
+            # the pages still hold the uncompressed prefix while compression is under way
+            assert torch.equal(runner.kv_cache[:, :, seqs[0].block_table[0], :100].cpu(),
+                               before[:, :, seqs[0].block_table[0], :100])
+        done += finished
+    assert steps == 3 and {s.seq_id for s in done} == {s.seq_id for s in seqs}
+    torch.cuda.synchronize()
+    for s, n in zip(seqs, lens):
+        hf = opaged.extract_kv(before, s.block_table, n)
+        ref = oracle(hf, n)
+        C = ref[0][0].shape[2]
+        assert runner._compressed_lens[s.seq_id] == C + 3 and not ov.pending(s.seq_id)
+        got = opaged.extract_kv(runner.kv_cache.cpu(), s.block_table, C + 3)
+        for layer in range(L):
+            for p in range(2):
+                if backend == "mlp":
+                    assert_mlp_close(got[layer][p][:, :, :C], ref[layer][p], dtype)
+                else:
+                    assert torch.equal(got[layer][p][:, :, :C], ref[layer][p])
+                tail = torch.stack([r[p, layer] for r in appended[s.seq_id]], dim=1).unsqueeze(0)   # [1, H, 3, D]
+                assert torch.equal(got[layer][p][:, :, C:], tail)
+    freed = free_compressed_blocks(bm, runner, seqs)
+    assert freed == sum(-(-(n + 3) // 256) - (-(-(runner_len) // 256)) for n, runner_len in
+                        zip(lens, [s.kv_cache_len for s in seqs]))
