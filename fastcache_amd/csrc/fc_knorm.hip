@@ -143,3 +143,82 @@ extern "C" int fc_knorm_score(const fc_kv_view* keys, float* scores, int32_t sco
 extern "C" int fc_knorm_mean_score(const fc_kv_view* keys, float* out, int32_t score_stride, void* stream) {
   return launch_knorm<true>(keys, out, score_stride, stream, "fc_knorm_mean_score");
 }
+
+// ---- observed attention: column sums of a materialised attention matrix -----------------------------
+// out[b][hk][s] = mean over the G query heads of the kv group of ( sum over queries q of attn[b][h][q][s] )
+//                 / (number of queries that can attend key s under the causal mask = Sk - s).
+// One thread per key column, 256 columns per workgroup, rows read coalesced; the query range is split
+// over gridDim.z slices that are combined with a fixed-order second pass (deterministic, no atomics).
+template <int DTYPE>
+__global__ __launch_bounds__(256) void attn_colsum_kernel(const char* __restrict__ attn, int Hq, int G, int Sq, int Sk,
+                                                          int qsplit, float* __restrict__ partial) {
+  const int s = blockIdx.x * 256 + threadIdx.x;
+  const int hk = blockIdx.y % (Hq / G), b = blockIdx.y / (Hq / G);
+  const int slice = blockIdx.z;
+  if (s >= Sk) return;
+  const int q0 = (int)((long long)Sq * slice / qsplit), q1 = (int)((long long)Sq * (slice + 1) / qsplit);
+  float acc = 0.f;
+  for (int g = 0; g < G; ++g) {
+    const long long base = (((long long)b * Hq + hk * G + g) * Sq) * Sk + s;
+    float a = 0.f;
+    for (int q = q0; q < q1; ++q) {
+      const long long i = base + (long long)q * Sk;
+      if constexpr (DTYPE == FC_F32) a += reinterpret_cast<const float*>(attn)[i];
+      else {
+        const unsigned short r = reinterpret_cast<const unsigned short*>(attn)[i];
+        a += DTYPE == FC_BF16 ? fc_bf16_to_float(r) : fc_half_to_float(r);
+      }
+    }
+    acc += a;
+  }
+  partial[(((long long)slice * gridDim.y + blockIdx.y)) * Sk + s] = acc;
+}
+
+__global__ __launch_bounds__(256) void attn_colsum_finish_kernel(const float* __restrict__ partial, int rows, int Sk,
+                                                                 int qsplit, int G, float* __restrict__ out) {
+  const int s = blockIdx.x * 256 + threadIdx.x;
+  const int r = blockIdx.y;
+  if (s >= Sk) return;
+  float acc = 0.f;
+  for (int k = 0; k < qsplit; ++k) acc += partial[((long long)k * rows + r) * Sk + s];
+  out[(long long)r * Sk + s] = acc / (float)(Sk - s) / (float)G;
+}
+
+extern "C" int64_t fc_observed_attention_workspace_bytes(int32_t batch, int32_t num_kv_heads, int32_t sk) {
+  if (batch <= 0 || num_kv_heads <= 0 || sk <= 0) return 0;
+  return (int64_t)16 * batch * num_kv_heads * sk * 4;
+}
+
+extern "C" int fc_observed_attention_score(const void* attn, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                           int32_t sq, int32_t sk, int32_t dtype, float* scores, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+  const char* who = "fc_observed_attention_score";
+  FC_REQUIRE(attn && scores && workspace, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(batch > 0 && num_kv_heads > 0 && num_q_heads > 0 && num_q_heads % num_kv_heads == 0 && sq > 0 && sk > 0,
+             FC_EINVAL, "%s: bad sizes", who);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+  FC_REQUIRE(workspace_bytes >= fc_observed_attention_workspace_bytes(batch, num_kv_heads, sk), FC_EINVAL,
+             "%s: workspace too small", who);
+  FC_REQUIRE((long long)batch * num_kv_heads <= 65535, FC_EUNSUPPORTED, "%s: too many (batch, head) rows", who);
+  const int rows = batch * num_kv_heads;
+  const int col_blocks = (sk + 255) / 256;
+  // enough query slices to fill the chip (at most 16, what the workspace holds)
+  int qsplit = 1;
+  while (qsplit < 16 && (long long)col_blocks * rows * qsplit < 2048 && qsplit * 64 <= sq) qsplit *= 2;
+  const int G = num_q_heads / num_kv_heads;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(col_blocks, rows, qsplit);
+  if (dtype == FC_F32)
+    hipLaunchKernelGGL((attn_colsum_kernel<FC_F32>), grid, dim3(256), 0, st, (const char*)attn, num_q_heads, G, sq, sk,
+                       qsplit, (float*)workspace);
+  else if (dtype == FC_F16)
+    hipLaunchKernelGGL((attn_colsum_kernel<FC_F16>), grid, dim3(256), 0, st, (const char*)attn, num_q_heads, G, sq, sk,
+                       qsplit, (float*)workspace);
+  else
+    hipLaunchKernelGGL((attn_colsum_kernel<FC_BF16>), grid, dim3(256), 0, st, (const char*)attn, num_q_heads, G, sq, sk,
+                       qsplit, (float*)workspace);
+  hipLaunchKernelGGL(attn_colsum_finish_kernel, dim3(col_blocks, rows), dim3(256), 0, st, (const float*)workspace, rows,
+                     sk, qsplit, G, scores);
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}

@@ -67,6 +67,87 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(const signed char*
   for (int j = lane; j < d; j += 64) qz_store<ODT>(out, base + j, (float)q[base + j] * sc);
 }
 
+// 4-bit codes of groups of `g` elements, two per byte (element 2j in the low nibble).
+// MODE 0: integer codes, scale = clamp(max|x| / 7, 1e-8), code = clamp(round(x / scale), -8, 7) + 8.
+// MODE 1: NF4, scale = clamp(max|x|, 1e-8), code = index of the table entry nearest to x / scale
+//         (table rounded to the tensor dtype, differences rounded to it as well, first minimum wins).
+__constant__ float kNf4Table[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+                                    -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+                                    0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f,
+                                    0.33791524171829224f, 0.44070982933044434f, 0.5626170039176941f,
+                                    0.7229568362236023f, 1.0f};
+
+template <int DTYPE, int MODE>
+__device__ __forceinline__ int qz_code4(float v, float sc) {
+  const float t = qz_round<DTYPE>(v / sc);
+  if constexpr (MODE == 0) {
+    float r = rintf(t);
+    r = fminf(fmaxf(r, -8.f), 7.f);
+    return (r != r) ? 0 : (int)r + 8;
+  } else {
+    int best = 0;
+    float bd = fabsf(qz_round<DTYPE>(t - qz_round<DTYPE>(kNf4Table[0])));
+#pragma unroll
+    for (int i = 1; i < 16; ++i) {
+      const float d = fabsf(qz_round<DTYPE>(t - qz_round<DTYPE>(kNf4Table[i])));
+      if (d < bd) { bd = d; best = i; }
+    }
+    return best;
+  }
+}
+
+template <int DTYPE, int MODE>
+__global__ __launch_bounds__(256) void quantize_group4_kernel(const char* __restrict__ x, long long groups, int g,
+                                                              unsigned char* __restrict__ packed,
+                                                              char* __restrict__ scale) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= groups) return;
+  const long long base = r * g;
+  float mx = 0.f;
+  bool has_nan = false;
+  for (int j = lane; j < g; j += 64) {
+    const float v = qz_load<DTYPE>(x, base + j);
+    has_nan |= v != v;
+    mx = fmaxf(mx, fabsf(v));
+  }
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mx = __builtin_nanf("");
+  float sc = MODE == 0 ? qz_round<DTYPE>(mx / 7.f) : mx;
+  sc = qz_round<DTYPE>(sc != sc ? sc : fmaxf(sc, 1e-8f));
+  if (lane == 0) qz_store<DTYPE>(scale, r, sc);
+  for (int j = lane; j < g / 2; j += 64) {
+    const int lo = qz_code4<DTYPE, MODE>(qz_load<DTYPE>(x, base + 2 * j), sc);
+    const int hi = qz_code4<DTYPE, MODE>(qz_load<DTYPE>(x, base + 2 * j + 1), sc);
+    packed[base / 2 + j] = (unsigned char)(lo | (hi << 4));
+  }
+}
+
+// TDT: dtype the level table is rounded to (the dtype asked for); SDT: dtype of scale; ODT: output dtype
+template <int TDT, int SDT, int ODT, int MODE>
+__global__ __launch_bounds__(256) void dequantize_group4_kernel(const unsigned char* __restrict__ packed,
+                                                                const char* __restrict__ scale, long long groups,
+                                                                int g, char* __restrict__ out) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= groups) return;
+  const float sc = qz_load<SDT>(scale, r);
+  const long long base = r * g;
+  for (int j = lane; j < g / 2; j += 64) {
+    const unsigned b = packed[base / 2 + j];
+    float lo, hi;
+    if constexpr (MODE == 0) {
+      lo = (float)(int)(b & 15u) - 8.f;
+      hi = (float)(int)(b >> 4) - 8.f;
+    } else {
+      lo = qz_round<TDT>(kNf4Table[b & 15u]);
+      hi = qz_round<TDT>(kNf4Table[b >> 4]);
+    }
+    qz_store<ODT>(out, base + 2 * j, lo * sc);
+    qz_store<ODT>(out, base + 2 * j + 1, hi * sc);
+  }
+}
+
 extern "C" int fc_quantize_rows(const void* x, int64_t rows, int32_t d, int32_t dtype, int32_t bits, int8_t* q,
                                 void* scale, void* stream) {
   const char* who = "fc_quantize_rows";
@@ -108,6 +189,57 @@ extern "C" int fc_dequantize_rows(const int8_t* q, const void* scale, int64_t ro
   else if (out_dtype == FC_F32 && scale_dtype == FC_BF16) DQ(FC_BF16, FC_F32);
   else { fc_set_error("%s: scale dtype %d with output dtype %d", who, scale_dtype, out_dtype); return FC_EUNSUPPORTED; }
 #undef DQ
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_quantize_group4(const void* x, int64_t groups, int32_t group_size, int32_t dtype, int32_t nf4,
+                                  uint8_t* packed, void* scale, void* stream) {
+  const char* who = "fc_quantize_group4";
+  FC_REQUIRE(x && packed && scale, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(groups >= 0 && group_size > 0 && group_size % 2 == 0, FC_EINVAL, "%s: bad sizes groups=%lld group_size=%d",
+             who, (long long)groups, group_size);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (groups == 0) return FC_OK;
+  const long long blocks = (groups + 3) / 4;
+  FC_REQUIRE(blocks <= 2147483647LL, FC_EUNSUPPORTED, "%s: too many groups", who);
+  hipStream_t st = (hipStream_t)stream;
+#define QG(DT, MD) hipLaunchKernelGGL((quantize_group4_kernel<DT, MD>), dim3((unsigned)blocks), dim3(256), 0, st,     \
+                                      (const char*)x, (long long)groups, group_size, (unsigned char*)packed, (char*)scale)
+#define QGD(DT) do { if (nf4) QG(DT, 1); else QG(DT, 0); } while (0)
+  if (dtype == FC_F32) QGD(FC_F32); else if (dtype == FC_F16) QGD(FC_F16); else QGD(FC_BF16);
+#undef QGD
+#undef QG
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_dequantize_group4(const uint8_t* packed, const void* scale, int64_t groups, int32_t group_size,
+                                    int32_t scale_dtype, int32_t table_dtype, int32_t nf4, void* out, void* stream) {
+  const char* who = "fc_dequantize_group4";
+  FC_REQUIRE(packed && scale && out, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(groups >= 0 && group_size > 0 && group_size % 2 == 0, FC_EINVAL, "%s: bad sizes groups=%lld group_size=%d",
+             who, (long long)groups, group_size);
+  if (groups == 0) return FC_OK;
+  const long long blocks = (groups + 3) / 4;
+  FC_REQUIRE(blocks <= 2147483647LL, FC_EUNSUPPORTED, "%s: too many groups", who);
+  hipStream_t st = (hipStream_t)stream;
+#define DG(T, S, O, MD) hipLaunchKernelGGL((dequantize_group4_kernel<T, S, O, MD>), dim3((unsigned)blocks), dim3(256), 0, \
+                                           st, (const unsigned char*)packed, (const char*)scale, (long long)groups,   \
+                                           group_size, (char*)out)
+#define DGD(T, S, O) do { if (nf4) DG(T, S, O, 1); else DG(T, S, O, 0); } while (0)
+  // output dtype = promotion of (table dtype, scale dtype): equal dtypes, or fp32 when either is fp32
+  const int t = table_dtype, sd = scale_dtype;
+  if (t == FC_F32 && sd == FC_F32) DGD(FC_F32, FC_F32, FC_F32);
+  else if (t == FC_F16 && sd == FC_F16) DGD(FC_F16, FC_F16, FC_F16);
+  else if (t == FC_BF16 && sd == FC_BF16) DGD(FC_BF16, FC_BF16, FC_BF16);
+  else if (t == FC_F32 && sd == FC_F16) DGD(FC_F32, FC_F16, FC_F32);
+  else if (t == FC_F32 && sd == FC_BF16) DGD(FC_F32, FC_BF16, FC_F32);
+  else if (t == FC_F16 && sd == FC_F32) DGD(FC_F16, FC_F32, FC_F32);
+  else if (t == FC_BF16 && sd == FC_F32) DGD(FC_BF16, FC_F32, FC_F32);
+  else { fc_set_error("%s: table dtype %d with scale dtype %d", who, t, sd); return FC_EUNSUPPORTED; }
+#undef DGD
+#undef DG
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }

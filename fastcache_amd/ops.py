@@ -162,6 +162,23 @@ def ccm_mlp(src: FcKvView, dst: FcKvView, weights: Tuple[torch.Tensor, ...], cf:
                            current_stream()), "fc_ccm_mlp")
 
 
+def observed_attention_score(attentions: torch.Tensor, num_kv_heads: int) -> torch.Tensor:
+    """fp32 ``[B, Hkv, Sk]`` from a materialised attention matrix ``[B, Hq, Sq, Sk]``: per key, the attention it
+    received summed over the queries, divided by the number of queries that could see it, averaged over the group."""
+    _lib.require_gpu(attentions, "attentions")
+    if attentions.dim() != 4:
+        raise FastcacheError(f"attentions must be [B, Hq, Sq, Sk], got {tuple(attentions.shape)}")
+    a = attentions.contiguous()
+    B, Hq, Sq, Sk = a.shape
+    out = torch.empty((B, num_kv_heads, Sk), dtype=torch.float32, device=a.device)
+    nbytes = fn("fc_observed_attention_workspace_bytes")(B, num_kv_heads, Sk)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=a.device)
+    check(fn("fc_observed_attention_score")(a.data_ptr(), B, Hq, num_kv_heads, Sq, Sk, _lib.dtype_code(a.dtype),
+                                            out.data_ptr(), ws.data_ptr(), nbytes, current_stream()),
+          "fc_observed_attention_score")
+    return out
+
+
 def quantize_rows(x: torch.Tensor, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-row (last dimension) symmetric quantisation: ``(q int8 like x, scale x.dtype [..., 1])``."""
     _lib.require_gpu(x, "x")
@@ -192,6 +209,40 @@ def dequantize_rows(q: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype) ->
     out = torch.empty(qc.shape, dtype=out_dtype, device=q.device)
     check(fn("fc_dequantize_rows")(qc.data_ptr(), sc.data_ptr(), rows, d, _lib.dtype_code(sc.dtype),
                                    _lib.dtype_code(out_dtype), out.data_ptr(), current_stream()), "fc_dequantize_rows")
+    return out
+
+
+def quantize_group4(x: torch.Tensor, group_size: int, nf4: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Groups of ``group_size`` consecutive elements -> ``(packed uint8 [..., D/2], scale [..., D/group_size])``."""
+    _lib.require_gpu(x, "x")
+    D = x.shape[-1]
+    if x.numel() == 0 or x.numel() % group_size or group_size % 2:
+        raise FastcacheError(f"quantize_group4: {tuple(x.shape)} is not a whole number of groups of {group_size}")
+    xc = x.contiguous()
+    groups = xc.numel() // group_size
+    packed = torch.empty(xc.numel() // 2, dtype=torch.uint8, device=x.device)
+    scale = torch.empty(groups, dtype=x.dtype, device=x.device)
+    check(fn("fc_quantize_group4")(xc.data_ptr(), groups, group_size, _lib.dtype_code(x.dtype), int(bool(nf4)),
+                                   packed.data_ptr(), scale.data_ptr(), current_stream()), "fc_quantize_group4")
+    return packed.view(*xc.shape[:-1], -1), scale.view(*xc.shape[:-1], -1)
+
+
+def dequantize_group4(packed: torch.Tensor, scale: torch.Tensor, group_size: int, nf4: bool,
+                      dtype: torch.dtype) -> torch.Tensor:
+    """Inverse of :func:`quantize_group4`; output ``[..., 2 * packed.shape[-1]]`` in promote(dtype, scale.dtype)."""
+    _lib.require_gpu(packed, "packed")
+    _lib.require_gpu(scale, "scale")
+    if packed.dtype != torch.uint8:
+        raise FastcacheError(f"dequantize_group4: uint8 codes expected, got {packed.dtype}")
+    n = packed.numel() * 2
+    if n % group_size or scale.numel() != n // group_size:
+        raise FastcacheError("dequantize_group4: one scale per group expected")
+    out_dtype = torch.promote_types(dtype, scale.dtype)
+    pc, sc = packed.contiguous(), scale.contiguous()
+    out = torch.empty((*pc.shape[:-1], pc.shape[-1] * 2), dtype=out_dtype, device=packed.device)
+    check(fn("fc_dequantize_group4")(pc.data_ptr(), sc.data_ptr(), n // group_size, group_size,
+                                     _lib.dtype_code(sc.dtype), _lib.dtype_code(dtype), int(bool(nf4)),
+                                     out.data_ptr(), current_stream()), "fc_dequantize_group4")
     return out
 
 

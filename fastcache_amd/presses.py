@@ -174,6 +174,42 @@ class SnapKVPress(ScorerPress):
 
 
 @dataclass
+class TOVAPress(ScorerPress):
+    """Attention of the last query over the other keys, averaged over all query heads and shared by the kv
+    heads; the last token is always kept.  Uses ``attentions`` when the model returns them, otherwise computes the
+    last query's softmax (window of one, no pooling) from ``kwargs['queries']`` or the module's ``q_proj``."""
+    compression_ratio: float = 0.0
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        B, Hkv, S, D = keys.shape
+        if attentions is not None:
+            per_head = attentions[..., -1, :-1].float()                               # [B, Hq, S-1]
+            mean = per_head.mean(1, keepdim=True)
+        else:
+            snap = SnapKVPress(window_size=1, kernel_size=1)
+            q = snap.window_queries(module, hidden_states, kwargs)                     # [B, Hq, 1, D]
+            group_sums = ops.snapkv_score(_lib.dense_view(keys), q.to(keys.dtype), 1, 1, True, "sum",
+                                          1.0 / math.sqrt(D))[0]                       # [B, Hkv, S]: sums per kv group
+            mean = group_sums[..., :S - 1].sum(1, keepdim=True) / q.shape[1]          # mean over all query heads
+        scores = torch.empty((B, Hkv, S), dtype=torch.float32, device=keys.device)
+        scores[..., :S - 1] = mean
+        scores[..., S - 1] = mean.max()
+        return scores
+
+
+@dataclass
+class ObservedAttentionPress(ScorerPress):
+    """Attention each key received during prefill (needs the model's attention weights, i.e. eager attention):
+    summed over the queries, divided by the number of queries that can see the key, averaged over the group."""
+    compression_ratio: float = 0.0
+    output_attentions: bool = False
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        assert attentions is not None, 'Set output_attentions=True and attn_implementation="eager" to use this hook'
+        return ops.observed_attention_score(attentions, keys.shape[1])
+
+
+@dataclass
 class StreamingLLMPress(ScorerPress):
     """Keep the first ``n_sink`` tokens and the most recent ones."""
     compression_ratio: float = 0.0
@@ -202,6 +238,8 @@ class RandomPress(ScorerPress):
 
 
 # names the reference gives its timed subclasses (utils_compress.py:302-324)
+TOVAPressWithTime = TOVAPress
+ObservedAttentionPressWithTime = ObservedAttentionPress
 KnormPressWithTime = KnormPress
 SnapKVPressWithTime = SnapKVPress
 StreamingLLMPressWithTime = StreamingLLMPress
@@ -209,17 +247,19 @@ RandomPressWithTime = RandomPress
 
 
 def press_select(compression_method: str = "Knorm", compression_ratio: float = 0.8) -> ScorerPress:
-    """utils_compress.py:327-349.  'ExpectedAttention', 'TOVA' and 'Quantized' are not part of this
-    build and raise; any other name gives the Knorm press, as in the reference."""
+    """utils_compress.py:327-349.  'ExpectedAttention' and 'Quantized' are not part of this build and
+    raise; any other name gives the Knorm press, as in the reference."""
     if compression_method == "StreamingLLM":
         press = StreamingLLMPress(compression_ratio=compression_ratio)
     elif compression_method == "RandomPress":
         press = RandomPress(compression_ratio=compression_ratio)
     elif compression_method == "SnapKV":
         press = SnapKVPress(compression_ratio=compression_ratio)
-    elif compression_method in ("ExpectedAttention", "TOVA", "Quantized"):
-        raise NotImplementedError(f"press '{compression_method}' is outside the KV-cache compression path "
-                                  "built here (Knorm, SnapKV, StreamingLLM, RandomPress)")
+    elif compression_method == "TOVA":
+        press = TOVAPress(compression_ratio=compression_ratio)
+    elif compression_method in ("ExpectedAttention", "Quantized"):
+        raise NotImplementedError(f"press '{compression_method}' is not part of this build (built: Knorm, SnapKV, "
+                                  "TOVA, ObservedAttention, StreamingLLM, RandomPress)")
     else:
         press = KnormPress(compression_ratio=compression_ratio)
     press.reset_timeCheck()

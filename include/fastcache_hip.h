@@ -175,6 +175,19 @@ int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weight
                int32_t cf, int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream);
 
 /*
+ * Observed-attention scores from a materialised attention matrix attn[batch][num_q_heads][sq][sk]
+ * (fp32 / fp16 / bf16, contiguous):
+ *   scores[b][hk][s] = mean over the query heads of kv group hk of (sum_q attn[b][h][q][s]) / (sk - s),
+ * fp32, contiguous [batch][num_kv_heads][sk].  workspace: fc_observed_attention_workspace_bytes bytes.
+ * Replaces ObservedAttentionPress.score of the kvpress package as the reference uses it
+ * (utils_ccm/utils_compress.py:22-24, 302-349).
+ */
+int64_t fc_observed_attention_workspace_bytes(int32_t batch, int32_t num_kv_heads, int32_t sk);
+int fc_observed_attention_score(const void* attn, int32_t batch, int32_t num_q_heads,
+                                int32_t num_kv_heads, int32_t sq, int32_t sk, int32_t dtype,
+                                float* scores, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * One Linear layer on dense row-major matrices: y[m][n] = act(x[m][k] * weight^T + bias), weight
  * in nn.Linear layout [n][k], fp16 or bf16 throughout, fp32 accumulation, one rounding to the
  * storage dtype.  bias may be NULL; apply_relu != 0 clamps at zero.  k must be a multiple of 16,
@@ -198,6 +211,21 @@ int fc_quantize_rows(const void* x, int64_t rows, int32_t d, int32_t dtype, int3
                      int8_t* q, void* scale, void* stream);
 int fc_dequantize_rows(const int8_t* q, const void* scale, int64_t rows, int32_t d,
                        int32_t scale_dtype, int32_t out_dtype, void* out, void* stream);
+
+/*
+ * 4-bit quantisation of groups of `group_size` consecutive elements, two codes per byte (element 2j in
+ * the low nibble), one scale per group in the dtype of x.
+ *   nf4 == 0: scale = clamp(max|x| / 7, 1e-8), code = clamp(round(x / scale), -8, 7) + 8;
+ *   nf4 != 0: scale = clamp(max|x|, 1e-8), code = index of the nearest of the 16 NF4 levels.
+ * De-quantisation: out = level * scale with level = code - 8, or the NF4 level rounded to table_dtype;
+ * the output dtype is the promotion of table_dtype and scale_dtype.
+ * Replaces QuantizationMethod._quantize_int4 / _quantize_nf4 / dequantize
+ * (nanovllm/autocompress/methods.py:654-734).
+ */
+int fc_quantize_group4(const void* x, int64_t groups, int32_t group_size, int32_t dtype, int32_t nf4,
+                       uint8_t* packed, void* scale, void* stream);
+int fc_dequantize_group4(const uint8_t* packed, const void* scale, int64_t groups, int32_t group_size,
+                         int32_t scale_dtype, int32_t table_dtype, int32_t nf4, void* out, void* stream);
 
 /*
  * Plain ordered token copy src[seg_start + i] -> dst[dst_start + i], i < count, per

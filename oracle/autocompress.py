@@ -63,3 +63,58 @@ def dequantize(X_quant: torch.Tensor, scale: torch.Tensor, dtype=None) -> torch.
     if dtype is None:
         dtype = torch.float16
     return X_quant.to(dtype) * scale
+
+
+# ---- QuantizationMethod (nanovllm/autocompress/methods.py:636-757) ---------------------------------------
+NF4_LEVELS = [-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
+              -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
+              0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
+              0.7229568362236023, 1.0]
+
+
+def quantize_int8(tensor: torch.Tensor):
+    """methods.py:639-643 (symmetric)."""
+    scale = tensor.abs().amax(dim=-1, keepdim=True) / 127.0
+    scale = scale.clamp(min=1e-8)
+    return (tensor / scale).round().clamp(-128, 127).to(torch.int8), scale
+
+
+def quantize_int4(tensor: torch.Tensor, group_size: int):
+    """methods.py:654-669.  The reference packs with ``|`` on the floating ``quantized`` tensor, which torch
+    rejects; the packing it describes (low nibble = even element + 8, high nibble = odd element + 8) is done
+    on integers here."""
+    shape = tensor.shape
+    t = tensor.reshape(-1, group_size)
+    scale = t.abs().amax(dim=-1, keepdim=True) / 7.0
+    scale = scale.clamp(min=1e-8)
+    q = (t / scale).round().clamp(-8, 7).to(torch.int32).view(-1, 2)
+    packed = ((q[:, 0] + 8) | ((q[:, 1] + 8) << 4)).to(torch.uint8)
+    return packed.view(*shape[:-1], -1), scale.view(*shape[:-1], -1)
+
+
+def quantize_nf4(tensor: torch.Tensor, group_size: int):
+    """methods.py:689-715."""
+    table = torch.tensor(NF4_LEVELS, dtype=tensor.dtype)
+    shape = tensor.shape
+    t = tensor.reshape(-1, group_size)
+    scale = t.abs().amax(dim=-1, keepdim=True)
+    scale = scale.clamp(min=1e-8)
+    normalized = t / scale
+    diff = (normalized.unsqueeze(-1) - table).abs()
+    q = diff.argmin(dim=-1).to(torch.uint8).view(-1, 2)
+    packed = (q[:, 0] | (q[:, 1] << 4)).to(torch.uint8)
+    return packed.view(*shape[:-1], -1), scale.view(*shape[:-1], -1)
+
+
+def dequantize_4bit(packed: torch.Tensor, scale: torch.Tensor, group_size: int, nf4: bool, dtype=torch.float16):
+    """methods.py:722-747.  ``unpacked * scale`` only broadcasts in the reference when there is one group per row;
+    here every group is scaled by its own factor.  The NF4 look-up indexes with integer (not uint8) tensors."""
+    low, high = (packed & 0x0F).long(), ((packed >> 4) & 0x0F).long()
+    if nf4:
+        table = torch.tensor(NF4_LEVELS, dtype=dtype)
+        lo, hi = table[low], table[high]
+    else:
+        lo, hi = low.to(dtype) - 8, high.to(dtype) - 8
+    unpacked = torch.stack([lo, hi], dim=-1).view(*packed.shape[:-1], -1)
+    g = unpacked.reshape(-1, group_size) * scale.reshape(-1, 1)
+    return g.view(*packed.shape[:-1], -1)

@@ -97,6 +97,36 @@ def snapkv_score(queries: torch.Tensor, keys: torch.Tensor, window_size: int, ke
     return F.pad(v, (0, W), value=v.max().item())
 
 
+def tova_score(queries: Optional[torch.Tensor], keys: torch.Tensor, attentions: Optional[torch.Tensor] = None,
+               scale: Optional[float] = None) -> torch.Tensor:
+    """kvpress ``TOVAPress.score`` (third party, restated from its published description; PARITY UNPINNED):
+    the attention of the LAST query over the other keys, averaged over ALL query heads, the same row for every
+    kv head; the last position gets the maximum so that it is never pruned.  ``attentions [B, Hq, Sq, S]`` is used
+    when given, otherwise the softmax is computed from ``queries [B, Hq, 1, D]`` (the last position)."""
+    B, Hkv, S, D = keys.shape
+    if attentions is not None:
+        attn = attentions[..., -1:, :-1].float()
+    else:
+        G = queries.shape[1] // Hkv
+        if scale is None:
+            scale = 1.0 / math.sqrt(D)
+        logits = torch.matmul(queries.float(), keys.float().repeat_interleave(G, dim=1).transpose(2, 3)) * scale
+        attn = F.softmax(logits, dim=-1, dtype=torch.float32)[..., :-1]          # [B, Hq, 1, S-1]
+    scores = attn.mean(1)                                                        # [B, 1, S-1]
+    scores = scores.repeat(1, Hkv, 1)
+    return F.pad(scores, (0, 1), value=scores.max().item())
+
+
+def observed_attention_score(attentions: torch.Tensor, num_kv_heads: int) -> torch.Tensor:
+    """kvpress ``ObservedAttentionPress.score`` (third party; PARITY UNPINNED): attention received by each key
+    summed over the queries, divided by the number of queries that can see the key, averaged over the group."""
+    B, Hq, Sq, S = attentions.shape
+    scores = attentions.float().sum(2)
+    n_tokens_in_sum = torch.arange(S, 0, -1).float()
+    scores = scores / n_tokens_in_sum
+    return scores.view(B, num_kv_heads, -1, S).mean(2)
+
+
 # --------------------------------------------------------------------------------------------
 # selection
 # --------------------------------------------------------------------------------------------

@@ -137,3 +137,36 @@ def test_hardware_profile_and_streams(dev):
         x += 1
     sm.synchronize_compress_to_main()
     assert float((x * 2).sum()) == 2.0 * (1 << 20)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["int8", "int4", "nf4"])
+def test_quantization_method_bit_exact(dev, dtype, kind):
+    """QuantizationMethod (int8 per row, int4 / NF4 per group of 128, two codes per byte) against the oracle:
+    codes, scales and de-quantised values bit for bit."""
+    g = torch.Generator().manual_seed(len(kind))
+    X = (torch.randn(2, 3, 50, 128, generator=g) * 1.7).to(dtype)
+    V = (torch.randn(2, 3, 50, 128, generator=g) * 0.3).to(dtype)
+    qm = ac.QuantizationMethod(kind, group_size=128)
+    (qk, sk), (qv, sv) = qm.compress(X.to(dev), V.to(dev))
+    for x, q, s in ((X, qk, sk), (V, qv, sv)):
+        if kind == "int8":
+            rq, rs = oa.quantize_int8(x)
+            ref = oa.dequantize(rq, rs, dtype)
+        else:
+            rq, rs = (oa.quantize_int4 if kind == "int4" else oa.quantize_nf4)(x, 128)
+            ref = oa.dequantize_4bit(rq, rs, 128, kind == "nf4", dtype)
+        assert q.dtype == rq.dtype and q.shape == rq.shape and torch.equal(q.cpu(), rq)
+        assert s.dtype == dtype and s.shape == rs.shape and torch.equal(s.cpu(), rs)
+        got = qm.dequantize(q, s, dtype)
+        assert got.dtype == ref.dtype and torch.equal(got.cpu(), ref)
+    assert qm.name == f"quant_{kind}" and qm.compression_ratio == (2.0 if kind == "int8" else 4.0)
+    # several groups per row
+    if kind != "int8":
+        qm2 = ac.QuantizationMethod(kind, group_size=32)
+        q, s = qm2._quantize(X.to(dev))
+        rq, rs = (oa.quantize_int4 if kind == "int4" else oa.quantize_nf4)(X, 32)
+        assert s.shape == (2, 3, 50, 4) and torch.equal(q.cpu(), rq) and torch.equal(s.cpu(), rs)
+        assert torch.equal(qm2.dequantize(q, s, dtype).cpu(), oa.dequantize_4bit(rq, rs, 32, kind == "nf4", dtype))
+    with pytest.raises(FastcacheError):
+        ac.QuantizationMethod("fp8").compress(X.to(dev), V.to(dev))

@@ -136,3 +136,47 @@ def test_snapkv_extreme_logits(dev, boost, where):
     got = ops.snapkv_score(_lib.dense_view(dk), q.to(dev), W, ksz, causal_window=True, reduction="sum").cpu()
     assert torch.isfinite(got).all()
     torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-4 * float(ref.max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_tova_press(dev, dtype):
+    """Last-query attention averaged over all heads (computed from the window query, or taken from given attention
+    weights); scores <= 1e-3 relative, kept indices equal outside near-ties, the last token always kept."""
+    from fastcache_amd.presses import TOVAPress
+    from oracle import presses as opress
+    g = torch.Generator().manual_seed(3)
+    B, Hq, Hkv, S, D = 2, 8, 2, 700, 128
+    q = torch.randn(B, Hq, 1, D, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, S, D, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, S, D, generator=g).to(dtype)
+    press = TOVAPress(compression_ratio=0.6)
+    sc = press.score(None, None, k.to(dev), v.to(dev), None, {"queries": q.to(dev)})
+    ref = opress.tova_score(q, k)
+    assert sc.shape == (B, Hkv, S)
+    assert float(((sc.cpu() - ref).abs() / ref.abs().clamp_min(1e-12)).max()) <= 1e-3
+    ck, cv = press.compress(None, None, k.to(dev), v.to(dev), None, {"queries": q.to(dev)})
+    n = int(S * 0.4)
+    assert ck.shape == (B, Hkv, n, D)
+    idx = opress.topk_lowest_index(sc.cpu(), n)
+    assert bool((idx[..., -1] == S - 1).all())
+    assert torch.equal(ck.cpu(), opress.gather_tokens(k, idx)) and torch.equal(cv.cpu(), opress.gather_tokens(v, idx))
+    # attention weights handed in by the model
+    attn = torch.softmax(torch.randn(B, Hq, 5, S, generator=g), -1)
+    sc2 = press.score(None, None, k.to(dev), v.to(dev), attn.to(dev), {})
+    assert torch.allclose(sc2.cpu(), opress.tova_score(None, k, attentions=attn), rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hq,Hkv,S", [(2, 8, 2, 300), (1, 4, 4, 1025), (1, 2, 1, 64)])
+def test_observed_attention_press(dev, dtype, B, Hq, Hkv, S):
+    from fastcache_amd.presses import ObservedAttentionPress
+    from oracle import presses as opress
+    g = torch.Generator().manual_seed(S)
+    attn = torch.softmax(torch.randn(B, Hq, S, S, generator=g) + torch.triu(torch.full((S, S), -1e9), 1), -1).to(dtype)
+    k = torch.zeros(B, Hkv, S, 128, dtype=torch.float16)
+    sc = ObservedAttentionPress(0.5).score(None, None, k.to(dev), k.to(dev), attn.to(dev), {})
+    ref = opress.observed_attention_score(attn, Hkv)
+    assert sc.shape == (B, Hkv, S) and sc.dtype == torch.float32
+    assert float(((sc.cpu() - ref).abs() / ref.abs().clamp_min(1e-12)).max()) <= 1e-3
+    with pytest.raises(AssertionError):
+        ObservedAttentionPress(0.5).score(None, None, k.to(dev), k.to(dev), None, {})

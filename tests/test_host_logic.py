@@ -162,8 +162,10 @@ def test_press_objects_surface():
     assert SnapKVPress(0.75, window_in_budget=False).n_kept(4096) == 1088
     assert isinstance(press_select("anything else", 0.5), KnormPress)
     assert isinstance(press_select("StreamingLLM", 0.5), StreamingLLMPress)
+    from fastcache_amd.presses import TOVAPress
+    assert isinstance(press_select("TOVA", 0.5), TOVAPress)
     with pytest.raises(NotImplementedError):
-        press_select("TOVA", 0.5)
+        press_select("ExpectedAttention", 0.5)
     with pytest.raises(AssertionError):
         KnormPress(compression_ratio=1.0)
     # ratio 0 returns the inputs untouched without touching the device

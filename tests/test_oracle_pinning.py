@@ -366,3 +366,67 @@ def test_quantize_numpy_float16_steps_and_hand_rows():
     # range: the most negative code -qmax-1 is reachable only through clamping; 8 bits keeps [-128, 127]
     q, sc = oa.quantize(torch.tensor([[127.0, -127.0, 63.5]]), 8)
     assert sc.item() == 1.0 and q.tolist() == [[127, -127, 64]]
+
+
+def test_quantization_method_oracle_by_hand_and_numpy():
+    """oracle.autocompress.quantize_int8 / int4 / nf4 / dequantize_4bit: hand-worked groups and numpy float16 steps."""
+    from oracle import autocompress as oa
+    # int4, group of 4, fp32: max 7 -> scale 1; codes [7, -7, 0, 3] + 8 = [15, 1, 8, 11]
+    p, s = oa.quantize_int4(torch.tensor([[7.0, -6.6, 0.4, 2.6]]), 4)
+    assert s.tolist() == [[7.0 / 7.0]] and p.tolist() == [[15 | (1 << 4), 8 | (11 << 4)]]
+    assert oa.dequantize_4bit(p, s, 4, False, torch.float32).tolist() == [[7.0, -7.0, 0.0, 3.0]]
+    # nf4: scale = max|x| = 2; normalised [1, -1, 0, 0.3]; nearest levels: 15, 0, 7, 11 (0.3379 closer than 0.2461)
+    p, s = oa.quantize_nf4(torch.tensor([[2.0, -2.0, 0.0, 0.6]]), 4)
+    assert s.tolist() == [[2.0]] and p.tolist() == [[15 | (0 << 4), 7 | (11 << 4)]]
+    d = oa.dequantize_4bit(p, s, 4, True, torch.float32)
+    assert d.tolist() == [[2.0, -2.0, 0.0, 2.0 * float(torch.tensor(oa.NF4_LEVELS[11]))]]
+    # two groups per row get their own scales
+    x = torch.tensor([[1.0, -1.0, 14.0, 7.0]])
+    p, s = oa.quantize_int4(x, 2)
+    assert s.tolist() == [[float(np.float32(1.0) / np.float32(7.0)), 2.0]] and oa.dequantize_4bit(p, s, 2, False, torch.float32).tolist()[0][2:] == [14.0, 8.0]
+    # float16 steps with numpy
+    g = torch.Generator().manual_seed(3)
+    X = (torch.randn(5, 256, generator=g) * 2).half()
+    p, s = oa.quantize_int4(X, 128)
+    xn = X.numpy().reshape(-1, 128)
+    sc = (np.abs(xn).max(-1, keepdims=True).astype(np.float32) / np.float32(7)).astype(np.float16)
+    q = np.clip(np.rint((xn.astype(np.float32) / sc.astype(np.float32)).astype(np.float16).astype(np.float32)), -8, 7).astype(np.int32) + 8
+    assert np.array_equal(s.numpy().reshape(-1, 1), sc)
+    assert np.array_equal(p.numpy().reshape(-1), (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8).reshape(-1))
+    q8, s8 = oa.quantize_int8(X)
+    rq, rs = oa.quantize(X, 8)
+    assert torch.equal(q8, rq) and torch.equal(s8, rs)
+
+
+def test_tova_and_observed_attention_float64_loops():
+    """oracle.presses.tova_score / observed_attention_score against float64 loops."""
+    g = torch.Generator().manual_seed(12)
+    B, Hq, Hkv, S, D = 2, 4, 2, 9, 8
+    q = torch.randn(B, Hq, 1, D, generator=g)
+    k = torch.randn(B, Hkv, S, D, generator=g)
+    got = opress.tova_score(q, k)
+    G = Hq // Hkv
+    ref = np.zeros((B, Hkv, S))
+    for b in range(B):
+        acc = np.zeros(S)
+        for h in range(Hq):
+            lg = np.array([float((q[b, h, 0].double() * k[b, h // G, s].double()).sum()) / math.sqrt(D) for s in range(S)])
+            p = np.exp(lg - lg.max())
+            acc += p / p.sum()
+        acc /= Hq
+        ref[b, :, :S - 1] = acc[:S - 1]
+    ref[:, :, S - 1] = ref[:, :, :S - 1].max()
+    assert np.allclose(got.numpy(), ref, atol=1e-6)
+    # with attention weights given, the last query row is used as is
+    attn = torch.softmax(torch.randn(B, Hq, S, S, generator=g), -1)
+    got2 = opress.tova_score(None, k, attentions=attn)
+    assert torch.allclose(got2[:, 0, :S - 1], attn[:, :, -1, :-1].mean(1)) and torch.equal(got2[:, 0], got2[:, 1])
+    assert float(got2[0, 0, -1]) == float(got2[..., :S - 1].max())
+    obs = opress.observed_attention_score(attn, Hkv)
+    ref = np.zeros((B, Hkv, S))
+    for b in range(B):
+        for hk in range(Hkv):
+            for s in range(S):
+                tot = sum(float(attn[b, hk * G + gi, qi, s]) for gi in range(G) for qi in range(S))
+                ref[b, hk, s] = tot / (S - s) / G
+    assert np.allclose(obs.numpy(), ref, atol=1e-6)
