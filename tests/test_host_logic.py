@@ -284,3 +284,42 @@ def test_engine_sync_compression_after_prefill_and_preemption():
     sched.preempt(b)
     sched.running.remove(b)
     assert b.status == SequenceStatus.WAITING and not b.is_compressed and b.block_table == [] and sched.waiting[0] is b
+
+
+def test_checkpoint_layouts_round_trip(tmp_path):
+    """The three file layouts the reference's runner accepts load into a module with the reference's key names;
+    a file written by save_checkpoint has the training script's structure."""
+    from fastcache_amd.utils_ccm.checkpoint import (load_checkpoint, load_checkpoint_only_model, load_compressor_state,
+                                                    save_checkpoint)
+    torch.manual_seed(1)
+    src = KVCacheLinearDecoupleCompressor(llava_cfg(2, 2), compression_factor=2)
+    sd = {k: v.clone() for k, v in src.state_dict().items()}
+    assert "compress_tk.1.6.bias" in sd and "attention.0.weight" in sd
+    opt = torch.optim.SGD(src.parameters(), lr=0.1)
+    path = save_checkpoint(3, src, opt, None, 0.25, True, str(tmp_path), "c.pth")
+    assert path.endswith("last_c.pth") and (tmp_path / "best_c.pth").exists()
+    raw = torch.load(path, weights_only=True)
+    assert set(raw) == {"epoch", "model_state_dict", "optimizer_state_dict", "scheduler_state_dict", "loss"}
+    assert set(raw["model_state_dict"]) == {"compressor"}
+
+    def fresh():
+        torch.manual_seed(99)
+        return KVCacheLinearDecoupleCompressor(llava_cfg(2, 2), compression_factor=2)
+
+    m = fresh()
+    assert load_compressor_state(m, path) == ([], [])
+    assert all(torch.equal(v, sd[k]) for k, v in m.state_dict().items())
+    flat, bare = tmp_path / "flat.pth", tmp_path / "bare.pth"
+    partial = {k: v for k, v in sd.items() if not k.startswith("attention")}
+    torch.save({"model_state_dict": partial}, flat)
+    torch.save(dict(sd, extra=torch.zeros(1)), bare)
+    m = fresh()
+    missing, unexpected = load_compressor_state(m, str(flat))
+    assert sorted(missing) == sorted(k for k in sd if k.startswith("attention")) and unexpected == []
+    assert torch.equal(m.state_dict()["compress_iv.0.0.weight"], sd["compress_iv.0.0.weight"])
+    m = fresh()
+    assert load_compressor_state(m, str(bare)) == ([], ["extra"])
+    m = fresh()
+    assert load_checkpoint(m, torch.optim.SGD(m.parameters(), lr=0.1), None, path) == (3, 0.25)
+    assert load_checkpoint(m, filename=str(tmp_path / "nope.pth")) == (0, float("inf"))
+    assert load_checkpoint_only_model(fresh(), path) and not load_checkpoint_only_model(fresh(), str(tmp_path / "no.pth"))
