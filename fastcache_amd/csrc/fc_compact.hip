@@ -1,6 +1,6 @@
 // Gather/compaction of kept K/V rows, and plain ordered token copies.
 //
-// One workgroup per (K|V, layer, sequence, kv head) column.  A token row of one head is 128
+// One workgroup per (K|V, layer, sequence, kv head) column (per pair of heads for 512-byte fp32 rows).  A token row of one head is 128
 // elements (256 or 512 bytes) and is moved by 16 or 32 lanes with 16-byte accesses.  The column is
 // walked in ascending chunks: all source rows of a chunk are loaded into registers, the
 // workgroup waits for the loads and synchronises, and only then are the chunk's destination
@@ -33,7 +33,8 @@ __device__ __forceinline__ long long cp_offset(const KvView& v, const int* tbl, 
 // GATHER: src token = indices[j]; otherwise src token = src_start + j.
 // The column is walked in chunks of CH rows with two register buffers: the loads of chunk c+1 are
 // issued right after the barrier that releases the stores of chunk c, so loads and stores overlap.
-template <int EB, bool GATHER>
+// HG = consecutive kv heads handled by one workgroup (divides num_kv_heads)
+template <int EB, bool GATHER, int HG>
 __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView sv, KvView dk, KvView dv,
                                                              const int* __restrict__ indices,
                                                              int index_stride, int heads_in_index,
@@ -41,9 +42,9 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
                                                              int src_start, int dst_start) {
   constexpr int LPR = FC_HEAD_DIM * EB / 16;
   constexpr int RPP = CP_THREADS / LPR;
-  constexpr int CH = RPP * CP_R;
+  constexpr int CH = RPP * CP_R / HG;   // tokens per chunk
   __shared__ int stbl[CP_TBL], dtbl[CP_TBL];
-  const int h = blockIdx.x, b = blockIdx.y;
+  const int h0 = blockIdx.x * HG, b = blockIdx.y;
   const int L = sk.num_layers;
   const int l = blockIdx.z % L;
   const bool is_v = blockIdx.z >= L;
@@ -67,16 +68,21 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
       dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
   __syncthreads();
 
+  // rows of a chunk are (token j, head) pairs with the head fastest, so that the HG head rows of a
+  // token (contiguous in memory) are moved by neighbouring lanes
+  const int hh = rg % HG, h = h0 + hh;
   const int* idx = GATHER ? indices + (((long long)l * sk.batch + b) * heads_in_index + (h % heads_in_index)) *
                                           (long long)index_stride
                           : nullptr;
   const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * EB + sub * 16;
   char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * EB + sub * 16;
+  constexpr int TPP = RPP / HG;   // tokens per pass
+  const int tg = rg / HG;
 
   auto load_idx = [&](int (&si)[CP_R], int j0) {
 #pragma unroll
     for (int u = 0; u < CP_R; ++u) {
-      const int j = j0 + u * RPP + rg;
+      const int j = j0 + u * TPP + tg;
       si[u] = j < n ? (GATHER ? idx[j] : src_start + j) : -1;
     }
   };
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   auto store_rows = [&](const uint4 (&buf)[CP_R], const bool (&ok)[CP_R], int j0) {
 #pragma unroll
     for (int u = 0; u < CP_R; ++u) {
-      const int j = j0 + u * RPP + rg;
+      const int j = j0 + u * TPP + tg;
       if (ok[u]) {
         const long long off = cp_offset(dst, dtbl, d_lds, b, dst_start + j);
         if (off >= 0) *reinterpret_cast<uint4*>(dbase + off * EB) = buf[u];
@@ -153,14 +159,22 @@ extern "C" int fc_compact(const fc_kv_view* src_k, const fc_kv_view* src_v, cons
   FC_REQUIRE(src_k->num_layers * 2 <= 65535, FC_EUNSUPPORTED, "%s: too many layers", who);
   if (!n_kept && k == 0) return FC_OK;
   KvView sk = fc_make_view(src_k), sv = fc_make_view(src_v), dk = fc_make_view(dst_k), dv = fc_make_view(dst_v);
-  dim3 grid(src_k->num_kv_heads, src_k->batch, src_k->num_layers * 2);
   hipStream_t st = (hipStream_t)stream;
-  if (src_k->dtype == FC_F32)
-    hipLaunchKernelGGL((compact_kernel<4, true>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
+  // 512-byte (fp32) rows: two heads per workgroup measured faster, as long as the grid stays large
+  const long long cols = 2LL * src_k->num_layers * src_k->batch * src_k->num_kv_heads;
+  if (src_k->dtype == FC_F32 && src_k->num_kv_heads % 2 == 0 && cols >= 2048) {
+    dim3 grid(src_k->num_kv_heads / 2, src_k->batch, src_k->num_layers * 2);
+    hipLaunchKernelGGL((compact_kernel<4, true, 2>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
                        index_stride, heads_in_index, k, n_kept, 0, 0);
-  else
-    hipLaunchKernelGGL((compact_kernel<2, true>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
-                       index_stride, heads_in_index, k, n_kept, 0, 0);
+  } else {
+    dim3 grid(src_k->num_kv_heads, src_k->batch, src_k->num_layers * 2);
+    if (src_k->dtype == FC_F32)
+      hipLaunchKernelGGL((compact_kernel<4, true, 1>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
+                         index_stride, heads_in_index, k, n_kept, 0, 0);
+    else
+      hipLaunchKernelGGL((compact_kernel<2, true, 1>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
+                         index_stride, heads_in_index, k, n_kept, 0, 0);
+  }
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }
@@ -181,10 +195,10 @@ extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int3
   dim3 grid(src->num_kv_heads, src->batch, src->num_layers);
   hipStream_t st = (hipStream_t)stream;
   if (src->dtype == FC_F32)
-    hipLaunchKernelGGL((compact_kernel<4, false>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
+    hipLaunchKernelGGL((compact_kernel<4, false, 1>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
                        nullptr, seg_start, dst_start);
   else
-    hipLaunchKernelGGL((compact_kernel<2, false>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
+    hipLaunchKernelGGL((compact_kernel<2, false, 1>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
                        nullptr, seg_start, dst_start);
   FC_CHECK_LAUNCH(who);
   return FC_OK;
