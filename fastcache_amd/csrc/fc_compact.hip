@@ -10,16 +10,24 @@
 // touch disjoint bytes, so columns need no ordering between each other.
 #include "fc_common.h"
 
+typedef unsigned cp_u32x4 __attribute__((ext_vector_type(4)));   // native vector: arrays of it stay in registers
+
 #define CP_THREADS 256
 #ifndef CP_R
 #define CP_R 8      // 16-byte loads in flight per lane and chunk
 #endif
 #define CP_TBL 1024 // block-table entries of one sequence cached in LDS (per view)
 
-__device__ __forceinline__ void cp_wait_then_barrier() {
-  // the loaded registers are not consumed before the barrier, so wait for them explicitly
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
+// The loaded registers are not consumed before the barrier, so wait for them explicitly.  The stores
+// of the previous chunk were issued AFTER these loads; when every lane of the wavefront issued all
+// CP_R of them (stores_behind), the loads are complete as soon as at most CP_R operations are still
+// outstanding, and the stores' completion is not waited for.
+__device__ __forceinline__ void cp_wait_then_barrier(bool stores_behind) {
+  if (stores_behind)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CP_R) : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 __device__ __forceinline__ long long cp_offset(const KvView& v, const int* tbl, bool tbl_lds, int b, int s) {
@@ -86,48 +94,54 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
       si[u] = j < n ? (GATHER ? idx[j] : src_start + j) : -1;
     }
   };
-  auto load_rows = [&](uint4 (&buf)[CP_R], bool (&ok)[CP_R], const int (&si)[CP_R]) {
+  // Every lane always loads (rows that do not exist read the view's first bytes instead) and the validity
+  // goes into a bit mask: with no control flow around the buffer elements they stay in registers.
+  const char* safe = src.base + sub * 16;
+  auto load_rows = [&](cp_u32x4 (&buf)[CP_R], unsigned& ok, const int (&si)[CP_R]) {
+    ok = 0;
 #pragma unroll
     for (int u = 0; u < CP_R; ++u) {
-      ok[u] = false;
       const int s = si[u];
-      if (s >= 0 && s < S) {
-        const long long off = cp_offset(src, stbl, s_lds, b, s);
-        if (off >= 0) {
-          buf[u] = *reinterpret_cast<const uint4*>(sbase + off * EB);
-          ok[u] = true;
-        }
-      }
+      long long off = -1;
+      if (s >= 0 && s < S) off = cp_offset(src, stbl, s_lds, b, s);
+      const bool valid = off >= 0;
+      const char* p = valid ? sbase + off * EB : safe;
+      buf[u] = *reinterpret_cast<const cp_u32x4*>(p);
+      ok |= valid ? (1u << u) : 0u;
     }
   };
-  auto store_rows = [&](const uint4 (&buf)[CP_R], const bool (&ok)[CP_R], int j0) {
+  // returns whether every lane of this wavefront stored all CP_R rows
+  auto store_rows = [&](const cp_u32x4 (&buf)[CP_R], unsigned ok, int j0) {
+    bool all = true;
 #pragma unroll
     for (int u = 0; u < CP_R; ++u) {
       const int j = j0 + u * TPP + tg;
-      if (ok[u]) {
-        const long long off = cp_offset(dst, dtbl, d_lds, b, dst_start + j);
-        if (off >= 0) *reinterpret_cast<uint4*>(dbase + off * EB) = buf[u];
-      }
+      long long off = -1;
+      if (ok & (1u << u)) off = cp_offset(dst, dtbl, d_lds, b, dst_start + j);
+      if (off >= 0) *reinterpret_cast<cp_u32x4*>(dbase + off * EB) = buf[u];
+      all &= off >= 0;
     }
+    return (bool)__all(all);
   };
 
-  uint4 bufa[CP_R], bufb[CP_R];
-  bool oka[CP_R], okb[CP_R];
+  cp_u32x4 bufa[CP_R], bufb[CP_R];
+  unsigned oka, okb;
   int sia[CP_R], sib[CP_R];
   load_idx(sia, 0);
   load_rows(bufa, oka, sia);
   load_idx(sib, CH);
+  bool behind = false;   // the newest operations in flight are exactly CP_R stores of this wavefront
   for (int j0 = 0; j0 < n; j0 += 2 * CH) {
     // chunk j0 is in flight in buffer a; the indices of chunk j0 + CH are in sib
-    cp_wait_then_barrier();
+    cp_wait_then_barrier(behind);
     if (j0 + CH < n) load_rows(bufb, okb, sib);
     load_idx(sia, j0 + 2 * CH);
-    store_rows(bufa, oka, j0);
+    behind = store_rows(bufa, oka, j0);
     if (j0 + CH >= n) break;
-    cp_wait_then_barrier();
+    cp_wait_then_barrier(behind);
     if (j0 + 2 * CH < n) load_rows(bufa, oka, sia);
     load_idx(sib, j0 + 3 * CH);
-    store_rows(bufb, okb, j0 + CH);
+    behind = store_rows(bufb, okb, j0 + CH);
   }
 }
 
