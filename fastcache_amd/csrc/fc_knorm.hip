@@ -6,7 +6,7 @@
 // scores are staged in LDS so that each head's TS scores leave as one contiguous segment.
 #include "fc_common.h"
 
-#define KN_TS 32
+#define KN_TS 16   // tokens per workgroup tile: small enough that short caches still give thousands of workgroups
 #define KN_THREADS 256
 
 template <int DTYPE>
