@@ -409,12 +409,12 @@ WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkl
 # HBM-side bytes per launch of a workload's dominant kernel, from two rocprofv3 counter runs
 # (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter reads for the
 # copy workload below, whose traffic is known (512 MiB read, 512 MiB written):
-#   copy:   FETCH_SIZE 2.634e5 KiB -> scale 1.990;  WRITE_SIZE 5.269e5 KiB -> scale 0.995
+#   copy:   FETCH_SIZE 2.623e5 KiB -> scale 1.999;  WRITE_SIZE 5.244e5 KiB -> scale 1.000
 # The commands and raw readings are in profiles/*_hbm_traffic.txt.
-_FETCH_SCALE = 524288 / 2.634e5
-_WRITE_SCALE = 524288 / 5.269e5
+_FETCH_SCALE = 524288 / 2.623e5
+_WRITE_SCALE = 524288 / 5.244e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
-    "cfg2-snapkv-qwen3-8b": (2.491e6, 1.423e5),
+    "cfg2-snapkv-qwen3-8b": (2.391e6, 3.636e4),
 }
 
 
