@@ -58,9 +58,25 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
   for (int shift = 24; shift >= 0; shift -= 8) {
     hist[tid] = 0;  // TK_THREADS == 256 bins
     __syncthreads();
-    for (int i = tid; i < n; i += TK_THREADS) {
-      unsigned u = key_at(i);
-      if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
+    for (int i0 = 0; i0 < n; i0 += TK_THREADS) {
+      const int i = i0 + tid;
+      const unsigned u = i < n ? key_at(i) : 0u;
+      bool todo = i < n && (u & mask) == prefix;
+      const unsigned bin = (u >> shift) & 255u;
+      // Scores of one row share their leading bits, so most lanes of a wavefront hit the same bin in the
+      // first passes and their atomics would serialise: the two most common bins are counted with a
+      // ballot and one atomic each, what is left goes through per-lane atomics.
+#pragma unroll
+      for (int rep = 0; rep < 2; ++rep) {
+        const unsigned long long act = __ballot(todo);
+        if (act == 0ull) break;
+        const int leader = __ffsll((long long)act) - 1;
+        const unsigned lb = __shfl(bin, leader, 64);
+        const unsigned long long same = __ballot(todo && bin == lb);
+        if (lane == leader) atomicAdd(&hist[lb], (unsigned)__popcll(same));
+        todo = todo && bin != lb;
+      }
+      if (todo) atomicAdd(&hist[bin], 1u);
     }
     __syncthreads();
     // suffix sums over bins: thread t owns bin 255 - t
