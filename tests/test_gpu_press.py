@@ -85,6 +85,13 @@ def _oracle_snapkv_scores(case, W, ksz, causal, reduction):
     dict(num_layers=1, batch=2, num_q_heads=14, num_kv_heads=2, seq_len=1000, window=64, ksz=7, dtype=torch.bfloat16),
     dict(num_layers=1, batch=1, num_q_heads=8, num_kv_heads=1, seq_len=100, window=64, ksz=3, dtype=torch.bfloat16),
     dict(num_layers=1, batch=1, num_q_heads=2, num_kv_heads=1, seq_len=520, window=48, ksz=7, dtype=torch.float16),
+    # pages smaller than a key tile and pages whose size is no power of two: the per-row addressing path
+    dict(num_layers=2, batch=2, num_q_heads=8, num_kv_heads=2, seq_len=333, window=64, ksz=7, dtype=torch.bfloat16,
+         block_size=16),
+    dict(num_layers=1, batch=2, num_q_heads=4, num_kv_heads=2, seq_len=400, window=32, ksz=5, dtype=torch.float16,
+         block_size=48),
+    # a group of 16 row blocks (the widest workgroup)
+    dict(num_layers=1, batch=1, num_q_heads=8, num_kv_heads=1, seq_len=300, window=64, ksz=7, dtype=torch.bfloat16),
 ])
 @pytest.mark.parametrize("causal,reduction", [(True, "mean"), (False, "sum")])
 def test_snapkv_scores_and_selection(dev, cfg, causal, reduction):
