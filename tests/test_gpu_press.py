@@ -187,3 +187,23 @@ def test_observed_attention_press(dev, dtype, B, Hq, Hkv, S):
     assert float(((sc.cpu() - ref).abs() / ref.abs().clamp_min(1e-12)).max()) <= 1e-3
     with pytest.raises(AssertionError):
         ObservedAttentionPress(0.5).score(None, None, k.to(dev), k.to(dev), None, {})
+
+
+@pytest.mark.parametrize("S", [17, 33, 64, 65, 127, 128, 129, 192, 193, 255, 256, 257, 320, 321, 449])
+@pytest.mark.parametrize("W,ksz", [(16, 5), (1, 1), (33, 31)])
+def test_snapkv_short_sequences_and_tile_boundaries(dev, S, W, ksz):
+    """Sequence lengths around every key-tile boundary of the first five tiles (prologue, steady state and drain of
+    the tile pipeline), windows that are not multiples of 32, widest pooling kernels."""
+    if S <= W:
+        pytest.skip("needs S > W")
+    case = synth.snapkv_case(seed=S + W, num_layers=1, batch=2, num_q_heads=4, num_kv_heads=2, seq_len=S, window=W,
+                             keep_dense=True, dtype=torch.bfloat16)
+    ref = _oracle_snapkv_scores(case, W, ksz, True, "sum")
+    dk = case.dense_k.to(dev)
+    got = ops.snapkv_score(_lib.dense_view(dk), case.queries.to(dev), W, ksz, causal_window=True, reduction="sum").cpu()
+    torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-3 * float(ref.abs().mean()))
+    pool = case.kv_cache.to(dev)
+    tables, lens = case.table_tensor(dev), case.lens_tensor(dev)
+    got_p = ops.snapkv_score(_lib.paged_view(pool[0], tables, lens, S), case.queries.to(dev), W, ksz,
+                             causal_window=True, reduction="sum", seq_lens=lens).cpu()
+    assert torch.equal(got_p, got)
