@@ -2,12 +2,14 @@
 // and single-query paged attention (split over 256-token chunks, then merged).
 //
 // Attention is HBM-bound (one pass over K and V, ~1 FLOP per byte per query head), so the kernel is
-// organised around the loads: a token row of one kv head is 256 bytes and is read by 16 lanes with
-// one 16-byte load each, four rows in flight per lane.  A workgroup owns one (sequence, kv head,
-// 256-token chunk) and serves all query heads of the group from the same K/V bytes.
-//   phase 1  logits: per lane 8 products per query head, summed across the 16 lanes of a row;
-//   phase 2  chunk softmax statistics (max, sum of exp2) per query head;
-//   phase 3  sum of p * V rows, 8 output dims per lane, reduced over the 16 row slots of a pass.
+// organised around keeping loads in flight.  A workgroup owns one (sequence, kv head, 256-token
+// chunk) and serves all query heads of the group from the same K/V bytes; each of its four
+// wavefronts streams two 32-token K tiles and then the matching V tiles from global memory straight
+// into a private two-stage LDS ring (global_load_lds, rows XOR-swizzled), 16 KB per wavefront in
+// flight, no workgroup barrier between a load and its use.
+//   phase 1  logits: one v_mfma_f32_32x32x16 block per tile, query heads as (zero-padded) rows;
+//   phase 2  chunk softmax statistics (max, sum of exp2), one wavefront per query head;
+//   phase 3  sum of p * V rows from LDS, 8 output dims per lane, 16 partial sums folded through LDS.
 // Each chunk writes (max, sum, unnormalised output) to the workspace; a second kernel merges the
 // chunks of a sequence.  Grid sizes depend only on the view's max_seq_len, never on the lengths on
 // the device, so both launches can be replayed from a graph while the lengths grow.
@@ -37,159 +39,259 @@ __device__ __forceinline__ unsigned short da_pack(float f) {
   return DTYPE == FC_BF16 ? fc_float_to_bf16(f) : fc_float_to_half(f);
 }
 
-// GT = query heads served per workgroup (a tile of the group)
-template <int DTYPE, int GT>
-__global__ __launch_bounds__(DA_THREADS) void decode_attn_kernel(KvView kc, KvView vc, int layer,
-                                                                 const char* __restrict__ q, int Hq,
-                                                                 const int* __restrict__ lens, float c,
-                                                                 float* __restrict__ part_o,
-                                                                 float* __restrict__ part_ml, int max_splits) {
-  __shared__ float sc[GT][DA_CHUNK];
-  __shared__ float red[4][GT][FC_HEAD_DIM];
-  __shared__ float wred[2][GT][4];
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// Wave-wide maximum / sum with DPP steps inside each row of 16 lanes and four lane reads across the
+// rows; the result is wave-uniform.
+template <int CTRL>
+__device__ __forceinline__ float da_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float da_lane(float v, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+__device__ __forceinline__ float da_wave_max(float v) {
+  v = fmaxf(v, da_dpp<0xB1>(v));    // quad_perm [1,0,3,2]
+  v = fmaxf(v, da_dpp<0x4E>(v));    // quad_perm [2,3,0,1]
+  v = fmaxf(v, da_dpp<0x141>(v));   // row_half_mirror
+  v = fmaxf(v, da_dpp<0x140>(v));   // row_mirror
+  return fmaxf(fmaxf(da_lane(v, 0), da_lane(v, 16)), fmaxf(da_lane(v, 32), da_lane(v, 48)));
+}
+__device__ __forceinline__ float da_wave_sum(float v) {
+  v += da_dpp<0xB1>(v);
+  v += da_dpp<0x4E>(v);
+  v += da_dpp<0x141>(v);
+  v += da_dpp<0x140>(v);
+  return (da_lane(v, 0) + da_lane(v, 16)) + (da_lane(v, 32) + da_lane(v, 48));
+}
+
+#define DA_TILE 32                     // keys per tile: one MFMA block, 8 KB of K or V rows
+#define DA_TILEB (DA_TILE * 256)
+#define DA_RING (4 * 2 * DA_TILEB)     // four wavefronts, two stages each
+
+template <int GT>
+struct DaCfg {
+  // ring | logits / probabilities [GT][256]
+  static constexpr int LDS = DA_RING + GT * DA_CHUNK * 4;
+};
+
+// GT = query heads served per workgroup (a tile of the group, at most 8).
+// FAST = a 32-token tile never straddles two pages (dense view, or pages of 32*2^n tokens), so a tile
+// load is a wave-uniform base plus a per-lane offset.
+//
+// Wavefront w owns the key tiles w and w+4 of the chunk (32 tokens each) and streams them through
+// its private two-stage ring in LDS with global_load_lds: K tile a, K tile b, then V tile a and
+// V tile b into the same stages as soon as the logits of the K tile in them are done, so 16 KB per
+// wavefront are in flight for most of the kernel and no load waits behind a workgroup barrier.
+// Logits are one v_mfma_f32_32x32x16 block per tile with the query heads as rows (padded with zero
+// rows to 32): whatever the group size, K is read from LDS once.
+template <int DTYPE, int GT, bool FAST>
+__global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, KvView vc, int layer,
+                                                                    const char* __restrict__ q, int Hq,
+                                                                    const int* __restrict__ lens, float c,
+                                                                    float* __restrict__ part_o,
+                                                                    float* __restrict__ part_ml, int max_splits) {
+  extern __shared__ __align__(16) char smem[];
+  float(*sc)[DA_CHUNK] = reinterpret_cast<float(*)[DA_CHUNK]>(smem + DA_RING);
+  float(*red)[GT][FC_HEAD_DIM] = reinterpret_cast<float(*)[GT][FC_HEAD_DIM]>(smem);  // [16] partial outputs, reuses the ring
+  static_assert(16 * GT * FC_HEAD_DIM * 4 <= DA_RING, "partial outputs must fit in the ring");
 
   const int split = blockIdx.x, b = blockIdx.z;
   const int Hkv = kc.num_kv_heads;
   const int G = Hq / Hkv;
   const int gtiles = (G + GT - 1) / GT;
   const int h = blockIdx.y / gtiles, g0 = (blockIdx.y - h * gtiles) * GT;
-  int len = lens[b];
+  int len = __builtin_amdgcn_readfirstlane(lens[b]);
   len = min(len, kc.max_seq_len);
   const int t0 = split * DA_CHUNK;
   if (t0 >= len) return;
   const int ntok = min(DA_CHUNK, len - t0);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int sub = tid & 15, rg = tid >> 4;  // 16 lanes per row, 16 rows per pass
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int sub = lane & 15, rg = lane >> 4;   // V rows: 16 lanes per row, 4 rows per pass
 
-  float qf[GT][8];
+  // query heads as MFMA A-operand rows; rows past the group tile are zero
+  uint4 qf[8];
+  {
+    const bool ok = lrow < GT && g0 + lrow < G;
+    const char* qp = q + (((long long)b * Hq + (h * G + g0 + (ok ? lrow : 0))) * FC_HEAD_DIM + lhalf * 8) * 2;
 #pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    const int hq = h * G + g0 + g;
-    if (g0 + g < G) {
-      const uint4 x = *reinterpret_cast<const uint4*>(q + (((long long)b * Hq + hq) * FC_HEAD_DIM + sub * 8) * 2);
-      da_unpack8<DTYPE>(x, qf[g]);
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = ok ? *reinterpret_cast<const uint4*>(qp + ks * 32) : make_uint4(0, 0, 0, 0);
+  }
+
+  const char* kbase = kc.base + ((long long)layer * kc.stride_layer + (long long)h * kc.stride_head) * 2;
+  const char* vbase = vc.base + ((long long)layer * vc.stride_layer + (long long)h * vc.stride_head) * 2;
+  const unsigned ring_lds = __builtin_amdgcn_readfirstlane(fc_lds_addr(smem)) + wave * (2 * DA_TILEB);
+  char* ring = smem + wave * (2 * DA_TILEB);
+
+  // Tile `tile` of the chunk into this wavefront's stage: eight wave-loads of four rows.  Lane i
+  // writes LDS chunk i of the 64 chunks of those rows and fetches the global chunk (i & 15) ^ (row & 15)
+  // of row i / 16 (XOR swizzle, so that the operand reads of 32 rows at the same chunk fall on
+  // distinct banks).  Rows past the sequence end re-read its last row; their logits are masked.
+  auto issue = [&](const KvView& v, const char* base, int tile, int stage) {
+    const int s0 = t0 + tile * DA_TILE;
+    const unsigned dst = ring_lds + stage * DA_TILEB;
+    const int rmax = len - 1 - s0;
+    if constexpr (FAST) {
+      long long tb;
+      if (v.block_tables) {
+        const int blk = max(__builtin_amdgcn_readfirstlane(v.block_tables[(long long)b * v.table_stride + (s0 >> v.block_shift)]), 0);
+        tb = (long long)blk * v.stride_block + (long long)(s0 & (v.block_size - 1)) * v.stride_token;
+      } else {
+        tb = (long long)b * v.stride_batch + (long long)s0 * v.stride_token;
+      }
+      const char* g = base + tb * 2;
+      const unsigned tok_bytes = (unsigned)v.stride_token * 2;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int r = 4 * u + rg;
+        const unsigned lo = (unsigned)min(r, rmax) * tok_bytes + ((sub ^ (r & 15)) << 4);
+        fc_load_lds(g, lo, dst + u * 1024);
+      }
     } else {
+      long long off[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qf[g][e] = 0.f;
-    }
-  }
-
-  const char* kbase = kc.base + ((long long)layer * kc.stride_layer + (long long)h * kc.stride_head) * 2 + sub * 16;
-  const char* vbase = vc.base + ((long long)layer * vc.stride_layer + (long long)h * vc.stride_head) * 2 + sub * 16;
-
-  // ---- phase 1: logits ---------------------------------------------------------------------------
-  for (int p0 = 0; p0 < DA_CHUNK / 16; p0 += 4) {
-    uint4 kx[4];
-    bool ok[4];
+      for (int u = 0; u < 8; ++u) {
+        const int r = 4 * u + rg;
+        off[u] = fc_token_offset(v, b, s0 + min(r, rmax));
+        if (off[u] < 0) off[u] = 0;
+      }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = (p0 + u) * 16 + rg;
-      ok[u] = t < ntok;
-      kx[u] = make_uint4(0, 0, 0, 0);
-      if (ok[u]) {
-        const long long off = fc_token_offset(kc, b, t0 + t);
-        if (off >= 0) kx[u] = *reinterpret_cast<const uint4*>(kbase + off * 2);
+      for (int u = 0; u < 8; ++u) {
+        const int r = 4 * u + rg;
+        fc_load_lds(base + off[u] * 2 + ((sub ^ (r & 15)) << 4), dst + u * 1024);
       }
     }
+  };
+
+  const int tile_a = wave, tile_b = wave + 4;
+  const bool has_a = tile_a * DA_TILE < ntok, has_b = tile_b * DA_TILE < ntok;   // wave-uniform
+  if (has_a) issue(kc, kbase, tile_a, 0);
+  if (has_b) issue(kc, kbase, tile_b, 1);
+
+  // ---- phase 1: logits of this wavefront's tiles --------------------------------------------------
+  // C[head][key]: the lane owns key lrow of the tile and the heads (i/4)*8 + lhalf*4 + i%4, of which
+  // only heads < 8 exist, that is registers 0..3.
+  const unsigned xs = (unsigned)((lhalf ^ (lrow & 15)) << 4) + lrow * 256;
+  auto logits = [&](int tile, int stage) {
+    f32x16 acc;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float kf[8];
-      da_unpack8<DTYPE>(kx[u], kf);
-      const int t = (p0 + u) * 16 + rg;
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-      for (int g = 0; g < GT; ++g) {
-        float a = 0.f;
+    for (int ks = 0; ks < 8; ++ks) {
+      const uint4 kf = *reinterpret_cast<const uint4*>(ring + stage * DA_TILEB + (xs ^ (unsigned)(ks * 32)));
+      if constexpr (DTYPE == FC_BF16)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qf[ks]), __builtin_bit_cast(bf16x8, kf),
+                                                      acc, 0, 0, 0);
+      else
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, qf[ks]), __builtin_bit_cast(f16x8, kf),
+                                                     acc, 0, 0, 0);
+    }
+    const int t = tile * DA_TILE + lrow;
+    const bool live = t < ntok;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) a = fmaf(qf[g][e], kf[e], a);
-        a += __shfl_xor(a, 8, 64);
-        a += __shfl_xor(a, 4, 64);
-        a += __shfl_xor(a, 2, 64);
-        a += __shfl_xor(a, 1, 64);
-        if (sub == 0) sc[g][t] = ok[u] ? a * c : -INFINITY;
-      }
+    for (int i = 0; i < 4; ++i) {
+      const int g = lhalf * 4 + i;
+      if (g < GT) sc[g][t] = live ? acc[i] * c : -INFINITY;
+    }
+  };
+  auto no_logits = [&](int tile) {
+    for (int i = lane; i < GT * DA_TILE; i += 64) sc[i / DA_TILE][tile * DA_TILE + (i % DA_TILE)] = -INFINITY;
+  };
+  if (has_a) {
+    if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
+    logits(tile_a, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the stage's reads are done before V lands in it
+    issue(vc, vbase, tile_a, 0);
+  } else {
+    no_logits(tile_a);
+  }
+  if (has_b) {
+    fc_wait_vm<8>();   // K tile b has landed, V tile a may still be in flight
+    logits(tile_b, 1);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    issue(vc, vbase, tile_b, 1);
+  } else {
+    no_logits(tile_b);
+  }
+  fc_lds_barrier();
+
+  // ---- phase 2: chunk statistics, one wavefront per query head -------------------------------------
+  for (int g = wave; g < GT; g += 4) {
+    float x[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) x[j] = sc[g][lane + 64 * j];
+    const float m = da_wave_max(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float p = __builtin_amdgcn_exp2f(x[j] - m);   // exp2(-inf) = 0 for the padded slots
+      sc[g][lane + 64 * j] = p;
+      sum += p;
+    }
+    sum = da_wave_sum(sum);
+    if (lane == 0 && g0 + g < G) {
+      float* ml = part_ml + (((long long)b * Hq + (h * G + g0 + g)) * max_splits + split) * 2;
+      ml[0] = m;
+      ml[1] = sum;
     }
   }
-  __syncthreads();
+  fc_lds_barrier();
 
-  // ---- phase 2: chunk statistics -------------------------------------------------------------------
-  float mg[GT], lg[GT];
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    float m = fc_wave_max(sc[g][tid]);
-    if (lane == 0) wred[0][g][wave] = m;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    const float m = fmaxf(fmaxf(wred[0][g][0], wred[0][g][1]), fmaxf(wred[0][g][2], wred[0][g][3]));
-    mg[g] = m;
-    const float p = __builtin_amdgcn_exp2f(sc[g][tid] - m);  // exp2(-inf) = 0 for the padded slots
-    sc[g][tid] = p;
-    const float s = fc_wave_sum(p);
-    if (lane == 0) wred[1][g][wave] = s;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < GT; ++g) lg[g] = (wred[1][g][0] + wred[1][g][1]) + (wred[1][g][2] + wred[1][g][3]);
-
-  // ---- phase 3: sum of p * V ---------------------------------------------------------------------
+  // ---- phase 3: sum of p * V over this wavefront's tiles -------------------------------------------
   float acc[GT][8];
 #pragma unroll
   for (int g = 0; g < GT; ++g)
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-  for (int p0 = 0; p0 < DA_CHUNK / 16; p0 += 4) {
-    uint4 vx[4];
+  auto pv = [&](int tile, int stage) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = (p0 + u) * 16 + rg;
-      vx[u] = make_uint4(0, 0, 0, 0);
-      if (t < ntok) {
-        const long long off = fc_token_offset(vc, b, t0 + t);
-        if (off >= 0) vx[u] = *reinterpret_cast<const uint4*>(vbase + off * 2);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int p = 0; p < 8; ++p) {
+      const int r = 4 * p + rg;
+      const uint4 vx = *reinterpret_cast<const uint4*>(ring + stage * DA_TILEB + r * 256 + ((sub ^ (r & 15)) << 4));
       float vf[8];
-      da_unpack8<DTYPE>(vx[u], vf);
-      const int t = (p0 + u) * 16 + rg;
+      da_unpack8<DTYPE>(vx, vf);
 #pragma unroll
       for (int g = 0; g < GT; ++g) {
-        const float p = sc[g][t];
+        const float pr = sc[g][tile * DA_TILE + r];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(p, vf[e], acc[g][e]);
+        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e]);
       }
     }
+  };
+  if (has_a) {
+    if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
+    pv(tile_a, 0);
   }
-  // rows of a pass sit 16 lanes apart: fold the 4 row slots of this wavefront, then the 4 wavefronts
+  if (has_b) {
+    fc_wait_vm<0>();
+    pv(tile_b, 1);
+  }
+  fc_lds_barrier();   // every wavefront is done with its ring before the ring becomes `red`
+  // 16 partial outputs (4 wavefronts x 4 row slots) through LDS, summed in a fixed order
+  {
+    const int slot = wave * 4 + rg;
 #pragma unroll
-  for (int g = 0; g < GT; ++g)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float a = acc[g][e];
-      a += __shfl_xor(a, 16, 64);
-      a += __shfl_xor(a, 32, 64);
-      if (lane < 16) red[wave][g][sub * 8 + e] = a;
+    for (int g = 0; g < GT; ++g) {
+      float4* dst = reinterpret_cast<float4*>(&red[slot][g][sub * 8]);
+      dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+      dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
     }
-  __syncthreads();
+  }
+  fc_lds_barrier();
   for (int i = tid; i < GT * FC_HEAD_DIM; i += DA_THREADS) {
     const int g = i / FC_HEAD_DIM, d = i - g * FC_HEAD_DIM;
     if (g0 + g < G) {
-      const int hq = h * G + g0 + g;
-      const float o = (red[0][g][d] + red[1][g][d]) + (red[2][g][d] + red[3][g][d]);
-      part_o[(((long long)b * Hq + hq) * max_splits + split) * FC_HEAD_DIM + d] = o;
+      float o = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < 16; ++sl) o += red[sl][g][d];
+      part_o[(((long long)b * Hq + (h * G + g0 + g)) * max_splits + split) * FC_HEAD_DIM + d] = o;
     }
   }
-#pragma unroll
-  for (int g = 0; g < GT; ++g)
-    if (tid == g && g0 + g < G) {
-      const int hq = h * G + g0 + g;
-      float* ml = part_ml + (((long long)b * Hq + hq) * max_splits + split) * 2;
-      ml[0] = mg[g];
-      ml[1] = lg[g];
-    }
 }
 
 template <int DTYPE>
@@ -207,13 +309,31 @@ __global__ __launch_bounds__(FC_HEAD_DIM) void decode_merge_kernel(const float* 
   const int ns = (len + DA_CHUNK - 1) / DA_CHUNK;
   const float* ml = part_ml + ((long long)b * Hq + hq) * max_splits * 2;
   const float* po = part_o + ((long long)b * Hq + hq) * max_splits * FC_HEAD_DIM + d;
+  // eight splits per step so that their loads are in flight together
   float M = -INFINITY;
-  for (int s = 0; s < ns; ++s) M = fmaxf(M, ml[2 * s]);
+  for (int s0 = 0; s0 < ns; s0 += 8) {
+    float m[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m[j] = s0 + j < ns ? ml[2 * (s0 + j)] : -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) M = fmaxf(M, m[j]);
+  }
   float L = 0.f, acc = 0.f;
-  for (int s = 0; s < ns; ++s) {
-    const float w = __builtin_amdgcn_exp2f(ml[2 * s] - M);
-    L = fmaf(w, ml[2 * s + 1], L);
-    acc = fmaf(w, po[(long long)s * FC_HEAD_DIM], acc);
+  for (int s0 = 0; s0 < ns; s0 += 8) {
+    float m[8], l[8], x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool ok = s0 + j < ns;
+      m[j] = ok ? ml[2 * (s0 + j)] : -INFINITY;
+      l[j] = ok ? ml[2 * (s0 + j) + 1] : 0.f;
+      x[j] = ok ? po[(long long)(s0 + j) * FC_HEAD_DIM] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float w = __builtin_amdgcn_exp2f(m[j] - M);
+      L = fmaf(w, l[j], L);
+      acc = fmaf(w, x[j], acc);
+    }
   }
   *o = da_pack<DTYPE>(acc / L);
 }
@@ -349,18 +469,33 @@ extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cac
     const int gtiles = (G + gt - 1) / gt;
     FC_REQUIRE(Hkv * gtiles <= 65535 && B <= 65535, FC_EUNSUPPORTED, "%s: grid too large", who);
     dim3 grid(splits, Hkv * gtiles, B);
-#define DA_LAUNCH(DT, GTV)                                                                                         \
-  hipLaunchKernelGGL((decode_attn_kernel<DT, GTV>), grid, dim3(DA_THREADS), 0, st, k, v, layer, (const char*)q,   \
-                     num_q_heads, context_lens, c, part_o, part_ml, splits)
-#define DA_DISPATCH(DT)                         \
-  switch (gt) {                                 \
-    case 8: DA_LAUNCH(DT, 8); break;            \
-    case 4: DA_LAUNCH(DT, 4); break;            \
-    case 2: DA_LAUNCH(DT, 2); break;            \
-    default: DA_LAUNCH(DT, 1); break;           \
+    const auto tile_in_page = [](const fc_kv_view* v, const KvView& d) {
+      return v->block_tables == nullptr || (d.block_shift >= 5);
+    };
+    const bool fast = tile_in_page(k_cache, k) && tile_in_page(v_cache, v);
+#define DA_LAUNCH(DT, GTV, FA)                                                                                   \
+  do {                                                                                                          \
+    static bool attr_done = false;                                                                              \
+    if (!attr_done) {                                                                                           \
+      (void)hipFuncSetAttribute((const void*)decode_attn_kernel<DT, GTV, FA>,                                   \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, DaCfg<GTV>::LDS);                         \
+      attr_done = true;                                                                                         \
+    }                                                                                                           \
+    hipLaunchKernelGGL((decode_attn_kernel<DT, GTV, FA>), grid, dim3(DA_THREADS), DaCfg<GTV>::LDS, st, k, v,    \
+                       layer, (const char*)q, num_q_heads, context_lens, c, part_o, part_ml, splits);           \
+  } while (0)
+#define DA_DISPATCH2(DT, FA)                        \
+  switch (gt) {                                     \
+    case 8: DA_LAUNCH(DT, 8, FA); break;            \
+    case 4: DA_LAUNCH(DT, 4, FA); break;            \
+    case 2: DA_LAUNCH(DT, 2, FA); break;            \
+    default: DA_LAUNCH(DT, 1, FA); break;           \
   }
+#define DA_DISPATCH(DT) \
+  if (fast) { DA_DISPATCH2(DT, true) } else { DA_DISPATCH2(DT, false) }
     if (bf) { DA_DISPATCH(FC_BF16) } else { DA_DISPATCH(FC_F16) }
 #undef DA_DISPATCH
+#undef DA_DISPATCH2
 #undef DA_LAUNCH
     FC_CHECK_LAUNCH(who);
   }

@@ -124,4 +124,46 @@ __device__ __forceinline__ float fc_wave_max(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
   return v;
 }
+
+// ---- global memory -> LDS without register staging --------------------------------------------
+__device__ __forceinline__ unsigned fc_lds_addr(const void* p) {
+  return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16 (lds_base is
+// wave-uniform).  The load is counted in vmcnt; the compiler does not know it writes LDS, so
+// every consumer sits behind an explicit wait (fc_wait_barrier, fc_wait_vm).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void fc_load_lds(const char* g, unsigned lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
+               : "memory", "m0");
+}
+// same with a wave-uniform 64-bit base and a 32-bit per-lane byte offset
+__device__ __forceinline__ void fc_load_lds(const char* g_uniform, unsigned lane_off, unsigned lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_off),
+               "s"(g_uniform)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+// Wait until at most N vector-memory operations of this wave are outstanding and all its LDS
+// operations are done, then synchronise the workgroup.
+template <int N>
+__device__ __forceinline__ void fc_wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// Wait until at most N vector-memory operations of this wave are outstanding (no barrier).
+template <int N>
+__device__ __forceinline__ void fc_wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// All LDS operations of this wave done, then synchronise the workgroup; outstanding vector-memory
+// operations stay in flight.
+__device__ __forceinline__ void fc_lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 #endif  // __HIPCC__

@@ -51,36 +51,6 @@ __device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16
 
 __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ unsigned sk_lds_addr(const void* p) {
-  return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
-}
-
-// 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16 (lds_base is
-// wave-uniform).  The load is counted in vmcnt; the compiler does not know it writes LDS, so
-// every consumer sits behind sk_wait_barrier.
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void sk_load_lds(const char* g, unsigned lds_base) {
-  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
-               : "memory", "m0");
-}
-// same with a wave-uniform 64-bit base and a 32-bit per-lane byte offset
-__device__ __forceinline__ void sk_load_lds(const char* g_uniform, unsigned lane_off, unsigned lds_base) {
-  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_off),
-               "s"(g_uniform)
-               : "memory", "m0");
-}
-#pragma clang diagnostic pop
-
-// Wait until at most N vector-memory operations of this wave are outstanding and all its LDS
-// operations are done, then synchronise the workgroup.
-template <int N>
-__device__ __forceinline__ void sk_wait_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
-}
-
 // Sum over aligned groups of N consecutive lanes (N a power of two up to 16) with DPP adds in a
 // fixed order; every lane of a group ends up with the group's sum.
 template <int CTRL>
@@ -165,7 +135,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // clamped to its last row (every lane always loads, so the outstanding-load count is exact);
   // those keys are masked in sweep 1 and never emitted in sweep 2.
   const char* kbase = kv.base + ((long long)l * kv.stride_layer + (long long)h * kv.stride_head) * 2;
-  const unsigned kbuf_lds = __builtin_amdgcn_readfirstlane(sk_lds_addr(kbuf));
+  const unsigned kbuf_lds = __builtin_amdgcn_readfirstlane(fc_lds_addr(kbuf));
   // FAST: a tile lies inside one page (or the view is dense), so a load is a wave-uniform tile base
   // plus a per-lane byte offset; the offset is recomputed per load rather than kept in registers.
   const unsigned tok_bytes = (unsigned)kv.stride_token * 2;
@@ -187,7 +157,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
         asm volatile("" : "+v"(ln));
         const int r = 4 * (wave * LPW + u) + (ln >> 4);
         const unsigned lo = (unsigned)min(r, rmax) * tok_bytes + (((ln & 15) ^ (r & 15)) << 4);
-        sk_load_lds(g, lo, kbuf_lds + stage * SK_TILEB + (wave * LPW + u) * 1024);
+        fc_load_lds(g, lo, kbuf_lds + stage * SK_TILEB + (wave * LPW + u) * 1024);
       }
     } else {
 #pragma unroll 1
@@ -198,7 +168,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       const int s = min(tile * SK_KT + r, S - 1);
       long long off = fc_token_offset(kv, b, s);
       if (off < 0) off = 0;
-      sk_load_lds(kbase + off * 2 + ch * 16, kbuf_lds + stage * SK_TILEB + j * 1024);
+      fc_load_lds(kbase + off * 2 + ch * 16, kbuf_lds + stage * SK_TILEB + j * 1024);
     }
     }
   };
@@ -215,7 +185,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // top of a tile iteration: tile position m has landed for every wave, the stage consumed by the
   // previous iteration is free and receives position m+ST-1; returns the stage to read
   auto acquire = [&]() {
-    if (m + ST - 2 < 2 * T) sk_wait_barrier<LPW*(ST - 2)>(); else sk_wait_barrier<0>();
+    if (m + ST - 2 < 2 * T) fc_wait_barrier<LPW*(ST - 2)>(); else fc_wait_barrier<0>();
     const int nx = m + ST - 1;
     if (nx < 2 * T) issue(plan_tile(nx), (kc + ST - 1) % ST);
     return kc % ST;
@@ -341,7 +311,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     }
     const bool bad = !(lsq <= 3.0e38f);   // inf or NaN
     if (attempt == 1 || !__builtin_amdgcn_readfirstlane(__syncthreads_or(bad))) break;
-    sk_wait_barrier<0>();   // the tiles prefetched for sweep 2 land before their stages are reused
+    fc_wait_barrier<0>();   // the tiles prefetched for sweep 2 land before their stages are reused
     mref = SK_NEG;
     lsq = 0.f;
   }

@@ -46,6 +46,47 @@ def test_decode_attention(dev, dtype, Hq, Hkv, lens):
         assert float((got.cpu().float() - ref.float()).abs().max()) < 4e-3
 
 
+@pytest.mark.parametrize("block_size", [16, 32, 48, 64])
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 2)])
+def test_decode_attention_small_and_odd_pages(dev, block_size, Hq, Hkv):
+    """Pages smaller than a 32-token tile or of a size that is no power of two take the per-row
+    addressing path; pages of 32 and 64 tokens take the tile path with several pages per chunk."""
+    dtype, lens = torch.bfloat16, [1, 31, 32, 33, 255, 256, 257, 530]
+    B = len(lens)
+    case = synth.make_paged_case(seed=8, num_layers=1, batch=B, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype,
+                                 block_size=block_size)
+    q = torch.randn(B, Hq, 128, generator=torch.Generator().manual_seed(6)).to(dtype)
+    tables, lens_t = case.table_tensor("cpu"), torch.tensor(lens, dtype=torch.int32)
+    ref = oattn.decode_attention(q, case.kv_cache[0, 0], case.kv_cache[1, 0], lens_t, tables, 128 ** -0.5)
+    pool, tab_d = case.kv_cache.to(dev), tables.to(dev)
+    max_len = tables.shape[1] * block_size
+    kview, vview = (_lib.paged_view(pool[i], tab_d, None, max_len) for i in range(2))
+    ws = ops.decode_attn_workspace(B, Hq, max_len, dev)
+    got = ops.decode_attn(kview, vview, 0, q.to(dev), lens_t.to(dev), 128 ** -0.5, ws).cpu()
+    assert float((got.float() - ref.float()).abs().max()) < 4e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decode_attention_dense_view(dev, dtype):
+    """A HuggingFace-layout cache [B, Hkv, S, D] gives the same output as the same rows in pages."""
+    Hq, Hkv, lens = 8, 4, [700, 64, 385]
+    B, S = len(lens), max(lens)
+    case = synth.make_paged_case(seed=4, num_layers=1, batch=B, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype,
+                                 keep_dense=True)
+    q = torch.randn(B, Hq, 128, generator=torch.Generator().manual_seed(7)).to(dtype).to(dev)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device=dev)
+    dk, dv = case.dense_k[0].to(dev), case.dense_v[0].to(dev)    # rows past a sequence's length hold other data
+    ws = ops.decode_attn_workspace(B, Hq, S, dev)
+    got = ops.decode_attn(_lib.dense_view(dk), _lib.dense_view(dv), 0, q, lens_d, 128 ** -0.5, ws).cpu()
+    pool, tab = case.kv_cache.to(dev), case.table_tensor(dev)
+    ws2 = ops.decode_attn_workspace(B, Hq, tab.shape[1] * 256, dev)
+    paged = ops.decode_attn(_lib.paged_view(pool[0], tab, None, tab.shape[1] * 256),
+                            _lib.paged_view(pool[1], tab, None, tab.shape[1] * 256), 0, q, lens_d, 128 ** -0.5, ws2).cpu()
+    assert torch.equal(got, paged)
+    ref = oattn.decode_attention(q.cpu(), case.kv_cache[0, 0], case.kv_cache[1, 0], lens_d.cpu(), tab.cpu(), 128 ** -0.5)
+    assert float((got.float() - ref.float()).abs().max()) < 4e-3
+
+
 def test_block_permutation_invariance(dev):
     """Moving the pages around (with the table following) leaves the output bit-identical."""
     dtype, Hq, Hkv, lens = torch.float16, 8, 4, [900, 300, 77]
