@@ -5,7 +5,8 @@
 hot path over one batch of synthetic input that is already resident in HBM.  The default workload
 is configuration 2 (SnapKV press over a Qwen3-8B-shaped paged pool: score -> window fill -> top-k
 -> in-place compaction, all 36 layers, batch 8, 4096 tokens per sequence).  ``--workload`` selects
-the other configurations (knorm, ccm, decode, hybrid); they are measured the same way.
+the other configurations (knorm, ccm, decode, hybrid; decode-eager = the decode launches without a
+graph, for the profiler); they are measured the same way.
 
 Extra objects on the line:
   roofline      the dominant kernel of the workload: algorithmic bytes per launch divided by its
@@ -306,11 +307,12 @@ class DecodeWorkload(Workload):
     metric = "decode tokens/sec"
     unit = "tokens/s"
 
-    def __init__(self, seed, device, graph_steps=128):
+    def __init__(self, seed, device, graph_steps=128, eager=False):
         super().__init__()
         from fastcache_amd import synth
         from fastcache_amd.engine.decode_graph import DecodeGraph
         self.L, self.B, self.Hq, self.Hkv, self.T = 32, 90, 32, 32, graph_steps
+        self.eager = eager
         self.device = device
         self.case = synth.decode_case(seed=seed, steps=self.T, device=device, device_draw=True)
         self.tables = self.case.table_tensor(device)
@@ -321,7 +323,8 @@ class DecodeWorkload(Workload):
                                    dtype=torch.float32).to(torch.float16)
         self.dg = DecodeGraph(self.case.kv_cache, self.tables, self.lens, mk(self.Hq), mk(self.Hkv), mk(self.Hkv),
                               D ** -0.5)
-        self.dg.capture()
+        if not eager:
+            self.dg.capture()
         self.tokens_per_step = self.B * self.T
         sum_len = sum(self.case.seq_lens)
         e = 2
@@ -335,12 +338,16 @@ class DecodeWorkload(Workload):
     def config(self):
         return {"workload": self.name, "layers": self.L, "batch": self.B, "q_heads": self.Hq, "kv_heads": self.Hkv,
                 "head_dim": D, "context_lens": "uniform[128, 2048]", "sum_context_lens": sum(self.case.seq_lens),
-                "block_size": 256, "decode_steps_per_graph": self.T, "graph": "one hipGraph of all steps and layers"}
+                "block_size": 256, "decode_steps_per_graph": self.T,
+                "graph": "none (eager launches, for the profiler)" if self.eager else "one hipGraph of all steps and layers"}
 
     def step(self):
         self.lens.copy_(self.lens0)
         with self.br:
-            self.dg.replay()
+            if self.eager:
+                self.dg.run_eager()
+            else:
+                self.dg.replay()
 
     def cpu_baseline(self, budget_s=12.0):
         from oracle import attention as oattn
@@ -403,7 +410,9 @@ class CopyWorkload(Workload):
 
 
 WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
-             "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True)}
+             "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True),
+             # the decode launches without a graph, 4 steps per bracket: rocprofv3 cannot walk the 128-step graph
+             "decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True)}
 
 
 # HBM-side bytes per launch of a workload's dominant kernel, from two rocprofv3 counter runs

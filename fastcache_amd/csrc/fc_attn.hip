@@ -98,7 +98,12 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
   float(*red)[GT][FC_HEAD_DIM] = reinterpret_cast<float(*)[GT][FC_HEAD_DIM]>(smem);  // [16] partial outputs, reuses the ring
   static_assert(16 * GT * FC_HEAD_DIM * 4 <= DA_RING, "partial outputs must fit in the ring");
 
-  const int split = blockIdx.x, b = blockIdx.z;
+  // Workgroups go to the eight XCDs round-robin in launch order (blockIdx.x fastest).  With the chunk
+  // index taken straight from blockIdx.x and a multiple of eight chunks per sequence, each XCD would
+  // serve one chunk position of every sequence, and the late positions are mostly empty; rotating the
+  // chunk index by the head and sequence spreads the live chunks over all XCDs.
+  const int b = blockIdx.z;
+  const int split = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
   const int Hkv = kc.num_kv_heads;
   const int G = Hq / Hkv;
   const int gtiles = (G + GT - 1) / GT;
