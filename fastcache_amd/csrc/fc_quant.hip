@@ -1,4 +1,5 @@
-// Symmetric per-row quantisation of KV rows to int8 storage (4- or 8-bit range) and back.
+// Symmetric quantisation of KV rows: per-row int8 storage (4- or 8-bit range) and back, packed 4-bit
+// groups (integer and NF4), and quantise -> dequantise in one pass with a per-row or whole-tensor scale.
 //
 // One wavefront per row of `d` elements.  The arithmetic follows what a tensor library does on a
 // tensor of the row's dtype, step by step: every intermediate (row maximum, scale, quotient) is
@@ -146,6 +147,137 @@ __global__ __launch_bounds__(256) void dequantize_group4_kernel(const unsigned c
     qz_store<ODT>(out, base + 2 * j, lo * sc);
     qz_store<ODT>(out, base + 2 * j + 1, hi * sc);
   }
+}
+
+// ---- quantise -> dequantise in one pass ("fake quantisation") ---------------------------------------
+// y = clamp(round(x / scale), -qmax-1, qmax) * scale, scale = max|x| / qmax taken per row of d elements
+// or over the whole tensor; no floor on the scale (an all-zero row gives 0/0 = NaN, as the eager
+// expression does), NaN and infinities propagate the IEEE way.  Same rounding discipline as above.
+template <int DTYPE>
+__device__ __forceinline__ float qz_fake(float v, float sc, float qmax) {
+  float t = rintf(qz_round<DTYPE>(v / sc));
+  t = (t != t) ? t : fminf(fmaxf(t, -qmax - 1.f), qmax);   // clamp keeps NaN
+  return t * sc;
+}
+
+template <int DTYPE>
+__global__ __launch_bounds__(256) void fake_quant_rows_kernel(const char* __restrict__ x, long long rows, int d,
+                                                              float qmax, char* __restrict__ y,
+                                                              char* __restrict__ scale, char* __restrict__ absmax) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows) return;
+  const long long base = r * d;
+  float mx = 0.f;
+  bool has_nan = false;
+  for (int j = lane; j < d; j += 64) {
+    const float v = qz_load<DTYPE>(x, base + j);
+    has_nan |= v != v;
+    mx = fmaxf(mx, fabsf(v));
+  }
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mx = __builtin_nanf("");
+  const float sc = qz_round<DTYPE>(mx / qmax);
+  if (lane == 0) {
+    if (scale) qz_store<DTYPE>(scale, r, sc);
+    if (absmax) qz_store<DTYPE>(absmax, r, mx);
+  }
+  for (int j = lane; j < d; j += 64) qz_store<DTYPE>(y, base + j, qz_fake<DTYPE>(qz_load<DTYPE>(x, base + j), sc, qmax));
+}
+
+#define QZ_PARTS 1024   // partial maxima of the whole-tensor variant
+
+// largest |x| of this block's grid-stride share; NaN if it saw one
+template <int DTYPE>
+__global__ __launch_bounds__(256) void absmax_partial_kernel(const char* __restrict__ x, long long n,
+                                                             float* __restrict__ partial) {
+  __shared__ float wm[4];
+  float mx = 0.f;
+  bool has_nan = false;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const float v = qz_load<DTYPE>(x, i);
+    has_nan |= v != v;
+    mx = fmaxf(mx, fabsf(v));
+  }
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mx = __builtin_nanf("");
+  if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = wm[0];
+    for (int w = 1; w < 4; ++w) m = (m != m || wm[w] != wm[w]) ? __builtin_nanf("") : fmaxf(m, wm[w]);
+    partial[blockIdx.x] = m;
+  }
+}
+
+template <int DTYPE>
+__global__ __launch_bounds__(256) void fake_quant_tensor_kernel(const char* __restrict__ x, long long n,
+                                                                const float* __restrict__ partial, int nparts,
+                                                                float qmax, char* __restrict__ y,
+                                                                char* __restrict__ scale, char* __restrict__ absmax) {
+  __shared__ float wm[4];
+  float mx = 0.f;
+  bool has_nan = false;
+  for (int i = threadIdx.x; i < nparts; i += 256) {
+    const float v = partial[i];
+    has_nan |= v != v;
+    mx = fmaxf(mx, v);
+  }
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mx = __builtin_nanf("");
+  if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = wm[0];
+  for (int w = 1; w < 4; ++w) mx = (mx != mx || wm[w] != wm[w]) ? __builtin_nanf("") : fmaxf(mx, wm[w]);
+  const float sc = qz_round<DTYPE>(mx / qmax);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (scale) qz_store<DTYPE>(scale, 0, sc);
+    if (absmax) qz_store<DTYPE>(absmax, 0, mx);
+  }
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    qz_store<DTYPE>(y, i, qz_fake<DTYPE>(qz_load<DTYPE>(x, i), sc, qmax));
+}
+
+extern "C" int64_t fc_fake_quantize_workspace_bytes(void) { return QZ_PARTS * (int64_t)sizeof(float); }
+
+extern "C" int fc_fake_quantize(const void* x, void* y, int64_t rows, int32_t d, int32_t dtype, int32_t bits,
+                                int32_t per_tensor, void* scale, void* absmax, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+  const char* who = "fc_fake_quantize";
+  FC_REQUIRE(x && y, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(rows >= 0 && d > 0, FC_EINVAL, "%s: bad sizes rows=%lld d=%d", who, (long long)rows, d);
+  FC_REQUIRE(bits >= 2 && bits <= 16, FC_EINVAL, "%s: bits must be in [2, 16] (got %d)", who, bits);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (rows == 0) return FC_OK;
+  const float qmax = (float)((1 << (bits - 1)) - 1);
+  hipStream_t st = (hipStream_t)stream;
+  if (!per_tensor) {
+    const long long blocks = (rows + 3) / 4;
+    FC_REQUIRE(blocks <= 2147483647LL, FC_EUNSUPPORTED, "%s: too many rows", who);
+#define FQ(DT) hipLaunchKernelGGL((fake_quant_rows_kernel<DT>), dim3((unsigned)blocks), dim3(256), 0, st, (const char*)x, \
+                                  (long long)rows, d, qmax, (char*)y, (char*)scale, (char*)absmax)
+    if (dtype == FC_F32) FQ(FC_F32); else if (dtype == FC_F16) FQ(FC_F16); else FQ(FC_BF16);
+#undef FQ
+  } else {
+    FC_REQUIRE(workspace && workspace_bytes >= fc_fake_quantize_workspace_bytes(), FC_EINVAL,
+               "%s: the whole-tensor scale needs a workspace of %lld bytes", who,
+               (long long)fc_fake_quantize_workspace_bytes());
+    const long long n = rows * (long long)d;
+    const int nparts = (int)((n + 255) / 256 < QZ_PARTS ? (n + 255) / 256 : QZ_PARTS);
+    const long long want = (n + 1023) / 1024;
+    const unsigned blocks = (unsigned)(want < 8192 ? (want > 0 ? want : 1) : 8192);
+#define FT(DT)                                                                                                       \
+  do {                                                                                                               \
+    hipLaunchKernelGGL((absmax_partial_kernel<DT>), dim3(nparts), dim3(256), 0, st, (const char*)x, n,               \
+                       (float*)workspace);                                                                           \
+    hipLaunchKernelGGL((fake_quant_tensor_kernel<DT>), dim3(blocks), dim3(256), 0, st, (const char*)x, n,            \
+                       (const float*)workspace, nparts, qmax, (char*)y, (char*)scale, (char*)absmax);                \
+  } while (0)
+    if (dtype == FC_F32) FT(FC_F32); else if (dtype == FC_F16) FT(FC_F16); else FT(FC_BF16);
+#undef FT
+  }
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
 }
 
 extern "C" int fc_quantize_rows(const void* x, int64_t rows, int32_t d, int32_t dtype, int32_t bits, int8_t* q,

@@ -212,6 +212,33 @@ def dequantize_rows(q: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype) ->
     return out
 
 
+def fake_quantize(x: torch.Tensor, bits: int, per_tensor: bool, out: Optional[torch.Tensor] = None,
+                  return_params: bool = False):
+    """Quantise and dequantise in one pass: ``clamp(round(x / scale), -2^(bits-1), 2^(bits-1)-1) * scale`` with
+    ``scale = max|x| / (2^(bits-1)-1)`` over the last dimension, or over the whole tensor when ``per_tensor``.
+    With ``return_params`` also ``(scale, max|x|)`` shaped ``[..., 1]`` (or 0-dim for the whole-tensor form)."""
+    _lib.require_gpu(x, "x")
+    if x.dim() < 1 or x.numel() == 0:
+        raise FastcacheError("fake_quantize: empty input")
+    xc = x.contiguous()
+    d = xc.shape[-1]
+    rows = xc.numel() // d
+    y = torch.empty_like(xc) if out is None else out
+    if y.shape != xc.shape or y.dtype != xc.dtype or not y.is_contiguous():
+        raise FastcacheError("fake_quantize: out must be contiguous with the shape and dtype of x")
+    pshape = () if per_tensor else xc.shape[:-1] + (1,)
+    scale = torch.empty(pshape, dtype=x.dtype, device=x.device) if return_params else None
+    amax = torch.empty(pshape, dtype=x.dtype, device=x.device) if return_params else None
+    ws, nbytes = None, 0
+    if per_tensor:
+        nbytes = int(fn("fc_fake_quantize_workspace_bytes")())
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    check(fn("fc_fake_quantize")(xc.data_ptr(), y.data_ptr(), rows, d, _lib.dtype_code(x.dtype), bits,
+                                 int(bool(per_tensor)), _lib.ptr(scale), _lib.ptr(amax), _lib.ptr(ws), nbytes,
+                                 current_stream()), "fc_fake_quantize")
+    return (y, scale, amax) if return_params else y
+
+
 def quantize_group4(x: torch.Tensor, group_size: int, nf4: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     """Groups of ``group_size`` consecutive elements -> ``(packed uint8 [..., D/2], scale [..., D/group_size])``."""
     _lib.require_gpu(x, "x")

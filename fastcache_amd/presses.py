@@ -237,6 +237,65 @@ class RandomPress(ScorerPress):
         return torch.rand(keys.shape[:3], dtype=torch.float32, device=keys.device, generator=g)
 
 
+class SimpleKVQuantizer:
+    """Symmetric ``nbits`` quantise-dequantise of every K and V tensor of a cache with ONE scale per tensor
+    (utils_ccm/utils_compress.py:117-163).  Used as ``with quantizer(model) as q: q.quantize_cache(pkv)``."""
+
+    def __init__(self, nbits: int = 4):
+        self.nbits = nbits
+        self.totalTime = 0
+
+    def reset_timeCheck(self):
+        self.totalTime = 0
+
+    def __call__(self, model):
+        return self.QuantizeContext(self)
+
+    def _quantize_tensor(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.fake_quantize(x, self.nbits, per_tensor=True)
+
+    def quantize_cache(self, past_key_values):
+        return tuple((self._quantize_tensor(k), self._quantize_tensor(v)) for k, v in past_key_values)
+
+    class QuantizeContext:
+        def __init__(self, quantizer):
+            self.quantizer = quantizer
+
+        def __enter__(self):
+            return self.quantizer
+
+        def __exit__(self, exc_type, exc_val, exc_tb):
+            pass
+
+
+class ImprovedKVQuantizer(SimpleKVQuantizer):
+    """The same with one scale per row of the last dimension; the scales and row maxima of the last
+    ``quantize_cache`` are kept in ``cache['k_<layer>']`` / ``cache['v_<layer>']``
+    (utils_ccm/utils_compress.py:27-95)."""
+
+    def __init__(self, nbits: int = 4):
+        super().__init__(nbits)
+        self.cache = {}
+
+    def _quantize_tensor_with_params(self, x: torch.Tensor, key: str):
+        y, scale, max_val = ops.fake_quantize(x, self.nbits, per_tensor=False, return_params=True)
+        return y, {"scale": scale, "max_val": max_val}
+
+    def quantize_cache(self, past_key_values):
+        quantized = []
+        for layer_idx, (k, v) in enumerate(past_key_values):
+            k_scaled, self.cache[f"k_{layer_idx}"] = self._quantize_tensor_with_params(k, f"k_{layer_idx}")
+            v_scaled, self.cache[f"v_{layer_idx}"] = self._quantize_tensor_with_params(v, f"v_{layer_idx}")
+            quantized.append((k_scaled, v_scaled))
+        return tuple(quantized)
+
+    def dequantize_cache(self, quantized_cache):
+        """``x * scale`` with the stored scales, exactly as the reference does (its input is already
+        de-quantised, so this scales a second time)."""
+        return tuple((k * self.cache[f"k_{i}"]["scale"], v * self.cache[f"v_{i}"]["scale"])
+                     for i, (k, v) in enumerate(quantized_cache))
+
+
 # names the reference gives its timed subclasses (utils_compress.py:302-324)
 TOVAPressWithTime = TOVAPress
 ObservedAttentionPressWithTime = ObservedAttentionPress
@@ -247,8 +306,8 @@ RandomPressWithTime = RandomPress
 
 
 def press_select(compression_method: str = "Knorm", compression_ratio: float = 0.8) -> ScorerPress:
-    """utils_compress.py:327-349.  'ExpectedAttention' and 'Quantized' are not part of this build and
-    raise; any other name gives the Knorm press, as in the reference."""
+    """utils_compress.py:327-349.  'ExpectedAttention' is not part of this build and raises; 'Quantized' gives
+    the 4-bit ``SimpleKVQuantizer``; any other name gives the Knorm press, as in the reference."""
     if compression_method == "StreamingLLM":
         press = StreamingLLMPress(compression_ratio=compression_ratio)
     elif compression_method == "RandomPress":
@@ -257,9 +316,11 @@ def press_select(compression_method: str = "Knorm", compression_ratio: float = 0
         press = SnapKVPress(compression_ratio=compression_ratio)
     elif compression_method == "TOVA":
         press = TOVAPress(compression_ratio=compression_ratio)
-    elif compression_method in ("ExpectedAttention", "Quantized"):
+    elif compression_method == "Quantized":
+        return SimpleKVQuantizer(nbits=4)
+    elif compression_method == "ExpectedAttention":
         raise NotImplementedError(f"press '{compression_method}' is not part of this build (built: Knorm, SnapKV, "
-                                  "TOVA, ObservedAttention, StreamingLLM, RandomPress)")
+                                  "TOVA, ObservedAttention, StreamingLLM, RandomPress, Quantized)")
     else:
         press = KnormPress(compression_ratio=compression_ratio)
     press.reset_timeCheck()

@@ -212,6 +212,19 @@ int fc_quantize_rows(const void* x, int64_t rows, int32_t d, int32_t dtype, int3
 int fc_dequantize_rows(const int8_t* q, const void* scale, int64_t rows, int32_t d,
                        int32_t scale_dtype, int32_t out_dtype, void* out, void* stream);
 
+/* Quantise and dequantise in one pass ("fake quantisation"), x and y [rows][d] contiguous in `dtype`:
+ *   scale = max|x| / (2^(bits-1) - 1), per row or (per_tensor != 0) over the whole tensor;
+ *   y = clamp(round(x / scale), -2^(bits-1), 2^(bits-1) - 1) * scale,
+ * every step rounded to `dtype` as the eager tensor expression does, no floor on the scale (a zero
+ * row gives NaN, as there).  scale / absmax: optional outputs in `dtype`, [rows] or [1].  The
+ * whole-tensor form needs a workspace of fc_fake_quantize_workspace_bytes().  x == y is allowed.
+ * Replaces SimpleKVQuantizer._quantize_tensor (utils_ccm/utils_compress.py:144-154, whole-tensor
+ * scale) and ImprovedKVQuantizer._quantize_tensor_with_params (utils_compress.py:51-70, per row). */
+int64_t fc_fake_quantize_workspace_bytes(void);
+int fc_fake_quantize(const void* x, void* y, int64_t rows, int32_t d, int32_t dtype, int32_t bits,
+                     int32_t per_tensor, void* scale, void* absmax, void* workspace, int64_t workspace_bytes,
+                     void* stream);
+
 /*
  * 4-bit quantisation of groups of `group_size` consecutive elements, two codes per byte (element 2j in
  * the low nibble), one scale per group in the dtype of x.

@@ -227,3 +227,21 @@ def adapter_compress_layer(method: str, keys: torch.Tensor, values: torch.Tensor
     if idx is None:
         return keys.contiguous(), values.contiguous()
     return gather_tokens(keys, idx), gather_tokens(values, idx)
+
+
+# --------------------------------------------------------------------------------------------
+# quantise -> dequantise of a cache (SimpleKVQuantizer / ImprovedKVQuantizer)
+# --------------------------------------------------------------------------------------------
+def fake_quantize(x: torch.Tensor, nbits: int, per_tensor: bool):
+    """``SimpleKVQuantizer._quantize_tensor`` (utils_ccm/utils_compress.py:144-154, one scale for the whole
+    tensor) and ``ImprovedKVQuantizer._quantize_tensor_with_params`` (utils_compress.py:51-70, one scale per row
+    of the last dimension): the same eager tensor expression, in the dtype of ``x``.
+    Returns ``(x_dequant, scale, max_val)``."""
+    if per_tensor:
+        max_val = torch.max(torch.abs(x))
+    else:
+        max_val = torch.max(torch.abs(x), dim=-1, keepdim=True)[0]
+    scale = max_val / (2 ** (nbits - 1) - 1)
+    x_quant = torch.round(x / scale)
+    x_quant = torch.clamp(x_quant, -2 ** (nbits - 1), 2 ** (nbits - 1) - 1)
+    return x_quant * scale, scale, max_val

@@ -170,3 +170,61 @@ def test_quantization_method_bit_exact(dev, dtype, kind):
         assert torch.equal(qm2.dequantize(q, s, dtype).cpu(), oa.dequantize_4bit(rq, rs, 32, kind == "nf4", dtype))
     with pytest.raises(FastcacheError):
         ac.QuantizationMethod("fp8").compress(X.to(dev), V.to(dev))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("per_tensor", [False, True])
+def test_fake_quantize_bit_exact(dev, dtype, bits, per_tensor):
+    """fc_fake_quantize against the eager expression of SimpleKVQuantizer / ImprovedKVQuantizer, bit for bit."""
+    from oracle import presses as op
+    g = torch.Generator().manual_seed(31)
+    x = (torch.randn(2, 4, 300, 128, generator=g) * 2.5).to(dtype)
+    x[0, 1, 7] = 0                                       # an all-zero row: NaN per row, plain zeros per tensor
+    ref, rsc, rmx = op.fake_quantize(x, bits, per_tensor)
+    got, sc, mx = ops.fake_quantize(x.to(dev), bits, per_tensor, return_params=True)
+    assert torch.equal(torch.nan_to_num(sc.cpu().view(rsc.shape).float(), nan=-1), torch.nan_to_num(rsc.float(), nan=-1))
+    assert torch.equal(torch.nan_to_num(mx.cpu().view(rmx.shape).float(), nan=-1), torch.nan_to_num(rmx.float(), nan=-1))
+    assert torch.equal(torch.isnan(got.cpu()), torch.isnan(ref))
+    assert torch.equal(torch.nan_to_num(got.cpu().float(), nan=0.0), torch.nan_to_num(ref.float(), nan=0.0))
+    # in place
+    xd = x.to(dev).clone()
+    ops.fake_quantize(xd, bits, per_tensor, out=xd)
+    assert torch.equal(torch.nan_to_num(xd.cpu().float(), nan=0.0), torch.nan_to_num(ref.float(), nan=0.0))
+
+
+def test_fake_quantize_large_tensor_and_nan(dev):
+    """More elements than one pass of the partial maxima covers; a NaN anywhere poisons the whole-tensor scale."""
+    from oracle import presses as op
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 1024, 1024, generator=g).half()
+    x[2, 1000, 1000] = 40.0                               # the maximum sits near the end
+    ref = op.fake_quantize(x, 4, True)[0]
+    got = ops.fake_quantize(x.to(dev), 4, True).cpu()
+    assert torch.equal(got, ref)
+    x[1, 5, 5] = float("nan")
+    assert torch.isnan(ops.fake_quantize(x.to(dev), 4, True)).all()
+
+
+def test_kv_quantizer_objects(dev):
+    """SimpleKVQuantizer / ImprovedKVQuantizer: the reference's context-manager surface over a cache tuple."""
+    from fastcache_amd.presses import ImprovedKVQuantizer, SimpleKVQuantizer, press_select
+    from oracle import presses as op
+    g = torch.Generator().manual_seed(2)
+    pkv = tuple((torch.randn(1, 4, 50, 128, generator=g).bfloat16(), torch.randn(1, 4, 50, 128, generator=g).bfloat16())
+                for _ in range(3))
+    dev_pkv = tuple((k.to(dev), v.to(dev)) for k, v in pkv)
+    qz = press_select("Quantized")
+    assert isinstance(qz, SimpleKVQuantizer) and qz.nbits == 4
+    with qz(None) as q:
+        out = q.quantize_cache(dev_pkv)
+    for (k, v), (qk, qv) in zip(pkv, out):
+        assert torch.equal(qk.cpu(), op.fake_quantize(k, 4, True)[0]) and torch.equal(qv.cpu(), op.fake_quantize(v, 4, True)[0])
+    iq = ImprovedKVQuantizer(nbits=8)
+    out = iq.quantize_cache(dev_pkv)
+    for i, ((k, v), (qk, qv)) in enumerate(zip(pkv, out)):
+        rk, rs, rm = op.fake_quantize(k, 8, False)
+        assert torch.equal(qk.cpu(), rk) and torch.equal(iq.cache[f"k_{i}"]["scale"].cpu(), rs)
+        assert torch.equal(iq.cache[f"k_{i}"]["max_val"].cpu(), rm)
+    deq = iq.dequantize_cache(out)
+    assert torch.equal(deq[0][0].cpu(), out[0][0].cpu() * iq.cache["k_0"]["scale"].cpu())

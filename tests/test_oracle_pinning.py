@@ -430,3 +430,38 @@ def test_tova_and_observed_attention_float64_loops():
                 tot = sum(float(attn[b, hk * G + gi, qi, s]) for gi in range(G) for qi in range(S))
                 ref[b, hk, s] = tot / (S - s) / G
     assert np.allclose(obs.numpy(), ref, atol=1e-6)
+
+
+def test_fake_quantize_numpy_float16_steps_by_hand_and_idempotent():
+    """oracle.presses.fake_quantize (SimpleKVQuantizer / ImprovedKVQuantizer): step-by-step numpy float16
+    arithmetic, hand-worked rows, and idempotence (quantised values lie on the grid of the same scale)."""
+    from oracle import presses as op
+    # by hand, fp32, 4 bits: whole-tensor max 7 -> scale 1: [7, -3.5, 0.5, 2.4] -> [7, -4, 0, 2]
+    y, sc, mx = op.fake_quantize(torch.tensor([[7.0, -3.5], [0.5, 2.4]]), 4, True)
+    assert sc.item() == 1.0 and mx.item() == 7.0 and y.tolist() == [[7.0, -4.0], [0.0, 2.0]]
+    # per row: second row has its own max 2.8 -> scale 0.4: [0.5, 2.8] -> round([1.25, 7]) * 0.4 = [0.4, 2.8]
+    y, sc, mx = op.fake_quantize(torch.tensor([[7.0, -3.5], [0.5, 2.8]], dtype=torch.float64), 4, False)
+    assert y[0].tolist() == [7.0, -4.0] and abs(y[1, 0].item() - 0.4) < 1e-12 and abs(y[1, 1].item() - 2.8) < 1e-12
+    assert sc.shape == (2, 1) and mx[:, 0].tolist() == [7.0, 2.8]
+    # the negative bound -2^(n-1) is one step beyond -max: it is reachable only by rounding, never exceeded
+    y, _, _ = op.fake_quantize(torch.tensor([[-7.0, 7.0, -7.4]]), 4, False)       # max 7.4, scale 7.4/7
+    assert y.min().item() >= -8 * (7.4 / 7) - 1e-6
+    g = torch.Generator().manual_seed(12)
+    X = (torch.randn(5, 64, generator=g) * 3).half()
+    for bits in (4, 8):
+        qmax = 2 ** (bits - 1) - 1
+        for per_tensor in (False, True):
+            y, sc, mx = op.fake_quantize(X, bits, per_tensor)
+            xn = X.numpy()
+            mxn = np.abs(xn).max() if per_tensor else np.abs(xn).max(axis=-1, keepdims=True)
+            scn = (np.float32(mxn) / np.float32(qmax)).astype(np.float16)
+            quo = (xn.astype(np.float32) / scn.astype(np.float32)).astype(np.float16)
+            qn = np.clip(np.rint(quo.astype(np.float32)), -qmax - 1, qmax)
+            yn = (qn * scn.astype(np.float32)).astype(np.float16)
+            assert np.array_equal(np.asarray(sc.numpy()), scn) and np.array_equal(y.numpy(), yn)
+    # idempotence in fp64 (no rounding of the intermediate steps): the grid and its maximum do not move
+    Xd = torch.randn(4, 32, generator=g, dtype=torch.float64)
+    y1 = op.fake_quantize(Xd, 4, False)[0]
+    torch.testing.assert_close(op.fake_quantize(y1, 4, False)[0], y1, rtol=0, atol=1e-12)
+    # an all-zero row has scale 0 and comes out as NaN (0 / 0), as the eager expression gives
+    assert torch.isnan(op.fake_quantize(torch.zeros(1, 4), 4, False)[0]).all()
