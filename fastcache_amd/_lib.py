@@ -73,6 +73,8 @@ SIGNATURES = {
     "fc_fake_quantize": (C.c_int, [_VP, _VP, C.c_int64, _I, _I, _I, _I, _VP, _VP, _VP, C.c_int64, _VP]),
     "fc_quantize_group4": (C.c_int, [_VP, C.c_int64, _I, _I, _I, _VP, _VP, _VP]),
     "fc_dequantize_group4": (C.c_int, [_VP, _VP, C.c_int64, _I, _I, _I, _I, _VP, _VP]),
+    "fc_expected_attention_workspace_bytes": (C.c_int64, [_I, _I, _I, _I]),
+    "fc_expected_attention_score": (C.c_int, [_V, _V, _VP, _VP, _I, _I, _I, _F, _VP, _I, _VP, C.c_int64, _VP]),
     "fc_observed_attention_workspace_bytes": (C.c_int64, [_I, _I, _I]),
     "fc_observed_attention_score": (C.c_int, [_VP, _I, _I, _I, _I, _I, _I, _VP, _VP, C.c_int64, _VP]),
     "fc_copy_tokens": (C.c_int, [_V, _V, _I, _I, _I, _VP]),

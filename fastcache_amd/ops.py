@@ -162,6 +162,39 @@ def ccm_mlp(src: FcKvView, dst: FcKvView, weights: Tuple[torch.Tensor, ...], cf:
                            current_stream()), "fc_ccm_mlp")
 
 
+def expected_attention_score(keys: FcKvView, values: FcKvView, mean_query: torch.Tensor,
+                             cov_query: Optional[torch.Tensor], n_sink: int = 4, use_vnorm: bool = True,
+                             epsilon: float = 0.0, score_stride: Optional[int] = None) -> torch.Tensor:
+    """Expected attention of future queries ~ N(mean_query, cov_query) over the cached keys, scaled by the value
+    norms: ``[L, B, Hkv, score_stride]`` fp32.  mean_query ``[L, B, Hq, D]`` (or ``[B, Hq, D]`` for one layer),
+    cov_query ``[L, B, Hq, D, D]`` or None; both are converted to contiguous fp32."""
+    _lib.require_gpu(mean_query, "mean_query")
+    L, B, Hkv, S = keys.num_layers, keys.batch, keys.num_kv_heads, keys.max_seq_len
+    mu = mean_query.float().contiguous()
+    if mu.dim() == 3:
+        mu = mu.unsqueeze(0)
+    if mu.dim() != 4 or mu.shape[0] != L or mu.shape[1] != B or mu.shape[3] != keys.head_dim:
+        raise FastcacheError(f"mean_query must be [L={L}, B={B}, Hq, {keys.head_dim}], got {tuple(mean_query.shape)}")
+    Hq = mu.shape[2]
+    cov = None
+    if cov_query is not None:
+        cov = cov_query.float().contiguous()
+        if cov.dim() == 4:
+            cov = cov.unsqueeze(0)
+        if tuple(cov.shape) != (L, B, Hq, keys.head_dim, keys.head_dim):
+            raise FastcacheError(f"cov_query must be [L, B, Hq, D, D], got {tuple(cov_query.shape)}")
+    stride = S if score_stride is None else int(score_stride)
+    out = torch.empty((L, B, Hkv, stride), dtype=torch.float32, device=mu.device)
+    nbytes = int(fn("fc_expected_attention_workspace_bytes")(L, B, Hq, S))
+    if nbytes < 0:
+        raise FastcacheError("fc_expected_attention_workspace_bytes: bad arguments")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=mu.device)
+    check(fn("fc_expected_attention_score")(C.byref(keys), C.byref(values), mu.data_ptr(), _lib.ptr(cov), Hq,
+                                            int(n_sink), int(bool(use_vnorm)), float(epsilon), out.data_ptr(), stride,
+                                            ws.data_ptr(), nbytes, current_stream()), "fc_expected_attention_score")
+    return out
+
+
 def observed_attention_score(attentions: torch.Tensor, num_kv_heads: int) -> torch.Tensor:
     """fp32 ``[B, Hkv, Sk]`` from a materialised attention matrix ``[B, Hq, Sq, Sk]``: per key, the attention it
     received summed over the queries, divided by the number of queries that could see it, averaged over the group."""

@@ -210,6 +210,73 @@ class ObservedAttentionPress(ScorerPress):
 
 
 @dataclass
+class ExpectedAttentionPress(ScorerPress):
+    """Attention each key can expect from the next ``n_future_positions`` queries, whose distribution is taken
+    as Gaussian: its mean and covariance come from the prompt's hidden states through the attention module's
+    ``q_proj`` and the average rotary matrix of the future positions; the scores are scaled by the value norms
+    and the first ``n_sink`` tokens are always kept.  The statistics (a few matrix products on model tensors)
+    are computed with torch; the scoring over the cache runs in libfastcache_hip.  They can also be given
+    directly as ``kwargs['mean_query']`` ``[B, Hq, D]`` / ``kwargs['cov_query']`` ``[B, Hq, D, D]``."""
+    compression_ratio: float = 0.0
+    n_future_positions: int = 512
+    n_sink: int = 4
+    use_covariance: bool = True
+    use_vnorm: bool = True
+    epsilon: float = 0.0
+
+    def future_rotary(self, module, q_len: int, head_dim: int, device, kwargs):
+        """cos / sin ``[n_future, D]`` of positions ``q_len .. q_len + n_future_positions``: from the module's (or
+        ``kwargs['rotary_emb']``'s) rotary embedding when there is one, else plain RoPE with ``config.rope_theta``."""
+        pos = torch.arange(q_len, q_len + self.n_future_positions, device=device).unsqueeze(0)
+        rotary = getattr(module, "rotary_emb", None) or (kwargs or {}).get("rotary_emb")
+        if rotary is not None:
+            cos, sin = rotary(torch.zeros(1, 1, head_dim, device=device), pos)
+            return cos[0].float(), sin[0].float()
+        theta = float(getattr(getattr(module, "config", None), "rope_theta", 10000.0))
+        inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=device, dtype=torch.float32) / head_dim))
+        ang = pos[0].float()[:, None] * inv_freq[None, :]
+        emb = torch.cat((ang, ang), dim=-1)
+        return emb.cos(), emb.sin()
+
+    @torch.no_grad()
+    def get_query_statistics(self, module, hidden_states, kwargs=None):
+        bsz, q_len, _ = hidden_states.shape
+        n, d = module.config.num_attention_heads, module.head_dim
+        h = hidden_states[:, self.n_sink:].float()
+        Wq = module.q_proj.weight.float()
+        mean_h = h.mean(dim=1, keepdim=True)
+        mu = torch.matmul(mean_h, Wq.T).squeeze(1).view(bsz, n, d)
+        cov = None
+        if self.use_covariance:
+            hc = h - mean_h
+            cov_h = torch.matmul(hc.transpose(1, 2), hc) / hc.shape[1]
+            cov = torch.matmul(Wq, torch.matmul(cov_h, Wq.T)).view(bsz, n, d, n, d)
+            cov = cov.diagonal(dim1=1, dim2=3).permute(0, 3, 1, 2)
+        cos, sin = self.future_rotary(module, q_len, d, hidden_states.device, kwargs)
+        # average over the future positions of R = cos * I + sin * P, P = [[0, -I], [I, 0]] (rotate_half)
+        half = d // 2
+        R = torch.diag_embed(cos).mean(0)
+        sm = sin.mean(0)
+        R[half:, :half] += torch.diag(sm[:half])
+        R[:half, half:] -= torch.diag(sm[half:])
+        mu = torch.matmul(mu, R.T)
+        if cov is not None:
+            cov = torch.matmul(R, torch.matmul(cov, R.T))
+        return mu, cov
+
+    def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
+        assert keys.size(2) > self.n_sink, f"Input should contain more tokens than n_sink={self.n_sink}"
+        if kwargs is not None and kwargs.get("mean_query") is not None:
+            mu, cov = kwargs["mean_query"], kwargs.get("cov_query")
+        else:
+            mu, cov = self.get_query_statistics(module, hidden_states, kwargs)
+        if not self.use_covariance:
+            cov = None
+        return ops.expected_attention_score(_lib.dense_view(keys), _lib.dense_view(values), mu, cov, self.n_sink,
+                                            self.use_vnorm, self.epsilon)[0]
+
+
+@dataclass
 class StreamingLLMPress(ScorerPress):
     """Keep the first ``n_sink`` tokens and the most recent ones."""
     compression_ratio: float = 0.0
@@ -298,6 +365,7 @@ class ImprovedKVQuantizer(SimpleKVQuantizer):
 
 # names the reference gives its timed subclasses (utils_compress.py:302-324)
 TOVAPressWithTime = TOVAPress
+ExpectedAttentionPressWithTime = ExpectedAttentionPress
 ObservedAttentionPressWithTime = ObservedAttentionPress
 KnormPressWithTime = KnormPress
 SnapKVPressWithTime = SnapKVPress
@@ -306,8 +374,8 @@ RandomPressWithTime = RandomPress
 
 
 def press_select(compression_method: str = "Knorm", compression_ratio: float = 0.8) -> ScorerPress:
-    """utils_compress.py:327-349.  'ExpectedAttention' is not part of this build and raises; 'Quantized' gives
-    the 4-bit ``SimpleKVQuantizer``; any other name gives the Knorm press, as in the reference."""
+    """utils_compress.py:327-349: 'Quantized' gives the 4-bit ``SimpleKVQuantizer``; any name the reference does
+    not list gives the Knorm press, as there."""
     if compression_method == "StreamingLLM":
         press = StreamingLLMPress(compression_ratio=compression_ratio)
     elif compression_method == "RandomPress":
@@ -319,8 +387,7 @@ def press_select(compression_method: str = "Knorm", compression_ratio: float = 0
     elif compression_method == "Quantized":
         return SimpleKVQuantizer(nbits=4)
     elif compression_method == "ExpectedAttention":
-        raise NotImplementedError(f"press '{compression_method}' is not part of this build (built: Knorm, SnapKV, "
-                                  "TOVA, ObservedAttention, StreamingLLM, RandomPress, Quantized)")
+        press = ExpectedAttentionPress(compression_ratio=compression_ratio)
     else:
         press = KnormPress(compression_ratio=compression_ratio)
     press.reset_timeCheck()

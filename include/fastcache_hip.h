@@ -175,6 +175,26 @@ int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weight
                int32_t cf, int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream);
 
 /*
+ * Expected-attention scores: attention each key can expect from future queries whose distribution is
+ * Gaussian with mean mean_query[layer][b][hq][128] and covariance cov_query[layer][b][hq][128][128]
+ * (fp32, contiguous; cov_query may be NULL = mean only).  For the keys past the first n_sink of a sequence
+ *   z[hq][s] = mean . k_s / sqrt(128) + k_s^T cov k_s / (2 * 128),   p = softmax over those keys,
+ *   scores[layer][b][hk][s] = (mean over the query heads of group hk of p[.][s] + epsilon) * ||v_s||_2
+ * (without use_vnorm: the group mean alone); the first n_sink keys get the largest score of their layer;
+ * entries past a sequence's length are -inf.  fp16 / bf16 caches; scores fp32 with row stride
+ * score_stride >= max_seq_len.  workspace: fc_expected_attention_workspace_bytes bytes.
+ * Replaces ExpectedAttentionPress.score of the kvpress package as the reference uses it
+ * (utils_ccm/utils_compress.py:22-24, 315-316, 338-340); the query statistics themselves are computed by
+ * the host from the attention module's q_proj (model code, not part of the library).
+ */
+int64_t fc_expected_attention_workspace_bytes(int32_t num_layers, int32_t batch, int32_t num_q_heads,
+                                              int32_t max_seq_len);
+int fc_expected_attention_score(const fc_kv_view* keys, const fc_kv_view* values, const float* mean_query,
+                                const float* cov_query, int32_t num_q_heads, int32_t n_sink, int32_t use_vnorm,
+                                float epsilon, float* scores, int32_t score_stride, void* workspace,
+                                int64_t workspace_bytes, void* stream);
+
+/*
  * Observed-attention scores from a materialised attention matrix attn[batch][num_q_heads][sq][sk]
  * (fp32 / fp16 / bf16, contiguous):
  *   scores[b][hk][s] = mean over the query heads of kv group hk of (sum_q attn[b][h][q][s]) / (sk - s),

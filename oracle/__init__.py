@@ -19,6 +19,9 @@ Pinning status (what independent check fixes each restatement; see tests/test_or
   ccm.*                              float64 loops for Linear/ReLU chain, reshape by hand
   autocompress.linear_act / mlp_nobias   float64 loops with the rounding points made explicit
   autocompress.quantize / dequantize      numpy float16 arithmetic step by step, hand-worked rows
+  presses.expected_attention_*        float64 loops over tokens / keys for the statistics and the score, closed
+                                     forms (zero covariance, identity rotation); the kvpress package itself is
+                                     unavailable offline: PARITY UNPINNED beyond the published formula
   presses.fake_quantize               numpy float16 arithmetic step by step, hand-worked rows, idempotence
   blocks.*                           invariants of the free deque / ref counts, hand-worked cases
   attention.decode_attention         float64 loops; flash-attn itself is unavailable offline:

@@ -117,6 +117,63 @@ def tova_score(queries: Optional[torch.Tensor], keys: torch.Tensor, attentions: 
     return F.pad(scores, (0, 1), value=scores.max().item())
 
 
+def expected_attention_query_statistics(hidden_states: torch.Tensor, q_weight: torch.Tensor, num_heads: int,
+                                        head_dim: int, cos: torch.Tensor, sin: torch.Tensor, n_sink: int = 4,
+                                        use_covariance: bool = True):
+    """kvpress ``ExpectedAttentionPress.get_query_statistics`` (third party, restated from its published
+    description; PARITY UNPINNED): Gaussian statistics of the queries the next positions will produce.
+    ``hidden_states [B, S, hidden]`` (the first ``n_sink`` positions are left out as outliers), ``q_weight``
+    ``[num_heads * head_dim, hidden]`` (``q_proj.weight``), ``cos`` / ``sin`` ``[n_future, head_dim]`` of the
+    future positions.  mean = W mean(h); covariance = W cov(h) W^T, per-head diagonal blocks, population
+    normalisation; both are then rotated by the AVERAGE rotary matrix of the future positions.
+    Returns ``(mu [B, H, D], cov [B, H, D, D] or None)`` in fp32."""
+    bsz = hidden_states.shape[0]
+    n, d = num_heads, head_dim
+    h = hidden_states[:, n_sink:].float()
+    Wq = q_weight.float()
+    mean_h = h.mean(dim=1, keepdim=True)
+    mu = torch.matmul(mean_h, Wq.T).squeeze(1).view(bsz, n, d)
+    cov = None
+    if use_covariance:
+        hc = h - mean_h
+        cov_h = torch.matmul(hc.transpose(1, 2), hc) / hc.shape[1]
+        cov = torch.matmul(Wq, torch.matmul(cov_h, Wq.T))                       # [B, n*d, n*d]
+        cov = cov.view(bsz, n, d, n, d).diagonal(dim1=1, dim2=3)                # [B, d, d, n]
+        cov = cov.permute(0, 3, 1, 2)
+    # rotary matrix of one position: R = cos * I + sin * P with P = [[0, -I], [I, 0]], so that
+    # R q = q * cos + rotate_half(q) * sin
+    Id = torch.eye(d)
+    P = torch.zeros(d, d)
+    P[d // 2:, :d // 2], P[:d // 2, d // 2:] = torch.eye(d // 2), -torch.eye(d // 2)
+    R = cos.float().unsqueeze(1) * Id + sin.float().unsqueeze(1) * P                # [n_future, d, d]
+    R = R.mean(dim=0)
+    mu = torch.matmul(mu, R.T)
+    if use_covariance:
+        cov = torch.matmul(R, torch.matmul(cov, R.T))
+    return mu, cov
+
+
+def expected_attention_score(keys: torch.Tensor, values: torch.Tensor, mean_query: torch.Tensor,
+                             cov_query: Optional[torch.Tensor], n_sink: int = 4, use_vnorm: bool = True,
+                             epsilon: float = 0.0) -> torch.Tensor:
+    """kvpress ``ExpectedAttentionPress.score`` given the query statistics (third party; PARITY UNPINNED):
+    keys / values ``[B, Hkv, S, D]``, mean ``[B, Hq, D]``, covariance ``[B, Hq, D, D]`` -> ``[B, Hkv, S]`` fp32."""
+    assert keys.size(2) > n_sink
+    k = keys[:, :, n_sink:].float()
+    v = values[:, :, n_sink:].float()
+    bsz, Hkv, q_len, d = k.shape
+    G = mean_query.shape[1] // Hkv
+    kt = k.repeat_interleave(G, dim=1).transpose(2, 3)                            # [B, Hq, D, n]
+    scores = torch.matmul(mean_query.float().unsqueeze(2), kt).squeeze(2) / math.sqrt(d)
+    if cov_query is not None:
+        scores = scores + torch.einsum("bhin,bhij,bhjn->bhn", kt, cov_query.float(), kt) / d / 2
+    scores = F.softmax(scores, dim=-1)
+    scores = scores.view(bsz, Hkv, G, q_len).mean(dim=2)
+    if use_vnorm:
+        scores = (scores + epsilon) * v.norm(dim=-1)
+    return F.pad(scores, (n_sink, 0), value=scores.max().item())
+
+
 def observed_attention_score(attentions: torch.Tensor, num_kv_heads: int) -> torch.Tensor:
     """kvpress ``ObservedAttentionPress.score`` (third party; PARITY UNPINNED): attention received by each key
     summed over the queries, divided by the number of queries that can see the key, averaged over the group."""

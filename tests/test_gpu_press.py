@@ -173,6 +173,92 @@ def test_tova_press(dev, dtype):
     assert torch.allclose(sc2.cpu(), opress.tova_score(None, k, attentions=attn), rtol=1e-6, atol=0)
 
 
+def _ea_case(seed, B, Hq, Hkv, S, dtype):
+    g = torch.Generator().manual_seed(seed)
+    k = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    v = (torch.randn(B, Hkv, S, 128, generator=g) * torch.rand(B, Hkv, S, 1, generator=g) * 2).to(dtype)
+    mu = torch.randn(B, Hq, 128, generator=g) * 0.5
+    a = torch.randn(B, Hq, 128, 128, generator=g) / 128 ** 0.5
+    cov = a @ a.transpose(-1, -2) * 0.5                      # symmetric positive semi-definite
+    return k, v, mu, cov
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hq,Hkv,S", [(2, 8, 2, 700), (1, 4, 4, 2500), (1, 14, 2, 100), (2, 2, 2, 37)])
+@pytest.mark.parametrize("use_cov,use_vnorm,eps", [(True, True, 0.0), (False, True, 0.02), (True, False, 0.0)])
+def test_expected_attention_scores(dev, dtype, B, Hq, Hkv, S, use_cov, use_vnorm, eps):
+    """fc_expected_attention_score vs the oracle: scores <= 1e-3 relative (fp32 on both sides; the covariance is
+    split into two 16-bit halves on the device), sinks carry the layer maximum."""
+    from oracle import presses as opress
+    k, v, mu, cov = _ea_case(S + Hq, B, Hq, Hkv, S, dtype)
+    ref = opress.expected_attention_score(k, v, mu, cov if use_cov else None, 4, use_vnorm, eps)
+    kd, vd = k.to(dev), v.to(dev)                            # the views hold raw pointers: keep the tensors alive
+    got = ops.expected_attention_score(_lib.dense_view(kd), _lib.dense_view(vd), mu.to(dev),
+                                       cov.to(dev) if use_cov else None, 4, use_vnorm, eps)[0].cpu()
+    assert got.shape == (B, Hkv, S)
+    assert float(((got - ref).abs() / ref.abs().clamp_min(1e-9)).max()) <= 1e-3
+    assert bool((got[..., :4] == got.max()).all())
+
+
+def test_expected_attention_paged_ragged_and_layers(dev):
+    """Paged pool, two layers, ragged lengths: every (layer, sequence) equals the dense single-layer call; entries past
+    a sequence's length are -inf; the sink value is the layer's own maximum."""
+    dtype, L, Hq, Hkv, lens = torch.bfloat16, 2, 8, 2, [300, 40, 513]
+    B, S = len(lens), max(lens)
+    case = synth.make_paged_case(seed=9, num_layers=L, batch=B, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype,
+                                 keep_dense=True)
+    g = torch.Generator().manual_seed(4)
+    mu = torch.randn(L, B, Hq, 128, generator=g) * 0.5
+    a = torch.randn(L, B, Hq, 128, 128, generator=g) / 128 ** 0.5
+    cov = a @ a.transpose(-1, -2) * 0.5
+    pool, tab, lens_d = case.kv_cache.to(dev), case.table_tensor(dev), case.lens_tensor(dev)
+    kview, vview = (_lib.paged_view(pool[i], tab, lens_d, S) for i in range(2))
+    got = ops.expected_attention_score(kview, vview, mu.to(dev), cov.to(dev), 4, True, 0.0).cpu()
+    assert got.shape == (L, B, Hkv, S)
+    from oracle import presses as opress
+    for l in range(L):
+        per_seq = [opress.expected_attention_score(case.dense_k[l][b:b + 1, :, :n], case.dense_v[l][b:b + 1, :, :n],
+                                                   mu[l, b:b + 1], cov[l, b:b + 1], 4, True, 0.0)[0] for b, n in enumerate(lens)]
+        layer_max = max(float(p[:, 4:].max()) for p in per_seq)
+        for b, n in enumerate(lens):
+            ref = per_seq[b].clone()
+            ref[:, :4] = layer_max                       # one batched call shares the sink value across its sequences
+            assert float(((got[l, b, :, :n] - ref).abs() / ref.abs().clamp_min(1e-9)).max()) <= 1e-3
+            assert bool(torch.isinf(got[l, b, :, n:]).all()) and bool((got[l, b, :, n:] < 0).all())
+
+
+def test_expected_attention_press_from_module(dev):
+    """The press end to end on a stand-in attention module: query statistics from q_proj and the future rotary
+    angles (torch on the device) vs the oracle's statistics, then scores and the kept rows."""
+    from types import SimpleNamespace
+    from fastcache_amd.presses import ExpectedAttentionPress
+    from oracle import presses as opress
+    g = torch.Generator().manual_seed(8)
+    B, S, hidden, Hq, Hkv, D = 2, 260, 256, 4, 2, 128
+    q_proj = torch.nn.Linear(hidden, Hq * D, bias=False)
+    with torch.no_grad():
+        q_proj.weight.copy_(torch.randn(Hq * D, hidden, generator=g) / hidden ** 0.5)
+    module = SimpleNamespace(config=SimpleNamespace(num_attention_heads=Hq, rope_theta=10000.0), head_dim=D,
+                             q_proj=q_proj.to(dev))
+    hs = torch.randn(B, S, hidden, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, S, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, S, D, generator=g).bfloat16()
+    press = ExpectedAttentionPress(compression_ratio=0.5, n_future_positions=64)
+    mu, cov = press.get_query_statistics(module, hs.to(dev))
+    ang = torch.arange(S, S + 64, dtype=torch.float32)[:, None] * (1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D)))[None]
+    cos, sin = torch.cat((ang, ang), -1).cos(), torch.cat((ang, ang), -1).sin()
+    rmu, rcov = opress.expected_attention_query_statistics(hs, q_proj.weight.detach().cpu(), Hq, D, cos, sin, 4)
+    torch.testing.assert_close(mu.cpu(), rmu, rtol=2e-3, atol=2e-3)
+    torch.testing.assert_close(cov.cpu(), rcov, rtol=2e-3, atol=2e-3)
+    sc = press.score(module, hs.to(dev), k.to(dev), v.to(dev), None, {})
+    ref = opress.expected_attention_score(k, v, mu.cpu(), cov.cpu(), 4, True, 0.0)     # same statistics on both sides
+    assert float(((sc.cpu() - ref).abs() / ref.abs().clamp_min(1e-9)).max()) <= 1e-3
+    ck, cv = press.compress(module, hs.to(dev), k.to(dev), v.to(dev), None, {})
+    idx = opress.topk_lowest_index(sc.cpu(), S // 2)
+    assert bool((idx[..., :4] == torch.arange(4)).all())                                # sinks are kept
+    assert torch.equal(ck.cpu(), opress.gather_tokens(k, idx)) and torch.equal(cv.cpu(), opress.gather_tokens(v, idx))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,Hq,Hkv,S", [(2, 8, 2, 300), (1, 4, 4, 1025), (1, 2, 1, 64)])
 def test_observed_attention_press(dev, dtype, B, Hq, Hkv, S):

@@ -164,8 +164,11 @@ def test_press_objects_surface():
     assert isinstance(press_select("StreamingLLM", 0.5), StreamingLLMPress)
     from fastcache_amd.presses import TOVAPress
     assert isinstance(press_select("TOVA", 0.5), TOVAPress)
-    with pytest.raises(NotImplementedError):
-        press_select("ExpectedAttention", 0.5)
+    from fastcache_amd.presses import ExpectedAttentionPress, SimpleKVQuantizer
+    ea = press_select("ExpectedAttention", 0.5)
+    assert isinstance(ea, ExpectedAttentionPress) and (ea.n_future_positions, ea.n_sink, ea.use_covariance,
+                                                        ea.use_vnorm, ea.epsilon) == (512, 4, True, True, 0.0)
+    assert isinstance(press_select("Quantized"), SimpleKVQuantizer)
     with pytest.raises(AssertionError):
         KnormPress(compression_ratio=1.0)
     # ratio 0 returns the inputs untouched without touching the device

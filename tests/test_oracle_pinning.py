@@ -465,3 +465,56 @@ def test_fake_quantize_numpy_float16_steps_by_hand_and_idempotent():
     torch.testing.assert_close(op.fake_quantize(y1, 4, False)[0], y1, rtol=0, atol=1e-12)
     # an all-zero row has scale 0 and comes out as NaN (0 / 0), as the eager expression gives
     assert torch.isnan(op.fake_quantize(torch.zeros(1, 4), 4, False)[0]).all()
+
+
+def test_expected_attention_oracle_brute_force_and_closed_forms():
+    """oracle.presses.expected_attention_query_statistics / expected_attention_score against float64 loops that
+    never form the rotation matrix or the W cov W^T product, and against closed forms."""
+    from oracle import presses as op
+    g = torch.Generator().manual_seed(17)
+    B, S, hidden, H, D, n_sink, n_future = 2, 23, 24, 3, 8, 4, 6
+    hs = torch.randn(B, S, hidden, generator=g, dtype=torch.float64)
+    Wq = torch.randn(H * D, hidden, generator=g, dtype=torch.float64) / 4
+    ang = torch.arange(S, S + n_future, dtype=torch.float64)[:, None] * (1.0 / (100.0 ** (torch.arange(0, D, 2, dtype=torch.float64) / D)))[None]
+    cos, sin = torch.cat((ang, ang), -1).cos(), torch.cat((ang, ang), -1).sin()
+    mu, cov = op.expected_attention_query_statistics(hs, Wq, H, D, cos, sin, n_sink=n_sink)
+    # brute force: the query of every kept token at every future position, rotated with the rotate_half rule
+    x = torch.zeros(B, S - n_sink, H, D, dtype=torch.float64)
+    for b in range(B):
+        for t in range(n_sink, S):
+            q = (Wq @ hs[b, t]).view(H, D)
+            for p in range(n_future):
+                rot = torch.cat((-q[:, D // 2:], q[:, :D // 2]), -1)
+                x[b, t - n_sink] += (q * cos[p] + rot * sin[p]) / n_future
+    mu_bf = x.mean(1)
+    xc = x - mu_bf[:, None]
+    cov_bf = torch.einsum("bthi,bthj->bhij", xc, xc) / (S - n_sink)
+    torch.testing.assert_close(mu.double(), mu_bf, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(cov.double(), cov_bf, rtol=1e-4, atol=1e-5)
+    assert op.expected_attention_query_statistics(hs, Wq, H, D, cos, sin, n_sink=n_sink, use_covariance=False)[1] is None
+
+    # score: explicit loops over keys
+    Hkv, Sk = 1, 19
+    k = torch.randn(B, Hkv, Sk, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, Hkv, Sk, D, generator=g, dtype=torch.float64)
+    got = op.expected_attention_score(k, v, mu_bf, cov_bf, n_sink=n_sink, use_vnorm=True, epsilon=0.01)
+    ref = torch.zeros(B, Hkv, Sk, dtype=torch.float64)
+    for b in range(B):
+        ps = []
+        for hq in range(H):
+            z = torch.tensor([float(mu_bf[b, hq] @ k[b, 0, n]) / math.sqrt(D)
+                              + float(k[b, 0, n] @ cov_bf[b, hq] @ k[b, 0, n]) / (2 * D) for n in range(n_sink, Sk)],
+                             dtype=torch.float64)
+            e = torch.exp(z - z.max())
+            ps.append(e / e.sum())
+        mean_p = torch.stack(ps).mean(0)
+        ref[b, 0, n_sink:] = (mean_p + 0.01) * torch.sqrt((v[b, 0, n_sink:] ** 2).sum(-1))
+    ref[:, :, :n_sink] = ref.max()
+    torch.testing.assert_close(got.double(), ref, rtol=1e-4, atol=1e-7)
+    # closed form: zero mean and covariance -> uniform softmax, score = ||v|| / (S - n_sink); sinks get the maximum
+    z0 = op.expected_attention_score(k, v, torch.zeros(B, H, D), torch.zeros(B, H, D, D), n_sink=n_sink)
+    torch.testing.assert_close(z0[:, :, n_sink:].double(), v[:, :, n_sink:].norm(dim=-1) / (Sk - n_sink), rtol=1e-5, atol=0)
+    assert bool((z0[:, :, :n_sink] == z0.max()).all())
+    # without the value norm the scores of the scored keys sum to one per row
+    p = op.expected_attention_score(k, v, mu_bf, None, n_sink=n_sink, use_vnorm=False)
+    torch.testing.assert_close(p[:, :, n_sink:].sum(-1), torch.ones(B, Hkv), rtol=1e-5, atol=0)
