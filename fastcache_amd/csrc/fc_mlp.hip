@@ -44,6 +44,10 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 #define ML_ROWB 272                 // LDS bytes per weight row: 128 elements + 16 bytes of padding
 #define ML_WBYTES (128 * ML_ROWB)   // one 128 x 128 weight block in LDS
 #define ML_TBL 256                  // block-table entries cached per wavefront and view
+// Nothing is scheduled across this point.  Without it the compiler, short of registers, sinks every
+// prefetch (weight fragments from LDS, token rows from memory) to just before its use and the
+// multiplications wait out the full latency each time.
+#define ML_PIN() __builtin_amdgcn_sched_barrier(0)
 
 template <int DTYPE>
 __device__ __forceinline__ f32x16 ml_mfma(const uint4& a, const uint4& b, f32x16 c) {
@@ -126,7 +130,8 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   int* stbl = tbls + (wave * 2) * ML_TBL;
   int* dtbl = stbl + ML_TBL;
   const int s_last = seg_start + c_rows * cf - 1, d_last = dst_start + c_rows - 1;
-  if (col_ok && SRC_T == 1)
+  // also for a wavefront whose column is past the last one (b = 0): its loads are unconditional and need valid addresses
+  if (SRC_T == 1)
     for (int i = lane; i <= (s_last >> src.block_shift); i += 64) stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
   if (col_ok && DST_T == 1)
     for (int i = lane; i <= (d_last >> dst.block_shift); i += 64) dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
@@ -196,14 +201,17 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   auto x_load = [&](uint4 (&xf)[ML_TB][8], int q) {
     const int it = q / cf, kc = q - it * cf;
     const int row0 = it * rows_per_iter + sub * ML_ROWS;
+    // Every lane always loads (no branch around the loads, so that the compiler keeps exact counts of
+    // the loads in flight and the prefetch really overlaps the multiplications): rows past the end, a
+    // column past the last one (b = h = 0) and unallocated pages read some valid row instead; what is
+    // computed from them is never stored.
 #pragma unroll
     for (int tb = 0; tb < ML_TB; ++tb) {
-      const int r = row0 + tb * 32 + lrow;
-      long long off = -1;
-      if (col_ok && r < c_rows) off = src_off(seg_start + cf * r + kc);
+      const int r = min(row0 + tb * 32 + lrow, c_rows - 1);
+      long long off = src_off(seg_start + cf * r + kc);
+      off = off < 0 ? 0 : off;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-        xf[tb][ks] = off >= 0 ? *reinterpret_cast<const uint4*>(sbase + off * 2 + ks * 32) : make_uint4(0, 0, 0, 0);
+      for (int ks = 0; ks < 8; ++ks) xf[tb][ks] = *reinterpret_cast<const uint4*>(sbase + off * 2 + ks * 32);
     }
   };
 
@@ -224,6 +232,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
     // scratch memory): past the last chunk the X rows are out of range and load nothing, and the
     // extra W1 chunk lands in the buffer nobody reads again.
     x_load(xnext, q + XD);
+    ML_PIN();   // the prefetch stays ahead of this stage's multiplications
     if (!W1R) {
       __syncthreads();  // chunk q is in w1buf[q & 1]; every wavefront is done with chunk q - 1
       w1_load((kc + 1 < cf) ? kc + 1 : 0);
@@ -240,11 +249,13 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
           for (int mb = 0; mb < 4; ++mb)
             af[(ks + 1) & 1][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + (ks + 1) * 32);
         }
+        ML_PIN();   // the four reads of the next k-step are issued before this k-step's multiplications
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
           for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[tb][ks], acc[mb][tb]);
         }
+        ML_PIN();
       }
     }
     if (!W1R) w1_store((q + 1) & 1);
@@ -275,11 +286,13 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
           for (int mb = 0; mb < 4; ++mb)
             af[(g + 1) & 1][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + (g + 1) * 32);
         }
+        ML_PIN();
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
           for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = ml_mfma<DTYPE>(af[g & 1][mb], hf[tb][g], acc[mb][tb]);
         }
+        ML_PIN();
       }
     }
     // ---- layer 3: Y = H2 * W3^T, A operand taken from layer 2's accumulators ---------------------
@@ -310,11 +323,13 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
           for (int nb = 0; nb < 4; ++nb)
             bfr[(g + 1) & 1][nb] = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB + (g + 1) * 32);
         }
+        ML_PIN();
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
 #pragma unroll
           for (int tb = 0; tb < ML_TB; ++tb) acc[nb][tb] = ml_mfma<DTYPE>(hf[tb][g], bfr[g & 1][nb], acc[nb][tb]);
         }
+        ML_PIN();
       }
     }
     // every wavefront of the column has consumed this iteration's source rows: stores may alias them
