@@ -8,15 +8,15 @@
 
 #define KN_TS 16   // tokens per workgroup tile: small enough that short caches still give thousands of workgroups
 #define KN_THREADS 256
+#define KN_U 4     // rows per lane and pass
 
+// sum of squares of the 16 bytes a lane holds of its row
 template <int DTYPE>
-__device__ __forceinline__ float row_sumsq_part(const char* p) {
-  // p points at this lane's 16 bytes of the row
+__device__ __forceinline__ float row_sumsq_part(const uint4& x) {
   if (DTYPE == FC_F32) {
-    float4 x = *reinterpret_cast<const float4*>(p);
-    return x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    const float a = __uint_as_float(x.x), b = __uint_as_float(x.y), c = __uint_as_float(x.z), d = __uint_as_float(x.w);
+    return a * a + b * b + c * c + d * d;
   } else {
-    uint4 x = *reinterpret_cast<const uint4*>(p);
     unsigned w[4] = {x.x, x.y, x.z, x.w};
     float acc = 0.f;
 #pragma unroll
@@ -34,6 +34,19 @@ __device__ __forceinline__ float row_sumsq_part(const char* p) {
     }
     return acc;
   }
+}
+
+// sum over an aligned group of 16 lanes (DPP, fixed order); every lane gets the sum
+template <int CTRL>
+__device__ __forceinline__ float kn_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float kn_sum16(float v) {
+  v += kn_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+  v += kn_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+  v += kn_dpp<0x141>(v);   // row_half_mirror
+  v += kn_dpp<0x140>(v);   // row_mirror
+  return v;
 }
 
 template <int DTYPE>
@@ -62,31 +75,38 @@ __global__ __launch_bounds__(KN_THREADS) void knorm_kernel(KvView kv, float* __r
   const bool head_fast = kv.stride_head <= kv.stride_token;
   const char* base = kv.base + (long long)l * kv.stride_layer * EB;
 
+  // KN_U rows per lane and pass: all their loads are issued (unconditionally, a dead row re-reads a
+  // valid one) before the first is reduced, so that a lane keeps several 16-byte loads in flight.
   const int rows = KN_TS * H;
-  for (int r0 = 0; r0 < rows; r0 += RPP) {
-    int r = r0 + rg;
-    float part = 0.f;
-    int t = 0, h = 0;
-    bool live = false;
-    if (r < rows) {
-      if (head_fast) { t = r / H; h = r - t * H; } else { h = r / KN_TS; t = r - h * KN_TS; }
-      int s = s0 + t;
-      if (s < S) {
-        long long off = fc_token_offset(kv, b, s);
-        if (off >= 0) {
-          live = true;
-          part = row_sumsq_part<DTYPE>(base + (off + (long long)h * kv.stride_head) * EB + sub * 16);
-        }
-      }
+  for (int r0 = 0; r0 < rows; r0 += RPP * KN_U) {
+    uint4 x[KN_U];
+    bool live[KN_U];
+    int tt[KN_U], hh[KN_U];
+#pragma unroll
+    for (int u = 0; u < KN_U; ++u) {
+      const int r = r0 + u * RPP + rg;
+      const int rc = min(r, rows - 1);
+      int t, h;
+      if (head_fast) { t = rc / H; h = rc - t * H; } else { h = rc / KN_TS; t = rc - h * KN_TS; }
+      const int s = s0 + t;
+      long long off = fc_token_offset(kv, b, max(min(s, S - 1), 0));
+      live[u] = r < rows && s < S && off >= 0;
+      off = off < 0 ? 0 : off;
+      tt[u] = t;
+      hh[u] = h;
+      x[u] = *reinterpret_cast<const uint4*>(base + (off + (long long)h * kv.stride_head) * EB + sub * 16);
     }
 #pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-    if (r < rows && sub == 0) {
-      float v;
-      if (!live) v = -INFINITY;
-      else if (MEAN) v = round_to_storage<DTYPE>(sqrtf(part));
-      else v = -sqrtf(part);
-      sc[h * (KN_TS + 1) + t] = v;
+    for (int u = 0; u < KN_U; ++u) {
+      float part = kn_sum16(row_sumsq_part<DTYPE>(x[u]));
+      if (LPR == 32) part += __shfl_xor(part, 16, 64);
+      if (r0 + u * RPP + rg < rows && sub == 0) {
+        float v;
+        if (!live[u]) v = -INFINITY;
+        else if (MEAN) v = round_to_storage<DTYPE>(sqrtf(part));
+        else v = -sqrtf(part);
+        sc[hh[u] * (KN_TS + 1) + tt[u]] = v;
+      }
     }
   }
   __syncthreads();
