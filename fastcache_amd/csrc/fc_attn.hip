@@ -9,7 +9,8 @@
 // flight, no workgroup barrier between a load and its use.
 //   phase 1  logits: one v_mfma_f32_32x32x16 block per tile, query heads as (zero-padded) rows;
 //   phase 2  chunk softmax statistics (max, sum of exp2), one wavefront per query head;
-//   phase 3  sum of p * V rows from LDS, 8 output dims per lane, 16 partial sums folded through LDS.
+//   phase 3  sum of p * V rows from LDS: on the VALU, 8 output dims per lane, 16 partial sums folded through
+//            LDS; for 8 heads per workgroup on the matrix pipe with V read transposed from LDS;
 // Each chunk writes (max, sum, unnormalised output) to the workspace; a second kernel merges the
 // chunks of a sequence.  Grid sizes depend only on the view's max_seq_len, never on the lengths on
 // the device, so both launches can be replayed from a graph while the lengths grow.
@@ -67,13 +68,16 @@ __device__ __forceinline__ float da_wave_sum(float v) {
   return (da_lane(v, 0) + da_lane(v, 16)) + (da_lane(v, 32) + da_lane(v, 48));
 }
 
+#define DA_PV_MFMA_MIN 8               // heads per workgroup from which p * V runs on the matrix pipe (measured: no gain below)
 #define DA_TILE 32                     // keys per tile: one MFMA block, 8 KB of K or V rows
 #define DA_TILEB (DA_TILE * 256)
 #define DA_RING (4 * 2 * DA_TILEB)     // four wavefronts, two stages each
 
 template <int GT>
 struct DaCfg {
-  // ring | logits / probabilities [GT][256]
+  // ring | logits, then probabilities [GT][256]: fp32, or with eight heads (p * V on the matrix pipe) each
+  // probability as two 16-bit halves hi + lo in the cache dtype
+  static constexpr bool PV_MFMA = GT >= DA_PV_MFMA_MIN;
   static constexpr int LDS = DA_RING + GT * DA_CHUNK * 4;
 };
 
@@ -95,6 +99,8 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
                                                                     float* __restrict__ part_ml, int max_splits) {
   extern __shared__ __align__(16) char smem[];
   float(*sc)[DA_CHUNK] = reinterpret_cast<float(*)[DA_CHUNK]>(smem + DA_RING);
+  unsigned(*p2)[DA_CHUNK] = reinterpret_cast<unsigned(*)[DA_CHUNK]>(smem + DA_RING);   // sc seen as (hi, lo) pairs
+  constexpr bool PV_MFMA = DaCfg<GT>::PV_MFMA;
   float(*red)[GT][FC_HEAD_DIM] = reinterpret_cast<float(*)[GT][FC_HEAD_DIM]>(smem);  // [16] partial outputs, reuses the ring
   static_assert(16 * GT * FC_HEAD_DIM * 4 <= DA_RING, "partial outputs must fit in the ring");
 
@@ -235,7 +241,13 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float p = __builtin_amdgcn_exp2f(x[j] - m);   // exp2(-inf) = 0 for the padded slots
-      sc[g][lane + 64 * j] = p;
+      if constexpr (PV_MFMA) {
+        const unsigned short hi = da_pack<DTYPE>(p);
+        const float hf = DTYPE == FC_BF16 ? fc_bf16_to_float(hi) : fc_half_to_float(hi);
+        p2[g][lane + 64 * j] = (unsigned)hi | ((unsigned)da_pack<DTYPE>(p - hf) << 16);
+      } else {
+        sc[g][lane + 64 * j] = p;
+      }
       sum += p;
     }
     sum = da_wave_sum(sum);
@@ -248,53 +260,133 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
   fc_lds_barrier();
 
   // ---- phase 3: sum of p * V over this wavefront's tiles -------------------------------------------
-  float acc[GT][8];
+  if constexpr (PV_MFMA) {
+    // O[head][d] = P[head][key] * V[key][d] on the matrix pipe.  A = P rows from LDS (8 consecutive keys per
+    // lane), as two operands hi and lo so that the probabilities keep ~16-22 mantissa bits; the B operand
+    // wants 8 consecutive KEYS of one output dimension per lane, i.e. V transposed, which is read as
+    // 2-byte pieces from the swizzled rows (lanes of a half-wave read neighbouring dimensions of one row,
+    // the two half-waves rows 8 apart whose chunks are swizzled onto other banks).
+    f32x16 oacc[4];
 #pragma unroll
-  for (int g = 0; g < GT; ++g)
+    for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-  auto pv = [&](int tile, int stage) {
+      for (int i = 0; i < 16; ++i) oacc[nb][i] = 0.f;
+    auto pv = [&](int tile, int stage) {
+      const char* vt = ring + stage * DA_TILEB + (lrow & 7) * 2;
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int r = 4 * p + rg;
-      const uint4 vx = *reinterpret_cast<const uint4*>(ring + stage * DA_TILEB + r * 256 + ((sub ^ (r & 15)) << 4));
-      float vf[8];
-      da_unpack8<DTYPE>(vx, vf);
+      for (int s = 0; s < 2; ++s) {
+        const int k0 = s * 16 + lhalf * 8;   // first of this lane's 8 keys of the k-step
+        uint4 a = make_uint4(0, 0, 0, 0), a2 = make_uint4(0, 0, 0, 0);
+        if (lrow < GT) {
+          const uint4 d0 = *reinterpret_cast<const uint4*>(&p2[lrow][tile * DA_TILE + k0]);
+          const uint4 d1 = *reinterpret_cast<const uint4*>(&p2[lrow][tile * DA_TILE + k0 + 4]);
+          // v_perm_b32 bytes: 0-3 second operand, 4-7 first operand
+          a = make_uint4(__builtin_amdgcn_perm(d0.y, d0.x, 0x05040100u), __builtin_amdgcn_perm(d0.w, d0.z, 0x05040100u),
+                         __builtin_amdgcn_perm(d1.y, d1.x, 0x05040100u), __builtin_amdgcn_perm(d1.w, d1.z, 0x05040100u));
+          a2 = make_uint4(__builtin_amdgcn_perm(d0.y, d0.x, 0x07060302u), __builtin_amdgcn_perm(d0.w, d0.z, 0x07060302u),
+                          __builtin_amdgcn_perm(d1.y, d1.x, 0x07060302u), __builtin_amdgcn_perm(d1.w, d1.z, 0x07060302u));
+        }
 #pragma unroll
-      for (int g = 0; g < GT; ++g) {
-        const float pr = sc[g][tile * DA_TILE + r];
+        for (int nb = 0; nb < 4; ++nb) {
+          const int chunk = nb * 4 + (lrow >> 3);
+          unsigned w[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e]);
+          for (int e2 = 0; e2 < 4; ++e2) {
+            const int ka = k0 + 2 * e2, kb = ka + 1;
+            const unsigned lo = *reinterpret_cast<const unsigned short*>(vt + ka * 256 + ((chunk ^ (ka & 15)) << 4));
+            const unsigned hi = *reinterpret_cast<const unsigned short*>(vt + kb * 256 + ((chunk ^ (kb & 15)) << 4));
+            w[e2] = lo | (hi << 16);
+          }
+          const uint4 bfrag = make_uint4(w[0], w[1], w[2], w[3]);
+          if constexpr (DTYPE == FC_BF16) {
+            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                               __builtin_bit_cast(bf16x8, bfrag), oacc[nb], 0, 0, 0);
+            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a2),
+                                                               __builtin_bit_cast(bf16x8, bfrag), oacc[nb], 0, 0, 0);
+          } else {
+            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                              __builtin_bit_cast(f16x8, bfrag), oacc[nb], 0, 0, 0);
+            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a2),
+                                                              __builtin_bit_cast(f16x8, bfrag), oacc[nb], 0, 0, 0);
+          }
+        }
+      }
+    };
+    if (has_a) {
+      if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
+      pv(tile_a, 0);
+    }
+    if (has_b) {
+      fc_wait_vm<0>();
+      pv(tile_b, 1);
+    }
+    fc_lds_barrier();   // every wavefront is done with its ring before the ring becomes `red`
+    // C layout: the lane holds output dimension nb*32 + lrow of the heads lhalf*4 + i (registers 0..3)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int g = lhalf * 4 + i;
+      if (g < GT) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) red[wave][g][nb * 32 + lrow] = oacc[nb][i];
       }
     }
-  };
-  if (has_a) {
-    if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
-    pv(tile_a, 0);
-  }
-  if (has_b) {
-    fc_wait_vm<0>();
-    pv(tile_b, 1);
-  }
-  fc_lds_barrier();   // every wavefront is done with its ring before the ring becomes `red`
-  // 16 partial outputs (4 wavefronts x 4 row slots) through LDS, summed in a fixed order
-  {
-    const int slot = wave * 4 + rg;
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      float4* dst = reinterpret_cast<float4*>(&red[slot][g][sub * 8]);
-      dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
-      dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+    fc_lds_barrier();
+    for (int i = tid; i < GT * FC_HEAD_DIM; i += DA_THREADS) {
+      const int g = i / FC_HEAD_DIM, d = i - g * FC_HEAD_DIM;
+      if (g0 + g < G) {
+        const float o = (red[0][g][d] + red[1][g][d]) + (red[2][g][d] + red[3][g][d]);
+        part_o[(((long long)b * Hq + (h * G + g0 + g)) * max_splits + split) * FC_HEAD_DIM + d] = o;
+      }
     }
-  }
-  fc_lds_barrier();
-  for (int i = tid; i < GT * FC_HEAD_DIM; i += DA_THREADS) {
-    const int g = i / FC_HEAD_DIM, d = i - g * FC_HEAD_DIM;
-    if (g0 + g < G) {
-      float o = 0.f;
+  } else {
+    float acc[GT][8];
 #pragma unroll
-      for (int sl = 0; sl < 16; ++sl) o += red[sl][g][d];
-      part_o[(((long long)b * Hq + (h * G + g0 + g)) * max_splits + split) * FC_HEAD_DIM + d] = o;
+    for (int g = 0; g < GT; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    auto pv = [&](int tile, int stage) {
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const int r = 4 * p + rg;
+        const uint4 vx = *reinterpret_cast<const uint4*>(ring + stage * DA_TILEB + r * 256 + ((sub ^ (r & 15)) << 4));
+        float vf[8];
+        da_unpack8<DTYPE>(vx, vf);
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          const float pr = sc[g][tile * DA_TILE + r];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e]);
+        }
+      }
+    };
+    if (has_a) {
+      if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
+      pv(tile_a, 0);
+    }
+    if (has_b) {
+      fc_wait_vm<0>();
+      pv(tile_b, 1);
+    }
+    fc_lds_barrier();   // every wavefront is done with its ring before the ring becomes `red`
+    // 16 partial outputs (4 wavefronts x 4 row slots) through LDS, summed in a fixed order
+    {
+      const int slot = wave * 4 + rg;
+#pragma unroll
+      for (int g = 0; g < GT; ++g) {
+        float4* dst = reinterpret_cast<float4*>(&red[slot][g][sub * 8]);
+        dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+        dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+      }
+    }
+    fc_lds_barrier();
+    for (int i = tid; i < GT * FC_HEAD_DIM; i += DA_THREADS) {
+      const int g = i / FC_HEAD_DIM, d = i - g * FC_HEAD_DIM;
+      if (g0 + g < G) {
+        float o = 0.f;
+#pragma unroll
+        for (int sl = 0; sl < 16; ++sl) o += red[sl][g][d];
+        part_o[(((long long)b * Hq + (h * G + g0 + g)) * max_splits + split) * FC_HEAD_DIM + d] = o;
+      }
     }
   }
 }
@@ -470,7 +562,9 @@ extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cac
   const float c = scale * DA_LOG2E;
   const bool bf = k_cache->dtype == FC_BF16;
   if (splits > 0) {
-    const int gt = G >= 8 ? 8 : G >= 4 ? 4 : G >= 2 ? 2 : 1;
+    // the smallest tile that holds the whole group (padded head rows cost nothing; splitting a group would
+    // read its K and V once per tile); groups of more than 8 heads are served 8 at a time
+    const int gt = G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
     const int gtiles = (G + gt - 1) / gt;
     FC_REQUIRE(Hkv * gtiles <= 65535 && B <= 65535, FC_EUNSUPPORTED, "%s: grid too large", who);
     dim3 grid(splits, Hkv * gtiles, B);

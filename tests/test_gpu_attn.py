@@ -19,6 +19,8 @@ pytestmark = pytest.mark.gpu
     (8, 2, [33, 1024, 513]),
     (14, 2, [300, 17]),
     (16, 1, [129, 0, 600]),
+    (6, 2, [77, 260]),          # a group of 3 in a tile of 4
+    (10, 2, [513]),             # a group of 5 in a tile of 8
 ])
 def test_decode_attention(dev, dtype, Hq, Hkv, lens):
     L, B = 2, len(lens)
