@@ -1,0 +1,129 @@
+"""GPU parity: the top-k selection and the gather / compaction kernels on their own, bit-exact.
+
+Indices: identical to the oracle's stable selection (ties to the lowest index, ascending output) on integer-valued
+and heavily tied rows, special values, ragged rows, rows longer than the on-chip key buffer.  Compaction: every
+output byte equals the gathered source byte, for dense and paged views in either direction, in place, with per-
+sequence kept counts and with one index row shared by all heads.
+"""
+import pytest
+import torch
+
+from fastcache_amd import _lib, ops, synth
+from oracle import presses as opress
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("S,k", [(1, 1), (7, 3), (64, 64), (65, 1), (1000, 250), (4096, 1024), (15360, 77),
+                                 (15361, 5000), (40000, 10000)])
+def test_topk_random_and_tied_rows(dev, S, k):
+    """Continuous scores, then scores drawn from 5 distinct values so that the k-th value has many ties.  Rows of
+    more than 15360 scores do not fit the key buffer in LDS and take the path that re-reads them."""
+    g = torch.Generator().manual_seed(S * 7 + k)
+    for tied in (False, True):
+        sc = torch.randint(0, 5, (3, 4, S), generator=g).float() if tied else torch.randn(3, 4, S, generator=g)
+        got = ops.topk_select(sc.to(dev), k).cpu().long()
+        assert torch.equal(got, opress.topk_lowest_index(sc, k))
+        assert bool((got[..., 1:] > got[..., :-1]).all()) if k > 1 else True
+
+
+def test_topk_special_values(dev):
+    """NaN ranks above +inf, -0 equals +0 (the lower index wins), -inf is taken last."""
+    row = torch.tensor([0.0, -0.0, float("inf"), float("nan"), -float("inf"), 1.0, float("nan"), -1.0, 0.0, 1.0])
+    for k in range(1, row.numel() + 1):
+        got = ops.topk_select(row[None].to(dev), k).cpu().long()
+        assert torch.equal(got, opress.topk_lowest_index(row[None], k)), k
+
+
+def test_topk_ragged_rows_and_kept_counts(dev):
+    """Per-sequence valid lengths and kept counts: rows ordered (layer, b, head) use entry b; the tail of a row's
+    output stays -1; a kept count above the length keeps the whole row."""
+    L, B, H, S, K = 2, 3, 4, 300, 120
+    g = torch.Generator().manual_seed(5)
+    sc = torch.randn(L, B, H, S, generator=g)
+    lens = torch.tensor([300, 17, 150], dtype=torch.int32)
+    kept = torch.tensor([120, 40, 33], dtype=torch.int32)
+    got = ops.topk_select(sc.to(dev), K, row_lens=lens.to(dev), n_kept=kept.to(dev), rows_per_len=H).cpu().long()
+    for b in range(B):
+        n, kk = int(lens[b]), min(int(kept[b]), int(lens[b]))
+        ref = opress.topk_lowest_index(sc[:, b, :, :n], kk)
+        assert torch.equal(got[:, b, :, :kk], ref)
+        assert bool((got[:, b, :, kk:] == -1).all())
+
+
+def test_topk_strided_rows(dev):
+    """Rows spaced by a stride larger than their length (a narrowed view of a wider score buffer)."""
+    g = torch.Generator().manual_seed(8)
+    buf = torch.randn(2, 5, 512, generator=g)
+    view = buf.to(dev)[..., :400]
+    got = ops.topk_select(view, 100).cpu().long()
+    assert torch.equal(got, opress.topk_lowest_index(buf[..., :400], 100))
+
+
+def _payload(shape, dtype, seed):
+    """Values that differ in every (row, column) so that a wrong row or a shifted column shows."""
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randint(-2000, 2000, shape, generator=g).float() / 8).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shared_heads", [False, True])
+def test_compact_dense_to_dense(dev, dtype, shared_heads):
+    L, B, H, S, K = 2, 2, 3, 333, 100
+    k, v = _payload((L, B, H, S, 128), dtype, 1), _payload((L, B, H, S, 128), dtype, 2)
+    g = torch.Generator().manual_seed(3)
+    hi = 1 if shared_heads else H
+    idx = torch.stack([torch.sort(torch.randperm(S, generator=g)[:K]).values for _ in range(L * B * hi)])
+    idx = idx.view(L, B, hi, K).int()
+    kd, vd = k.to(dev), v.to(dev)
+    ok, ov = torch.zeros(L, B, H, K, 128, dtype=dtype, device=dev), torch.zeros(L, B, H, K, 128, dtype=dtype, device=dev)
+    ops.compact(_lib.dense_view(kd), _lib.dense_view(vd), _lib.dense_view(ok), _lib.dense_view(ov), idx.to(dev))
+    full = idx.long().expand(L, B, H, K)
+    for l in range(L):
+        assert torch.equal(ok[l].cpu(), opress.gather_tokens(k[l], full[l]))
+        assert torch.equal(ov[l].cpu(), opress.gather_tokens(v[l], full[l]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("block_size", [256, 16, 48])
+def test_compact_paged_in_place_with_kept_counts(dev, dtype, block_size):
+    """In-place compaction of a paged pool with a different kept count per sequence: the first n_kept[b] tokens of
+    every (layer, sequence, head) equal the gathered rows, pages of other sequences and spare pages are untouched."""
+    L, H, lens = 2, 4, [700, 64, 301]
+    B = len(lens)
+    case = synth.make_paged_case(seed=6, num_layers=L, batch=B, num_kv_heads=H, seq_lens=lens, dtype=dtype,
+                                 keep_dense=True, block_size=block_size, fill_value=7.0)
+    kept = [200, 64, 1]
+    K = max(kept)
+    g = torch.Generator().manual_seed(11)
+    idx = torch.full((L, B, H, K), -1, dtype=torch.int32)
+    for l in range(L):
+        for b in range(B):
+            for h in range(H):
+                idx[l, b, h, :kept[b]] = torch.sort(torch.randperm(lens[b], generator=g)[:kept[b]]).values.int()
+    pool = case.kv_cache.to(dev)
+    tab, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+    S = max(lens)
+    views = [_lib.paged_view(pool[p], tab, lens_d, S) for p in range(2)]
+    ops.compact(views[0], views[1], views[0], views[1], idx.to(dev), n_kept=torch.tensor(kept, dtype=torch.int32, device=dev))
+    after = pool.cpu()
+    used = set()
+    for b in range(B):
+        blocks = case.block_tables[b]
+        used.update(blocks)
+        for p, dense in enumerate((case.dense_k, case.dense_v)):
+            for l in range(L):
+                rows = torch.cat([after[p, l, blk] for blk in blocks])[:kept[b]]            # [n, H, D]
+                want = opress.gather_tokens(dense[l][b:b + 1, :, :lens[b]], idx[l, b:b + 1, :, :kept[b]].long())[0]
+                assert torch.equal(rows.permute(1, 0, 2), want), (b, p, l)
+    spare = [i for i in range(after.shape[2]) if i not in used]
+    assert bool((after[:, :, spare] == 7.0).all())
+
+
+def test_compact_rejects_bad_arguments(dev):
+    k = torch.zeros(1, 1, 2, 8, 128, device=dev)
+    view = _lib.dense_view(k)
+    with pytest.raises(_lib.FastcacheError):
+        ops.compact(view, view, view, view, torch.zeros(1, 1, 2, 4, dtype=torch.int64, device=dev))       # not int32
+    with pytest.raises(_lib.FastcacheError):
+        ops.compact(view, view, view, view, torch.zeros(2, 1, 2, 4, dtype=torch.int32, device=dev))       # layer mismatch
