@@ -44,30 +44,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-// Wave-wide maximum / sum with DPP steps inside each row of 16 lanes and four lane reads across the
-// rows; the result is wave-uniform.
-template <int CTRL>
-__device__ __forceinline__ float da_dpp(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float da_lane(float v, int l) {
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
-}
-__device__ __forceinline__ float da_wave_max(float v) {
-  v = fmaxf(v, da_dpp<0xB1>(v));    // quad_perm [1,0,3,2]
-  v = fmaxf(v, da_dpp<0x4E>(v));    // quad_perm [2,3,0,1]
-  v = fmaxf(v, da_dpp<0x141>(v));   // row_half_mirror
-  v = fmaxf(v, da_dpp<0x140>(v));   // row_mirror
-  return fmaxf(fmaxf(da_lane(v, 0), da_lane(v, 16)), fmaxf(da_lane(v, 32), da_lane(v, 48)));
-}
-__device__ __forceinline__ float da_wave_sum(float v) {
-  v += da_dpp<0xB1>(v);
-  v += da_dpp<0x4E>(v);
-  v += da_dpp<0x141>(v);
-  v += da_dpp<0x140>(v);
-  return (da_lane(v, 0) + da_lane(v, 16)) + (da_lane(v, 32) + da_lane(v, 48));
-}
-
 #define DA_PV_MFMA_MIN 8               // heads per workgroup from which p * V runs on the matrix pipe (measured: no gain below)
 #define DA_TILE 32                     // keys per tile: one MFMA block, 8 KB of K or V rows
 #define DA_TILEB (DA_TILE * 256)
@@ -236,7 +212,7 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
     float x[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) x[j] = sc[g][lane + 64 * j];
-    const float m = da_wave_max(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
+    const float m = fc_wave_max_uniform(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
     float sum = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -250,7 +226,7 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
       }
       sum += p;
     }
-    sum = da_wave_sum(sum);
+    sum = fc_wave_sum_uniform(sum);
     if (lane == 0 && g0 + g < G) {
       float* ml = part_ml + (((long long)b * Hq + (h * G + g0 + g)) * max_splits + split) * 2;
       ml[0] = m;

@@ -125,6 +125,43 @@ __device__ __forceinline__ float fc_wave_max(float v) {
   return v;
 }
 
+// ---- cross-lane sums and maxima without LDS traffic ----------------------------------------------
+// One DPP step: every lane reads the lane that CTRL names inside its row of 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ float fc_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// Sum over aligned groups of N consecutive lanes (N a power of two up to 16), in a fixed order; every
+// lane of a group ends up with the group's sum.
+template <int N>
+__device__ __forceinline__ float fc_group_sum(float v) {
+  if constexpr (N >= 2) v += fc_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+  if constexpr (N >= 4) v += fc_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+  if constexpr (N >= 8) v += fc_dpp<0x141>(v);   // row_half_mirror
+  if constexpr (N >= 16) v += fc_dpp<0x140>(v);  // row_mirror
+  return v;
+}
+template <int N>
+__device__ __forceinline__ float fc_group_max(float v) {
+  if constexpr (N >= 2) v = fmaxf(v, fc_dpp<0xB1>(v));
+  if constexpr (N >= 4) v = fmaxf(v, fc_dpp<0x4E>(v));
+  if constexpr (N >= 8) v = fmaxf(v, fc_dpp<0x141>(v));
+  if constexpr (N >= 16) v = fmaxf(v, fc_dpp<0x140>(v));
+  return v;
+}
+__device__ __forceinline__ float fc_read_lane(float v, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+// Wave-wide, wave-uniform results: DPP inside the four rows, then four lane reads.
+__device__ __forceinline__ float fc_wave_sum_uniform(float v) {
+  v = fc_group_sum<16>(v);
+  return (fc_read_lane(v, 0) + fc_read_lane(v, 16)) + (fc_read_lane(v, 32) + fc_read_lane(v, 48));
+}
+__device__ __forceinline__ float fc_wave_max_uniform(float v) {
+  v = fc_group_max<16>(v);
+  return fmaxf(fmaxf(fc_read_lane(v, 0), fc_read_lane(v, 16)), fmaxf(fc_read_lane(v, 32), fc_read_lane(v, 48)));
+}
+
 // ---- global memory -> LDS without register staging --------------------------------------------
 __device__ __forceinline__ unsigned fc_lds_addr(const void* p) {
   return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;

@@ -141,19 +141,6 @@ __global__ __launch_bounds__(EA_THREADS) void ea_logits_kernel(KvView kv, const 
   }
 }
 
-// 16 lanes of a row -> every lane gets the sum (DPP, fixed order)
-template <int CTRL>
-__device__ __forceinline__ float ea_dpp(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float ea_sum16(float v) {
-  v += ea_dpp<0xB1>(v);
-  v += ea_dpp<0x4E>(v);
-  v += ea_dpp<0x141>(v);
-  v += ea_dpp<0x140>(v);
-  return v;
-}
-
 #define EA_FIN_THREADS 256
 #define EA_MAX_GROUP 64
 
@@ -220,8 +207,8 @@ __global__ __launch_bounds__(EA_FIN_THREADS) void ea_finish_kernel(KvView vv, co
         }
       }
     }
-    p = ea_sum16(p) * inv_g;
-    sq = ea_sum16(sq);
+    p = fc_group_sum<16>(p) * inv_g;
+    sq = fc_group_sum<16>(sq);
     if (ok && sub == 0) {
       const float sc = use_vnorm ? (p + epsilon) * sqrtf(sq) : p;
       out[s] = sc;

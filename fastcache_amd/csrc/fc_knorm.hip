@@ -36,19 +36,6 @@ __device__ __forceinline__ float row_sumsq_part(const uint4& x) {
   }
 }
 
-// sum over an aligned group of 16 lanes (DPP, fixed order); every lane gets the sum
-template <int CTRL>
-__device__ __forceinline__ float kn_dpp(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float kn_sum16(float v) {
-  v += kn_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
-  v += kn_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
-  v += kn_dpp<0x141>(v);   // row_half_mirror
-  v += kn_dpp<0x140>(v);   // row_mirror
-  return v;
-}
-
 template <int DTYPE>
 __device__ __forceinline__ float round_to_storage(float x) {
   if (DTYPE == FC_BF16) return fc_bf16_to_float(fc_float_to_bf16(x));
@@ -98,7 +85,7 @@ __global__ __launch_bounds__(KN_THREADS) void knorm_kernel(KvView kv, float* __r
     }
 #pragma unroll
     for (int u = 0; u < KN_U; ++u) {
-      float part = kn_sum16(row_sumsq_part<DTYPE>(x[u]));
+      float part = fc_group_sum<16>(row_sumsq_part<DTYPE>(x[u]));
       if (LPR == 32) part += __shfl_xor(part, 16, 64);
       if (r0 + u * RPP + rg < rows && sub == 0) {
         float v;

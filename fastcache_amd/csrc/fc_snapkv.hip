@@ -51,21 +51,6 @@ __device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16
 
 __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Sum over aligned groups of N consecutive lanes (N a power of two up to 16) with DPP adds in a
-// fixed order; every lane of a group ends up with the group's sum.
-template <int CTRL>
-__device__ __forceinline__ float sk_dpp_get(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-template <int N>
-__device__ __forceinline__ float sk_group_sum(float v) {
-  if constexpr (N >= 2) v += sk_dpp_get<0xB1>(v);    // quad_perm [1,0,3,2]
-  if constexpr (N >= 4) v += sk_dpp_get<0x4E>(v);    // quad_perm [2,3,0,1]
-  if constexpr (N >= 8) v += sk_dpp_get<0x141>(v);   // row_half_mirror
-  if constexpr (N >= 16) v += sk_dpp_get<0x140>(v);  // row_mirror
-  return v;
-}
-
 template <int NW>
 struct SkCfg {
   static constexpr int ST = NW >= 8 ? 4 : 3;   // key tiles resident or in flight per workgroup
@@ -340,7 +325,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   constexpr int KPW = SK_KT / NW;
   const int fkey = wave * KPW + lane / NW, fp = lane % NW;
   auto fold = [&](int u) {   // tile processed u-th (tile T-1-u): sum the wavefronts' partial sums per key
-    const float v = sk_group_sum<NW>(vpart[u & 3][fp][fkey]);
+    const float v = fc_group_sum<NW>(vpart[u & 3][fp][fkey]);
     if (fp == 0) vraw[(T - 1 - u) & 3][fkey] = v;
   };
   auto emit_tile = [&](int e) {   // moving average of tile e, whose neighbours are folded
@@ -350,7 +335,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       const int x = s + j - hw;
       if (x >= 0 && x < SW) a += vraw[(x / SK_KT) & 3][x % SK_KT];
     }
-    a = sk_group_sum<NW>(a);
+    a = fc_group_sum<NW>(a);
     if (fp == 0 && s < SW) out_row[s] = a * out_mul;
   };
   auto probs = [&](const f32x16& acc, int u, int cb) {
