@@ -40,9 +40,6 @@ __device__ __forceinline__ unsigned short da_pack(float f) {
   return DTYPE == FC_BF16 ? fc_float_to_bf16(f) : fc_float_to_half(f);
 }
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 #define DA_PV_MFMA_MIN 8               // heads per workgroup from which p * V runs on the matrix pipe (measured: no gain below)
 #define DA_TILE 32                     // keys per tile: one MFMA block, 8 KB of K or V rows
@@ -171,12 +168,7 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       const uint4 kf = *reinterpret_cast<const uint4*>(ring + stage * DA_TILEB + (xs ^ (unsigned)(ks * 32)));
-      if constexpr (DTYPE == FC_BF16)
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qf[ks]), __builtin_bit_cast(bf16x8, kf),
-                                                      acc, 0, 0, 0);
-      else
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, qf[ks]), __builtin_bit_cast(f16x8, kf),
-                                                     acc, 0, 0, 0);
+      acc = fc_mfma<DTYPE>(qf[ks], kf, acc);
     }
     const int t = tile * DA_TILE + lrow;
     const bool live = t < ntok;
@@ -274,17 +266,8 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
             w[e2] = lo | (hi << 16);
           }
           const uint4 bfrag = make_uint4(w[0], w[1], w[2], w[3]);
-          if constexpr (DTYPE == FC_BF16) {
-            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                               __builtin_bit_cast(bf16x8, bfrag), oacc[nb], 0, 0, 0);
-            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a2),
-                                                               __builtin_bit_cast(bf16x8, bfrag), oacc[nb], 0, 0, 0);
-          } else {
-            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                              __builtin_bit_cast(f16x8, bfrag), oacc[nb], 0, 0, 0);
-            oacc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a2),
-                                                              __builtin_bit_cast(f16x8, bfrag), oacc[nb], 0, 0, 0);
-          }
+          oacc[nb] = fc_mfma<DTYPE>(a, bfrag, oacc[nb]);
+          oacc[nb] = fc_mfma<DTYPE>(a2, bfrag, oacc[nb]);
         }
       }
     };

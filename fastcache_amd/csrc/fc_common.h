@@ -125,6 +125,24 @@ __device__ __forceinline__ float fc_wave_max(float v) {
   return v;
 }
 
+// ---- matrix pipe ---------------------------------------------------------------------------------
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// C[32][32] += A[32][16] * B[16][32] in fp32 (v_mfma_f32_32x32x16).  Operands: lane (row or column l % 32,
+// half l / 32) holds the 8 consecutive k = half * 8 .. half * 8 + 7 as 16 bytes.  Result: the lane holds column
+// l % 32 and, in register i, row (i / 4) * 8 + half * 4 + i % 4.
+template <int DTYPE>
+__device__ __forceinline__ f32x16 fc_mfma(const uint4& a, const uint4& b, f32x16 c) {
+  if constexpr (DTYPE == FC_BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+}
+
 // ---- cross-lane sums and maxima without LDS traffic ----------------------------------------------
 // One DPP step: every lane reads the lane that CTRL names inside its row of 16 lanes.
 template <int CTRL>

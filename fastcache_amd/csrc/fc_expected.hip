@@ -16,9 +16,6 @@
 // Kernel 3 writes the sink scores once the layer's maximum is known.
 #include "fc_common.h"
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 #define EA_WAVES 8
 #define EA_THREADS (EA_WAVES * 64)
@@ -27,15 +24,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 #define EA_KEYS_PER_WG 2048       // keys one workgroup walks with its copy of C
 #define EA_LDS (2 * EA_CBYTES + 128 * 4)
 
-template <int DTYPE>
-__device__ __forceinline__ f32x16 ea_mfma(const uint4& a, const uint4& b, f32x16 c) {
-  if constexpr (DTYPE == FC_BF16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-}
 template <int DTYPE>
 __device__ __forceinline__ float ea_to_float(unsigned short h) {
   return DTYPE == FC_BF16 ? fc_bf16_to_float(h) : fc_half_to_float(h);
@@ -121,8 +109,8 @@ __global__ __launch_bounds__(EA_THREADS) void ea_logits_kernel(KvView kv, const 
         for (int jt = 0; jt < 4; ++jt) {
           const uint4 a = *reinterpret_cast<const uint4*>(ahi + jt * 32 * EA_ROWB + ks * 32);
           const uint4 a2 = *reinterpret_cast<const uint4*>(alo + jt * 32 * EA_ROWB + ks * 32);
-          acc[jt] = ea_mfma<DTYPE>(a, kf[ks], acc[jt]);
-          acc[jt] = ea_mfma<DTYPE>(a2, kf[ks], acc[jt]);
+          acc[jt] = fc_mfma<DTYPE>(a, kf[ks], acc[jt]);
+          acc[jt] = fc_mfma<DTYPE>(a2, kf[ks], acc[jt]);
         }
     }
     float z = 0.f;

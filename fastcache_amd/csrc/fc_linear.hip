@@ -9,21 +9,8 @@
 // is rounded to the storage dtype once.  Wider outputs are covered 128 columns at a time.
 #include "fc_common.h"
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 #define LN_WAVES 4
-
-template <int DTYPE>
-__device__ __forceinline__ f32x16 ln_mfma(const uint4& a, const uint4& b, f32x16 c) {
-  if constexpr (DTYPE == FC_BF16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-}
 
 // NT = 32-column tiles handled per pass (1..4)
 template <int DTYPE, int NT>
@@ -52,7 +39,7 @@ __global__ __launch_bounds__(LN_WAVES * 64) void linear_act_kernel(const char* _
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const uint4 b = *reinterpret_cast<const uint4*>(wp + ((long long)t * 32 * K + k0) * 2);
-      acc[t] = ln_mfma<DTYPE>(a, b, acc[t]);
+      acc[t] = fc_mfma<DTYPE>(a, b, acc[t]);
     }
   }
 

@@ -25,11 +25,8 @@
 // read tokens no earlier iteration writes.
 #include "fc_common.h"
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
@@ -48,16 +45,6 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // prefetch (weight fragments from LDS, token rows from memory) to just before its use and the
 // multiplications wait out the full latency each time.
 #define ML_PIN() __builtin_amdgcn_sched_barrier(0)
-
-template <int DTYPE>
-__device__ __forceinline__ f32x16 ml_mfma(const uint4& a, const uint4& b, f32x16 c) {
-  if constexpr (DTYPE == FC_BF16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-}
 
 // two fp32 -> packed storage dtype, round to nearest even
 template <int DTYPE>
@@ -253,7 +240,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = ml_mfma<DTYPE>(af[ks & 1][mb], xcur[tb][ks], acc[mb][tb]);
+          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = fc_mfma<DTYPE>(af[ks & 1][mb], xcur[tb][ks], acc[mb][tb]);
         }
         ML_PIN();
       }
@@ -290,7 +277,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = ml_mfma<DTYPE>(af[g & 1][mb], hf[tb][g], acc[mb][tb]);
+          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = fc_mfma<DTYPE>(af[g & 1][mb], hf[tb][g], acc[mb][tb]);
         }
         ML_PIN();
       }
@@ -327,7 +314,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
 #pragma unroll
-          for (int tb = 0; tb < ML_TB; ++tb) acc[nb][tb] = ml_mfma<DTYPE>(hf[tb][g], bfr[g & 1][nb], acc[nb][tb]);
+          for (int tb = 0; tb < ML_TB; ++tb) acc[nb][tb] = fc_mfma<DTYPE>(hf[tb][g], bfr[g & 1][nb], acc[nb][tb]);
         }
         ML_PIN();
       }

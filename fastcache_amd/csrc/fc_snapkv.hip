@@ -30,24 +30,11 @@
 // reads block 0 instead of faulting.
 #include "fc_common.h"
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 #define SK_KT 64           // keys per tile
 #define SK_TILEB (SK_KT * 256)  // LDS bytes per key tile (rows unpadded, 16-byte chunks XOR-swizzled)
 #define SK_NEG (-1.0e30f)  // "minus infinity" that stays finite under subtraction
 #define SK_TBL 1024        // block-table entries of one sequence cached in LDS
-
-template <int DTYPE>
-__device__ __forceinline__ f32x16 sk_mfma(const uint4& a, const uint4& b, f32x16 c) {
-  if constexpr (DTYPE == FC_BF16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-}
 
 __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -192,7 +179,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       const uint4 kf = *reinterpret_cast<const uint4*>(kbuf + (a0 ^ (unsigned)(ks * 32)));
-      acc = keys_rows ? sk_mfma<DTYPE>(kf, qf[ks], acc) : sk_mfma<DTYPE>(qf[ks], kf, acc);
+      acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc) : fc_mfma<DTYPE>(qf[ks], kf, acc);
     }
   };
   // ask the scheduler to spread the VALU work of one block between the MFMAs of the next
