@@ -242,3 +242,19 @@ def test_bucketed_decode_graphs_match_eager_layers(dev):
         # restore the prefixes for the next batch size
         pool_g.copy_(case.kv_cache)
         pool_e.copy_(case.kv_cache)
+
+
+def test_decode_attention_empty_rows(dev):
+    """Rows with no cached token give zeros, whatever their table row holds; their neighbours are unaffected."""
+    dtype, Hq, Hkv = torch.bfloat16, 8, 2
+    case = synth.make_paged_case(seed=3, num_layers=1, batch=3, num_kv_heads=Hkv, seq_lens=[300, 1, 5], dtype=dtype)
+    q = torch.randn(3, Hq, 128, generator=torch.Generator().manual_seed(2)).to(dtype).to(dev)
+    pool, tab = case.kv_cache.to(dev), case.table_tensor(dev)
+    max_len = tab.shape[1] * 256
+    kview, vview = _lib.paged_view(pool[0], tab, None, max_len), _lib.paged_view(pool[1], tab, None, max_len)
+    ws = ops.decode_attn_workspace(3, Hq, max_len, dev)
+    full = ops.decode_attn(kview, vview, 0, q, torch.tensor([300, 1, 5], dtype=torch.int32, device=dev), 128 ** -0.5, ws).cpu()
+    some = ops.decode_attn(kview, vview, 0, q, torch.tensor([300, 0, 0], dtype=torch.int32, device=dev), 128 ** -0.5, ws).cpu()
+    assert torch.equal(some[0], full[0]) and bool((some[1:] == 0).all())
+    none = ops.decode_attn(kview, vview, 0, q, torch.zeros(3, dtype=torch.int32, device=dev), 128 ** -0.5, ws).cpu()
+    assert bool((none == 0).all())

@@ -228,3 +228,15 @@ def test_kv_quantizer_objects(dev):
         assert torch.equal(iq.cache[f"k_{i}"]["max_val"].cpu(), rm)
     deq = iq.dequantize_cache(out)
     assert torch.equal(deq[0][0].cpu(), out[0][0].cpu() * iq.cache["k_0"]["scale"].cpu())
+
+
+@pytest.mark.parametrize("shape,bits", [((1, 100), 2), ((3, 5, 7), 16), ((2, 1), 4), ((4, 1000), 3)])
+def test_fake_quantize_odd_shapes(dev, shape, bits):
+    """Rows that are no multiple of the wavefront, one-element rows, the smallest and the widest code range."""
+    from oracle import presses as op
+    g = torch.Generator().manual_seed(sum(shape) + bits)
+    x = torch.randn(*shape, generator=g)
+    for per_tensor in (False, True):
+        ref = op.fake_quantize(x, bits, per_tensor)[0]
+        got = ops.fake_quantize(x.to(dev), bits, per_tensor).cpu()
+        assert torch.equal(torch.nan_to_num(got, nan=-7.0), torch.nan_to_num(ref, nan=-7.0)), per_tensor

@@ -293,3 +293,27 @@ def test_snapkv_short_sequences_and_tile_boundaries(dev, S, W, ksz):
     got_p = ops.snapkv_score(_lib.paged_view(pool[0], tables, lens, S), case.queries.to(dev), W, ksz,
                              causal_window=True, reduction="sum", seq_lens=lens).cpu()
     assert torch.equal(got_p, got)
+
+
+def test_expected_attention_edge_cases(dev):
+    """No sinks; a single scored key; a sequence not longer than the sinks next to a normal one; mean only."""
+    from oracle import presses as opress
+    k, v, mu, cov = _ea_case(3, 1, 2, 2, 9, torch.float16)
+    kd, vd = k.to(dev), v.to(dev)
+    for n_sink, use_cov in ((0, True), (8, True), (4, False)):
+        ref = opress.expected_attention_score(k, v, mu, cov if use_cov else None, n_sink, True, 0.0)
+        got = ops.expected_attention_score(_lib.dense_view(kd), _lib.dense_view(vd), mu.to(dev),
+                                           cov.to(dev) if use_cov else None, n_sink, True, 0.0)[0].cpu()
+        assert float(((got - ref).abs() / ref.abs().clamp_min(1e-9)).max()) <= 1e-3, (n_sink, use_cov)
+    # ragged paged batch: sequence 1 has fewer tokens than sinks -> all its tokens carry the layer maximum
+    lens = [40, 3]
+    case = synth.make_paged_case(seed=2, num_layers=1, batch=2, num_kv_heads=2, seq_lens=lens, dtype=torch.bfloat16,
+                                 keep_dense=True)
+    g = torch.Generator().manual_seed(1)
+    mu2 = torch.randn(1, 2, 4, 128, generator=g) * 0.3
+    pool, tab, lens_d = case.kv_cache.to(dev), case.table_tensor(dev), case.lens_tensor(dev)
+    got = ops.expected_attention_score(_lib.paged_view(pool[0], tab, lens_d, 40), _lib.paged_view(pool[1], tab, lens_d, 40),
+                                       mu2.to(dev), None, 4, True, 0.0)[0].cpu()
+    ref0 = opress.expected_attention_score(case.dense_k[0][0:1], case.dense_v[0][0:1], mu2[0, 0:1], None, 4, True, 0.0)[0]
+    assert float(((got[0] - ref0).abs() / ref0.abs().clamp_min(1e-9)).max()) <= 1e-3
+    assert bool((got[1, :, :3] == ref0.max()).all()) and bool(torch.isinf(got[1, :, 3:]).all())
