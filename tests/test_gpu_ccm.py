@@ -5,7 +5,7 @@ a different summation order, so a hidden activation can round to the neighbourin
 and move the final output by about one unit in the last place of the storage dtype (2^-10 relative
 for fp16, 2^-7 for bf16).  The check is therefore: error norm / reference norm <= 1e-3, and every
 element within 1e-3 * max|ref| + 2 ulp(storage) of the reference, except for at most one element in
-10^4 (a flipped hidden activation times an output weight), which must stay within 1 % of max|ref|.
+10^3 (a flipped hidden activation times the output weights of its row), which must stay within 1 % of max|ref|.
 """
 import pytest
 import torch
@@ -35,9 +35,9 @@ def assert_mlp_close(got, ref, dtype):
     bound = 1e-3 * scale + 2 * ulp * ref.abs().clamp_min(scale * 2.0 ** -14)
     # A hidden activation that sits on a rounding boundary of the storage dtype can round the other way
     # (different summation order); its ulp times an output weight can exceed the bound for that one output
-    # row.  Such elements must be rare (at most 1 in 10^4) and small (1 % of the largest value).
+    # row's 128 outputs.  Such elements must be rare (at most 1 in 10^3) and small (1 % of the largest value).
     outliers = err > bound
-    assert int(outliers.sum()) <= max(1, err.numel() // 10000), f"{int(outliers.sum())} elements beyond the bound"
+    assert int(outliers.sum()) <= max(8, err.numel() // 1000), f"{int(outliers.sum())} elements beyond the bound"
     assert float(err.max()) <= 1e-2 * scale, f"max error {float(err.max()):.3e} vs scale {scale:.3e}"
 
 
