@@ -6,7 +6,7 @@ hot path over one batch of synthetic input that is already resident in HBM.  The
 is configuration 2 (SnapKV press over a Qwen3-8B-shaped paged pool: score -> window fill -> top-k
 -> in-place compaction, all 36 layers, batch 8, 4096 tokens per sequence).  ``--workload`` selects
 the other configurations (knorm, ccm, decode, hybrid; decode-eager = the decode launches without a
-graph, for the profiler); they are measured the same way.
+graph, for the profiler; snapkv-lse = cfg2 with the window queries' log-sum-exp given, single pass over K); they are measured the same way.
 
 Extra objects on the line:
   roofline      the dominant kernel of the workload: algorithmic bytes per launch divided by its
@@ -86,10 +86,13 @@ class SnapKVWorkload(Workload):
     dtype_name = "bf16"
     kernel_name = "snapkv_kernel"
 
-    def __init__(self, seed, device):
+    def __init__(self, seed, device, given_lse=False):
         super().__init__()
         from fastcache_amd import synth
         self.L, self.B, self.Hq, self.Hkv, self.S, self.W, self.ksz = 36, 8, 32, 8, 4096, 64, 7
+        self.given_lse = given_lse
+        if given_lse:
+            self.name = self.name + "+given-lse"
         self.ratio = 0.75
         self.device = device
         self.case = synth.snapkv_case(seed=seed, num_layers=self.L, batch=self.B, num_q_heads=self.Hq,
@@ -109,6 +112,18 @@ class SnapKVWorkload(Workload):
         self.kernel_bytes = q_bytes + k_bytes + score_bytes
         self.kernel_flops = 2 * self.B * self.L * self.Hq * self.W * self.S * D
         self.pass_bytes = q_bytes + k_bytes + gather_bytes
+        self.lse = None
+        if given_lse:
+            # what the prefill's attention kernel would hand over: ln sum exp(scale * q.k) per window query
+            self.lse = torch.empty((self.L, self.B, self.Hq, self.W), dtype=torch.float32, device=device)
+            G = self.Hq // self.Hkv
+            mask = torch.triu(torch.full((self.W, self.S), float("-inf"), device=device), diagonal=self.S - self.W + 1)
+            for layer in range(self.L):
+                for b in range(self.B):
+                    blocks = self.tables[b, :self.S // 256].long()
+                    k = self.case.kv_cache[0, layer, blocks].reshape(self.S, self.Hkv, D).permute(1, 0, 2).float()
+                    logits = torch.matmul(self.queries[layer, b].float(), k.repeat_interleave(G, 0).transpose(1, 2))
+                    self.lse[layer, b] = torch.logsumexp(logits * D ** -0.5 + mask, dim=-1)
 
     def config(self):
         return {"workload": self.name, "layers": self.L, "batch": self.B, "q_heads": self.Hq,
@@ -129,8 +144,14 @@ class SnapKVWorkload(Workload):
         row_max = torch.empty((L, B, Hkv), dtype=torch.float32, device=self.device)
         st = current_stream()
         with self.br:
-            check(fn("fc_snapkv_score")(C.byref(kview), self.queries.data_ptr(), self.Hq, self.W, self.ksz, 1,
-                                        D ** -0.5, 1.0, scores.data_ptr(), S, row_max.data_ptr(), st), "fc_snapkv_score")
+            if self.lse is None:
+                check(fn("fc_snapkv_score")(C.byref(kview), self.queries.data_ptr(), self.Hq, self.W, self.ksz, 1,
+                                            D ** -0.5, 1.0, scores.data_ptr(), S, row_max.data_ptr(), st),
+                      "fc_snapkv_score")
+            else:
+                check(fn("fc_snapkv_score_lse")(C.byref(kview), self.queries.data_ptr(), self.lse.data_ptr(), self.Hq,
+                                                self.W, self.ksz, 1, D ** -0.5, 1.0, scores.data_ptr(), S,
+                                                row_max.data_ptr(), st), "fc_snapkv_score_lse")
         # the window fill needs every row maximum of the layer, so it is its own (small) launch
         check(fn("fc_snapkv_fill_window")(scores.data_ptr(), S, L, B, Hkv, self.lens.data_ptr(), S, self.W,
                                           row_max.data_ptr(), st), "fc_snapkv_fill_window")
@@ -411,6 +432,8 @@ class CopyWorkload(Workload):
 
 WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
              "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True),
+             # cfg2 with the window queries' log-sum-exp handed in (not the BASELINE metric: the reference has no such input)
+             "snapkv-lse": lambda seed, dev: SnapKVWorkload(seed, dev, given_lse=True),
              # the decode launches without a graph, 4 steps per bracket: rocprofv3 cannot walk the 128-step graph
              "decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True)}
 

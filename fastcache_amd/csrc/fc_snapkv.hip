@@ -25,6 +25,8 @@
 // fp32.  The second sweep reads K again (a workgroup's column does not stay in L2 between the
 // sweeps), so the kernel's memory traffic is about twice the algorithmic figure.
 // Optionally the kernel also emits the maximum of each score row for the window fill.
+// When the caller supplies the log-sum-exp of every window query (a fused attention kernel returns it),
+// sweep 1 is skipped: its result is exactly that number.
 //
 // Table entries of a live sequence must be allocated blocks: a negative entry inside the sequence
 // reads block 0 instead of faulting.
@@ -47,7 +49,7 @@ struct SkCfg {
 template <int DTYPE, int NW, bool FAST>
 __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     KvView kv, const char* __restrict__ q, int Hq, int W, int ksz, int causal, float c, float out_mul,
-    float* __restrict__ scores, int score_stride, float* __restrict__ row_max) {
+    float* __restrict__ scores, int score_stride, float* __restrict__ row_max, const float* __restrict__ lse) {
   constexpr int THREADS = NW * 64;
   constexpr int ST = SkCfg<NW>::ST;
   constexpr int LPW = 16 / NW;   // 1 KB wave-loads (4 key rows) per wavefront and tile
@@ -150,9 +152,9 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // and positions m+1 .. m+ST-2 are in flight meanwhile.
   auto plan_tile = [&](int pos) { return pos < T ? pos : 2 * T - 1 - pos; };
   int kc = 0, m = 0;
-  auto prologue = [&]() {
-    m = 0;
-    for (int i = 0; i < ST - 1 && i < 2 * T; ++i) issue(plan_tile(i), (kc + i) % ST);
+  auto prologue = [&](int first) {   // first = 0: both sweeps; first = T: the second sweep alone
+    m = first;
+    for (int i = 0; i < ST - 1 && first + i < 2 * T; ++i) issue(plan_tile(first + i), (kc + i) % ST);
   };
   // top of a tile iteration: tile position m has landed for every wave, the stage consumed by the
   // previous iteration is free and receives position m+ST-1; returns the stage to read
@@ -271,8 +273,11 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   };
   // leading tiles without any masked key
   const int TF = causal ? min(S, SW + 1) / SK_KT : S / SK_KT;
-  for (int attempt = 0; attempt < 2; ++attempt) {
-    prologue();
+  // With the log-sum-exp of every window query given (the attention kernel of the prefill has it), the
+  // first sweep is not needed at all.
+  if (lse) prologue(T);
+  for (int attempt = 0; attempt < 2 && !lse; ++attempt) {
+    prologue(0);
     if (always_general || attempt == 1) {
       sweep1_plain(0, T, true);
     } else {
@@ -297,7 +302,10 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     const float mnew = fmaxf(mref, m2);
     const float ll = lsq * sk_exp2((mref - mnew) * c) + l2 * sk_exp2((m2 - mnew) * c);
     const bool ok = rb_valid && qi + lrow < W;
-    const float nmfin = ok ? -mnew * c - __builtin_amdgcn_logf(ll) : SK_NEG;   // v_log_f32 is log2
+    float nmfin = ok ? -mnew * c - __builtin_amdgcn_logf(ll) : SK_NEG;   // v_log_f32 is log2
+    if (lse && ok)   // natural-log sum of exp(scale * q.k) over the keys the query sees
+      nmfin = -1.4426950408889634f *
+              lse[((((long long)l * kv.batch + b) * Hq + (h * G + qg)) * W + qi + lrow)];
 #pragma unroll
     for (int i = 0; i < 16; ++i) nm[i] = __shfl(nmfin, (i >> 2) * 8 + lhalf * 4 + (i & 3), 64);
   }
@@ -436,10 +444,9 @@ __global__ __launch_bounds__(1024) void snapkv_fill_kernel(float* __restrict__ s
   }
 }
 
-extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_heads, int32_t window,
-                               int32_t kernel_size, int32_t causal_window, float scale, float out_scale,
-                               float* scores, int32_t score_stride, float* row_max, void* stream) {
-  const char* who = "fc_snapkv_score";
+static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void* queries, int32_t num_q_heads,
+                             int32_t window, int32_t kernel_size, int32_t causal_window, float scale, float out_scale,
+                             float* scores, int32_t score_stride, float* row_max, const float* lse, void* stream) {
   int rc = fc_check_view(keys, who);
   if (rc) return rc;
   FC_REQUIRE(queries && scores, FC_EINVAL, "%s: null pointer", who);
@@ -475,7 +482,7 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
     }                                                                                                        \
     hipLaunchKernelGGL((snapkv_kernel<DT, NWV, FA>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,       \
                        num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,    \
-                       row_max);                                                                             \
+                       row_max, lse);                                                                        \
   } while (0)
 #define SK_DISPATCH2(DT, FA)                 \
   if (waves <= 1) SK_LAUNCH(DT, 1, FA);      \
@@ -494,6 +501,23 @@ extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int3
 #undef SK_LAUNCH
   FC_CHECK_LAUNCH(who);
   return FC_OK;
+}
+
+extern "C" int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_heads, int32_t window,
+                               int32_t kernel_size, int32_t causal_window, float scale, float out_scale,
+                               float* scores, int32_t score_stride, float* row_max, void* stream) {
+  return snapkv_score_impl("fc_snapkv_score", keys, queries, num_q_heads, window, kernel_size, causal_window, scale,
+                           out_scale, scores, score_stride, row_max, nullptr, stream);
+}
+
+extern "C" int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float* lse, int32_t num_q_heads,
+                                   int32_t window, int32_t kernel_size, int32_t causal_window, float scale,
+                                   float out_scale, float* scores, int32_t score_stride, float* row_max,
+                                   void* stream) {
+  const char* who = "fc_snapkv_score_lse";
+  FC_REQUIRE(lse, FC_EINVAL, "%s: null log-sum-exp pointer", who);
+  return snapkv_score_impl(who, keys, queries, num_q_heads, window, kernel_size, causal_window, scale, out_scale,
+                           scores, score_stride, row_max, lse, stream);
 }
 
 extern "C" int fc_snapkv_fill_window(float* scores, int32_t score_stride, int32_t num_layers, int32_t batch,

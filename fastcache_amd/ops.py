@@ -48,11 +48,16 @@ def knorm_mean_score(keys: FcKvView, device, score_stride: Optional[int] = None)
 
 def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size: int,
                  causal_window: bool = True, reduction: str = "mean", scale: Optional[float] = None,
-                 seq_lens: Optional[torch.Tensor] = None, score_stride: Optional[int] = None) -> torch.Tensor:
+                 seq_lens: Optional[torch.Tensor] = None, score_stride: Optional[int] = None,
+                 lse: Optional[torch.Tensor] = None) -> torch.Tensor:
     """SnapKV observation-window scores -> fp32 ``[L, B, Hkv, stride]`` with the window positions
-    set to the per-layer maximum.  queries ``[L, B, Hq, W, D]`` (or ``[B, Hq, W, D]`` for one layer)."""
+    set to the per-layer maximum.  queries ``[L, B, Hq, W, D]`` (or ``[B, Hq, W, D]`` for one layer).
+    ``lse`` (optional, fp32 ``[L, B, Hq, W]``): natural-log sum of ``exp(scale * q.k)`` over the keys each window
+    query sees, as the prefill's attention kernel returns it; with it the keys are read once instead of twice."""
     if queries.dim() == 4:
         queries = queries.unsqueeze(0)
+        if lse is not None and lse.dim() == 3:
+            lse = lse.unsqueeze(0)
     if not queries.is_contiguous():
         queries = queries.contiguous()
     _lib.require_gpu(queries, "queries")
@@ -75,9 +80,18 @@ def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size
     out = torch.empty((L, B, keys.num_kv_heads, stride), dtype=torch.float32, device=dev)
     st = current_stream()
     row_max = torch.empty((L, B, keys.num_kv_heads), dtype=torch.float32, device=dev)
-    check(fn("fc_snapkv_score")(C.byref(keys), queries.data_ptr(), Hq, window, kernel_size,
-                                int(causal_window), scale, out_scale, out.data_ptr(), stride, row_max.data_ptr(), st),
-          "fc_snapkv_score")
+    if lse is None:
+        check(fn("fc_snapkv_score")(C.byref(keys), queries.data_ptr(), Hq, window, kernel_size,
+                                    int(causal_window), scale, out_scale, out.data_ptr(), stride, row_max.data_ptr(),
+                                    st), "fc_snapkv_score")
+    else:
+        _lib.require_gpu(lse, "lse")
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (L, B, Hq, W):
+            raise FastcacheError(f"lse must be fp32 [L={L}, B={B}, Hq={Hq}, W={W}], got {lse.dtype} {tuple(lse.shape)}")
+        lse = lse.contiguous()
+        check(fn("fc_snapkv_score_lse")(C.byref(keys), queries.data_ptr(), lse.data_ptr(), Hq, window, kernel_size,
+                                        int(causal_window), scale, out_scale, out.data_ptr(), stride,
+                                        row_max.data_ptr(), st), "fc_snapkv_score_lse")
     check(fn("fc_snapkv_fill_window")(out.data_ptr(), stride, L, B, keys.num_kv_heads, ptr(seq_lens),
                                       keys.max_seq_len, window, row_max.data_ptr(), st), "fc_snapkv_fill_window")
     return out

@@ -169,8 +169,9 @@ class SnapKVPress(ScorerPress):
         assert S > self.window_size, "Query length should be greater than the window size"
         q = self.window_queries(module, hidden_states, kwargs)
         head_dim = keys.shape[-1]
+        lse = kwargs.get("lse") if kwargs is not None else None      # [B, Hq, W] from the prefill's attention kernel
         return ops.snapkv_score(_lib.dense_view(keys), q.to(keys.dtype), self.window_size, self.kernel_size,
-                                self.causal_window, self.reduction, 1.0 / math.sqrt(head_dim))[0]
+                                self.causal_window, self.reduction, 1.0 / math.sqrt(head_dim), lse=lse)[0]
 
 
 @dataclass

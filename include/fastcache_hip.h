@@ -113,6 +113,18 @@ int fc_snapkv_score(const fc_kv_view* keys, const void* queries, int32_t num_q_h
                     float* scores, int32_t score_stride, float* row_max, void* stream);
 
 /*
+ * The same scores when the caller already has the log-sum-exp of every window query,
+ *   lse[layer][b][hq][w] = ln sum_s exp(scale * q . k_s)   over the keys the query sees
+ * (fp32, contiguous; with causal_window the keys up to the query's own position) -- what a fused
+ * attention kernel returns for its rows (flash-attn's softmax_lse for the last `window` positions of the
+ * prefill).  The kernel then needs a single pass over K instead of two.  The reference has no
+ * counterpart: its SnapKVPress recomputes the window attention from scratch (call sites as above).
+ */
+int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float* lse, int32_t num_q_heads,
+                        int32_t window, int32_t kernel_size, int32_t causal_window, float scale,
+                        float out_scale, float* scores, int32_t score_stride, float* row_max, void* stream);
+
+/*
  * Sets the window entries scores[l][b][h][S_b-W .. S_b) to the maximum over
  * scores[l][:, :, :S_b-W] of the same layer, the way kvpress pads the observation window
  * back in (F.pad(value=scores.max())) so that it always survives selection.

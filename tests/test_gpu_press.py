@@ -317,3 +317,32 @@ def test_expected_attention_edge_cases(dev):
     ref0 = opress.expected_attention_score(case.dense_k[0][0:1], case.dense_v[0][0:1], mu2[0, 0:1], None, 4, True, 0.0)[0]
     assert float(((got[0] - ref0).abs() / ref0.abs().clamp_min(1e-9)).max()) <= 1e-3
     assert bool((got[1, :, :3] == ref0.max()).all()) and bool(torch.isinf(got[1, :, 3:]).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,S,W,ksz,causal,bs", [(8, 2, 700, 64, 7, True, 256), (4, 4, 333, 32, 5, False, 256),
+                                                       (14, 2, 1000, 48, 3, True, 48), (2, 1, 65, 16, 1, True, 256)])
+def test_snapkv_scores_from_given_log_sum_exp(dev, dtype, Hq, Hkv, S, W, ksz, causal, bs):
+    """With the log-sum-exp of the window queries handed in (what the prefill's attention kernel returns), the
+    single-pass variant gives the scores of the two-pass kernel and of the oracle."""
+    L, B = 2, 2
+    case = synth.snapkv_case(seed=S, num_layers=L, batch=B, num_q_heads=Hq, num_kv_heads=Hkv, seq_len=S, window=W,
+                             keep_dense=True, dtype=dtype, block_size=bs)
+    G = Hq // Hkv
+    lse = torch.empty(L, B, Hq, W)
+    for l in range(L):
+        logits = torch.matmul(case.queries[l].float(), case.dense_k[l].float().repeat_interleave(G, 1).transpose(2, 3)) / 128 ** 0.5
+        if causal:
+            logits = logits + torch.triu(torch.full((W, S), float("-inf")), diagonal=S - W + 1)
+        lse[l] = torch.logsumexp(logits, dim=-1)
+    pool, tab, lens = case.kv_cache.to(dev), case.table_tensor(dev), case.lens_tensor(dev)
+    kview = _lib.paged_view(pool[0], tab, lens, S)
+    q = case.queries.to(dev)
+    two_pass = ops.snapkv_score(kview, q, W, ksz, causal_window=causal, reduction="sum", seq_lens=lens).cpu()
+    one_pass = ops.snapkv_score(kview, q, W, ksz, causal_window=causal, reduction="sum", seq_lens=lens, lse=lse.to(dev)).cpu()
+    ref = _oracle_snapkv_scores(case, W, ksz, causal, "sum")
+    tol = 1e-3 * float(ref.abs().mean())
+    torch.testing.assert_close(one_pass, ref, rtol=1e-3, atol=tol)
+    torch.testing.assert_close(one_pass, two_pass, rtol=2e-4, atol=tol)
+    with pytest.raises(_lib.FastcacheError):
+        ops.snapkv_score(kview, q, W, ksz, lse=lse[..., :-1].to(dev))
