@@ -533,12 +533,7 @@ extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cac
     const bool fast = tile_in_page(k_cache, k) && tile_in_page(v_cache, v);
 #define DA_LAUNCH(DT, GTV, FA)                                                                                   \
   do {                                                                                                          \
-    static bool attr_done = false;                                                                              \
-    if (!attr_done) {                                                                                           \
-      (void)hipFuncSetAttribute((const void*)decode_attn_kernel<DT, GTV, FA>,                                   \
-                          hipFuncAttributeMaxDynamicSharedMemorySize, DaCfg<GTV>::LDS);                         \
-      attr_done = true;                                                                                         \
-    }                                                                                                           \
+    FC_ALLOW_LDS((decode_attn_kernel<DT, GTV, FA>), DaCfg<GTV>::LDS);                                         \
     hipLaunchKernelGGL((decode_attn_kernel<DT, GTV, FA>), grid, dim3(DA_THREADS), DaCfg<GTV>::LDS, st, k, v,    \
                        layer, (const char*)q, num_q_heads, context_lens, c, part_o, part_ml, splits);           \
   } while (0)

@@ -29,6 +29,19 @@ void fc_set_error(const char* fmt, ...);
     }                                                                          \
   } while (0)
 
+// Kernels that use more than 64 KB of dynamic LDS need their limit raised once per device; `fn` names one
+// instantiation (a separate flag word per expansion of the macro, one bit per device).  Setting it twice is harmless.
+#define FC_ALLOW_LDS(fn, bytes)                                                                            \
+  do {                                                                                                     \
+    static unsigned long long allowed__ = 0ull;                                                            \
+    int dev__ = 0;                                                                                         \
+    (void)hipGetDevice(&dev__);                                                                            \
+    if (!((allowed__ >> (dev__ & 63)) & 1ull)) {                                                           \
+      (void)hipFuncSetAttribute((const void*)(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); \
+      allowed__ |= 1ull << (dev__ & 63);                                                                   \
+    }                                                                                                      \
+  } while (0)
+
 int fc_check_view(const fc_kv_view* v, const char* who);
 
 static inline int fc_elem_bytes(int dtype) { return dtype == FC_F32 ? 4 : 2; }

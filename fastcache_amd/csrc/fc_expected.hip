@@ -261,12 +261,7 @@ extern "C" int fc_expected_attention_score(const fc_kv_view* keys, const fc_kv_v
   const bool bf = keys->dtype == FC_BF16;
 #define EA_RUN(DT)                                                                                                   \
   do {                                                                                                               \
-    static bool attr_done = false;                                                                                   \
-    if (!attr_done) {                                                                                                \
-      (void)hipFuncSetAttribute((const void*)ea_logits_kernel<DT>, hipFuncAttributeMaxDynamicSharedMemorySize,       \
-                                EA_LDS);                                                                             \
-      attr_done = true;                                                                                              \
-    }                                                                                                                \
+    FC_ALLOW_LDS((ea_logits_kernel<DT>), EA_LDS);                                                             \
     hipLaunchKernelGGL((ea_logits_kernel<DT>), dim3(chunks, num_q_heads, L * B), dim3(EA_THREADS), EA_LDS, st, k,    \
                        mean_query, cov_query, num_q_heads, n_sink, raw, S, gmax);                                    \
     hipLaunchKernelGGL((ea_finish_kernel<DT>), dim3(Hkv, B, L), dim3(EA_FIN_THREADS), 0, st, v, (const float*)raw, S, \

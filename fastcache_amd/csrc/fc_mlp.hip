@@ -441,12 +441,7 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     const int mode = (sm == 0 && dm == 0) ? 0 : (sm == 1 && dm == 1) ? 1 : (sm == 0 && dm == 1) ? 2 : (sm == 1 && dm == 0) ? 3 : 4;
 #define ML_LAUNCH(DT, ST, DTT, WR)                                                                                     \
   do {                                                                                                             \
-    static bool attr_done = false;                                                                                 \
-    if (!attr_done) {                                                                                              \
-      hipFuncSetAttribute((const void*)mlp_kernel<DT, ST, DTT, WR>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
-                          (int)lds);                                                                               \
-      attr_done = true;                                                                                            \
-    }                                                                                                              \
+    FC_ALLOW_LDS((mlp_kernel<DT, ST, DTT, WR>), (int)lds);                                                    \
     hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT, WR>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,   \
                        (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,             \
                        (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);                               \

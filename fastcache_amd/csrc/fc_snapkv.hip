@@ -474,12 +474,7 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
   const char* q = (const char*)queries;
 #define SK_LAUNCH(DT, NWV, FA)                                                                                  \
   do {                                                                                                       \
-    static bool attr_done = false;                                                                           \
-    if (!attr_done) {                                                                                        \
-      hipFuncSetAttribute((const void*)snapkv_kernel<DT, NWV, FA>,                                           \
-                          hipFuncAttributeMaxDynamicSharedMemorySize, SkCfg<NWV>::LDS);                      \
-      attr_done = true;                                                                                      \
-    }                                                                                                        \
+    FC_ALLOW_LDS((snapkv_kernel<DT, NWV, FA>), SkCfg<NWV>::LDS);                                              \
     hipLaunchKernelGGL((snapkv_kernel<DT, NWV, FA>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,       \
                        num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,    \
                        row_max, lse);                                                                        \
