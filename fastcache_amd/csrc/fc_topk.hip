@@ -1,6 +1,7 @@
 // Row-wise top-k selection with lowest-index tie-break and ascending-index output.
 //
-// One workgroup (4 wavefronts) per score row.  The row is mapped to order-preserving 32-bit
+// One workgroup per score row: 4 wavefronts, or 16 for rows of more than 8192 scores (few such rows make a
+// launch, so each has to be walked by more lanes).  The row is mapped to order-preserving 32-bit
 // keys and staged in LDS; an MSB-first radix select (4 passes of 8 bits, LDS histogram) finds
 // the exact key T of the k-th largest element and how many elements equal to T are still
 // needed.  A final ordered pass keeps every key > T plus the first `need` keys == T in index
@@ -8,9 +9,10 @@
 // deterministic.  Rows too long for LDS are re-read from global memory (L2-resident).
 #include "fc_common.h"
 
-#define TK_THREADS 256
-#define TK_WAVES (TK_THREADS / FC_WAVE)
-#define TK_LDS_MAX_KEYS 15360  // 60 KiB of keys
+#define TK_BINS 256
+#define TK_LDS_MAX_KEYS 15360        // 60 KiB of keys: several workgroups of 256 threads per CU
+#define TK_LONG_ROW 8192             // rows longer than this take 1024 threads
+#define TK_LDS_MAX_KEYS_LONG 36864   // 144 KiB of keys: one workgroup of 1024 threads per CU
 
 __device__ __forceinline__ unsigned tk_key(float f) {
   unsigned u = __float_as_uint(f);
@@ -19,16 +21,17 @@ __device__ __forceinline__ unsigned tk_key(float f) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-template <bool LDS_KEYS>
+template <bool LDS_KEYS, int TK_THREADS>
 __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restrict__ scores,
                                                           int score_stride, int len,
                                                           const int* __restrict__ row_lens,
                                                           int rows_per_len, int row_lens_mod, int k,
                                                           const int* __restrict__ n_kept,
                                                           int* __restrict__ indices, int index_stride) {
+  constexpr int TK_WAVES = TK_THREADS / FC_WAVE;
   extern __shared__ unsigned lds_keys[];
-  __shared__ unsigned hist[256];
-  __shared__ unsigned wave_tot[TK_WAVES];
+  __shared__ unsigned hist[TK_BINS];
+  __shared__ unsigned wave_tot[TK_BINS / FC_WAVE];
   __shared__ unsigned sel_bin, sel_remaining;
   __shared__ unsigned w_eq[TK_WAVES], w_gt[TK_WAVES];
 
@@ -56,7 +59,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
 
   unsigned prefix = 0, mask = 0, remaining = (unsigned)kk;
   for (int shift = 24; shift >= 0; shift -= 8) {
-    hist[tid] = 0;  // TK_THREADS == 256 bins
+    if (tid < TK_BINS) hist[tid] = 0;
     __syncthreads();
     for (int i0 = 0; i0 < n; i0 += TK_THREADS) {
       const int i = i0 + tid;
@@ -79,23 +82,28 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
       if (todo) atomicAdd(&hist[bin], 1u);
     }
     __syncthreads();
-    // suffix sums over bins: thread t owns bin 255 - t
-    const unsigned h = hist[255 - tid];
-    unsigned incl = h;
+    // suffix sums over bins: thread t < 256 owns bin 255 - t
+    unsigned h = 0, incl = 0;
+    if (tid < TK_BINS) {
+      h = hist[TK_BINS - 1 - tid];
+      incl = h;
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      unsigned up = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += up;
+      for (int o = 1; o < 64; o <<= 1) {
+        unsigned up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+      }
+      if (lane == 63) wave_tot[wave] = incl;
     }
-    if (lane == 63) wave_tot[wave] = incl;
     __syncthreads();
-    unsigned base = 0;
-    for (int w = 0; w < wave; ++w) base += wave_tot[w];
-    incl += base;
-    const unsigned excl = incl - h;  // elements in strictly larger bins
-    if (excl < remaining && remaining <= incl) {
-      sel_bin = 255u - (unsigned)tid;
-      sel_remaining = remaining - excl;
+    if (tid < TK_BINS) {
+      unsigned base = 0;
+      for (int w = 0; w < wave; ++w) base += wave_tot[w];
+      incl += base;
+      const unsigned excl = incl - h;  // elements in strictly larger bins
+      if (excl < remaining && remaining <= incl) {
+        sel_bin = (unsigned)(TK_BINS - 1 - tid);
+        sel_remaining = remaining - excl;
+      }
     }
     __syncthreads();
     prefix |= sel_bin << shift;
@@ -161,13 +169,18 @@ extern "C" int fc_topk_select(const float* scores, int32_t score_stride, int32_t
              FC_EINVAL, "fc_topk_select: rows_per_len and row_lens_mod must be positive when per-row sizes are given");
   if (rows == 0 || len == 0) return FC_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (len <= TK_LDS_MAX_KEYS) {
-    hipLaunchKernelGGL((topk_kernel<true>), dim3(rows), dim3(TK_THREADS), (size_t)len * 4, st, scores,
-                       score_stride, len, row_lens, rows_per_len, row_lens_mod, k, n_kept, indices, index_stride);
+#define TK_LAUNCH(LK, TH, LDSB)                                                                                    \
+  hipLaunchKernelGGL((topk_kernel<LK, TH>), dim3(rows), dim3(TH), (size_t)(LDSB), st, scores, score_stride, len,  \
+                     row_lens, rows_per_len, row_lens_mod, k, n_kept, indices, index_stride)
+  if (len <= TK_LONG_ROW) {
+    TK_LAUNCH(true, 256, (size_t)len * 4);
+  } else if (len <= TK_LDS_MAX_KEYS_LONG) {
+    FC_ALLOW_LDS((topk_kernel<true, 1024>), TK_LDS_MAX_KEYS_LONG * 4);
+    TK_LAUNCH(true, 1024, (size_t)len * 4);
   } else {
-    hipLaunchKernelGGL((topk_kernel<false>), dim3(rows), dim3(TK_THREADS), 0, st, scores, score_stride,
-                       len, row_lens, rows_per_len, row_lens_mod, k, n_kept, indices, index_stride);
+    TK_LAUNCH(false, 1024, 0);
   }
+#undef TK_LAUNCH
   FC_CHECK_LAUNCH("fc_topk_select");
   return FC_OK;
 }
