@@ -46,10 +46,17 @@ struct SkCfg {
   static constexpr int LDS = ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4 + SK_TBL * 4;
 };
 
-template <int DTYPE, int NW, bool FAST>
+// MODE 0: the whole kernel for one (layer, sequence, kv head) column.
+// The key range of a column can also be cut into `nsplit` pieces, one workgroup each, for launches with too few
+// columns to fill the GPU:
+// MODE 1: sweep 1 over the piece's tiles only; (largest scaled logit, sum of exp2) per query go to `part`;
+// MODE 2: sweep 2 over the piece's tiles with the log-sum-exp given; the per-key sums go to `raw` unpooled
+//         (a small kernel takes the moving average afterwards, across the pieces' borders).
+template <int DTYPE, int NW, bool FAST, int MODE>
 __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     KvView kv, const char* __restrict__ q, int Hq, int W, int ksz, int causal, float c, float out_mul,
-    float* __restrict__ scores, int score_stride, float* __restrict__ row_max, const float* __restrict__ lse) {
+    float* __restrict__ scores, int score_stride, float* __restrict__ row_max, const float* __restrict__ lse,
+    int nsplit, float* __restrict__ part, float* __restrict__ raw) {
   constexpr int THREADS = NW * 64;
   constexpr int ST = SkCfg<NW>::ST;
   constexpr int LPW = 16 / NW;   // 1 KB wave-loads (4 key rows) per wavefront and tile
@@ -60,8 +67,10 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   float(*vraw)[SK_KT] = reinterpret_cast<float(*)[SK_KT]>(smem + ST * SK_TILEB + 4 * NW * SK_KT * 4);
   int* tbl = reinterpret_cast<int*>(smem + ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4);
 
-  const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
   const int Hkv = kv.num_kv_heads;
+  const int b = blockIdx.y, l = blockIdx.z;
+  const int h = MODE == 0 ? (int)blockIdx.x : (int)blockIdx.x % Hkv;
+  const int split = MODE == 0 ? 0 : (int)blockIdx.x / Hkv;
   const int G = Hq / Hkv;
   const int WB = (W + 31) / 32;        // 32-row blocks per query head
   const int RBT = G * WB;              // row blocks of the group
@@ -72,12 +81,22 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   float* out_row = scores + (((long long)l * kv.batch + b) * Hkv + h) * (long long)score_stride;
 
   if (S <= W) {  // nothing outside the window to score
+    if (MODE != 0) return;   // the pooling kernel writes such rows
     for (int s = tid; s < score_stride; s += THREADS) out_row[s] = s < S ? 0.f : -INFINITY;
     if (row_max && tid == 0) row_max[((long long)l * kv.batch + b) * Hkv + h] = -INFINITY;
     return;
   }
   const int SW = S - W;                       // scored keys
   const int T = (S + SK_KT - 1) / SK_KT;      // key tiles
+  // this workgroup's tiles [tb, te) and the number of tile positions it walks
+  int tb = 0, te = T;
+  if (MODE != 0) {
+    const int tps = (T + nsplit - 1) / nsplit;
+    tb = split * tps;
+    te = min(T, tb + tps);
+    if (tb >= te) return;
+  }
+  const int P = MODE == 0 ? 2 * T : te - tb;
 
   // ---- query fragment: this wavefront's 32 query rows as MFMA A-operands ------------------
   uint4 qf[8];
@@ -150,18 +169,22 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // tiles read last are the likeliest to still be cached).  m is the position in the plan, kc the
   // number of tiles consumed so far; tile position m lives in stage (kc % ST) when it is consumed
   // and positions m+1 .. m+ST-2 are in flight meanwhile.
-  auto plan_tile = [&](int pos) { return pos < T ? pos : 2 * T - 1 - pos; };
+  auto plan_tile = [&](int pos) {
+    if (MODE == 1) return tb + pos;        // ascending
+    if (MODE == 2) return te - 1 - pos;    // descending
+    return pos < T ? pos : 2 * T - 1 - pos;
+  };
   int kc = 0, m = 0;
   auto prologue = [&](int first) {   // first = 0: both sweeps; first = T: the second sweep alone
     m = first;
-    for (int i = 0; i < ST - 1 && first + i < 2 * T; ++i) issue(plan_tile(first + i), (kc + i) % ST);
+    for (int i = 0; i < ST - 1 && first + i < P; ++i) issue(plan_tile(first + i), (kc + i) % ST);
   };
   // top of a tile iteration: tile position m has landed for every wave, the stage consumed by the
   // previous iteration is free and receives position m+ST-1; returns the stage to read
   auto acquire = [&]() {
-    if (m + ST - 2 < 2 * T) fc_wait_barrier<LPW*(ST - 2)>(); else fc_wait_barrier<0>();
+    if (m + ST - 2 < P) fc_wait_barrier<LPW*(ST - 2)>(); else fc_wait_barrier<0>();
     const int nx = m + ST - 1;
-    if (nx < 2 * T) issue(plan_tile(nx), (kc + ST - 1) % ST);
+    if (nx < P) issue(plan_tile(nx), (kc + ST - 1) % ST);
     return kc % ST;
   };
 
@@ -275,16 +298,18 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   const int TF = causal ? min(S, SW + 1) / SK_KT : S / SK_KT;
   // With the log-sum-exp of every window query given (the attention kernel of the prefill has it), the
   // first sweep is not needed at all.
-  if (lse) prologue(T);
-  for (int attempt = 0; attempt < 2 && !lse; ++attempt) {
+  const bool skip_sweep1 = MODE == 2 || (MODE == 0 && lse != nullptr);
+  if (skip_sweep1) prologue(MODE == 2 ? 0 : T);
+  for (int attempt = 0; attempt < 2 && !skip_sweep1; ++attempt) {
     prologue(0);
     if (always_general || attempt == 1) {
-      sweep1_plain(0, T, true);
+      sweep1_plain(tb, te, true);
     } else {
-      sweep1_plain(0, 1, true);
+      sweep1_plain(tb, tb + 1, true);
       nmq = -mref * c;
-      if (TF > 1) sweep1_piped(1, TF);
-      sweep1_plain(max(TF, 1), T, false);
+      const int tf_end = min(TF, te);
+      if (tf_end > tb + 1) sweep1_piped(tb + 1, tf_end);
+      sweep1_plain(max(tf_end, tb + 1), te, false);
     }
     const bool bad = !(lsq <= 3.0e38f);   // inf or NaN
     if (attempt == 1 || !__builtin_amdgcn_readfirstlane(__syncthreads_or(bad))) break;
@@ -302,6 +327,14 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     const float mnew = fmaxf(mref, m2);
     const float ll = lsq * sk_exp2((mref - mnew) * c) + l2 * sk_exp2((m2 - mnew) * c);
     const bool ok = rb_valid && qi + lrow < W;
+    if constexpr (MODE == 1) {   // this piece's statistics of the query, in log2 units; done
+      if (ok && lhalf == 0) {
+        float* pp = part + (((((long long)l * kv.batch + b) * Hq + (h * G + qg)) * W + qi + lrow) * nsplit + split) * 2;
+        pp[0] = mnew * c;
+        pp[1] = ll;
+      }
+      return;
+    }
     float nmfin = ok ? -mnew * c - __builtin_amdgcn_logf(ll) : SK_NEG;   // v_log_f32 is log2
     if (lse && ok)   // natural-log sum of exp(scale * q.k) over the keys the query sees
       nmfin = -1.4426950408889634f *
@@ -319,9 +352,16 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // Every wavefront folds and emits 64/NW keys of a tile with NW lanes per key.
   constexpr int KPW = SK_KT / NW;
   const int fkey = wave * KPW + lane / NW, fp = lane % NW;
-  auto fold = [&](int u) {   // tile processed u-th (tile T-1-u): sum the wavefronts' partial sums per key
+  const int tend = MODE == 2 ? te : T;          // sweep 2 walks tiles tend-1, tend-2, ...
+  const int P2 = MODE == 2 ? te - tb : T;       // ... P2 of them
+  auto fold = [&](int u) {   // tile processed u-th (tile tend-1-u): sum the wavefronts' partial sums per key
     const float v = fc_group_sum<NW>(vpart[u & 3][fp][fkey]);
-    if (fp == 0) vraw[(T - 1 - u) & 3][fkey] = v;
+    if constexpr (MODE == 2) {
+      const int s = (tend - 1 - u) * SK_KT + fkey;
+      if (fp == 0 && s < SW) raw[(((long long)l * kv.batch + b) * Hkv + h) * (long long)score_stride + s] = v;
+    } else {
+      if (fp == 0) vraw[(T - 1 - u) & 3][fkey] = v;
+    }
   };
   auto emit_tile = [&](int e) {   // moving average of tile e, whose neighbours are folded
     const int s = e * SK_KT + fkey;
@@ -344,7 +384,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     f32x16 acc_a, acc_b;
     int stage = acquire();
     mfma_block(false, stage, 0, acc_a);
-    for (int u = 0; u < T - 1; ++u) {
+    for (int u = 0; u < P2 - 1; ++u) {
       mfma_block(false, stage, 1, acc_b);
       probs(acc_a, u, 0);
       interleave();
@@ -354,17 +394,23 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       // the sums of the tile processed before this one are complete: fold them; tile T-u+2 had
       // both neighbours folded (by other wavefronts) before the barrier just passed
       if (u >= 1) fold(u - 1);
-      if (u >= 3) emit_tile(T - u + 2);
+      if (MODE == 0 && u >= 3) emit_tile(T - u + 2);
       mfma_block(false, stage, 0, acc_a);
       probs(acc_b, u, 1);
       interleave();
     }
     mfma_block(false, stage, 1, acc_b);
-    probs(acc_a, T - 1, 0);
+    probs(acc_a, P2 - 1, 0);
     interleave();
-    probs(acc_b, T - 1, 1);
+    probs(acc_b, P2 - 1, 1);
     ++m;
     ++kc;
+  }
+  if constexpr (MODE == 2) {   // the last two tiles' sums; pooling, tail and row maximum are the pooling kernel's
+    __syncthreads();
+    if (P2 >= 2) fold(P2 - 2);
+    fold(P2 - 1);
+    return;
   }
 
   // ---- drain: fold the last two tiles processed (tiles 1 and 0) and write tiles 3, 2, 1, 0.  Tile 3 needs
@@ -393,6 +439,67 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       for (int w = 1; w < NW; ++w) mx = fmaxf(mx, vpart[0][w][0]);
       row_max[((long long)l * kv.batch + b) * Hkv + h] = mx;
     }
+  }
+}
+
+// Split columns: the pieces' (max, sum) per window query -> natural-log sum of exponentials.
+__global__ __launch_bounds__(256) void snapkv_merge_stats_kernel(const float* __restrict__ part, long long queries_total,
+                                                                 int queries_per_seq, int batch,
+                                                                 const int* __restrict__ seq_lens, int max_seq_len,
+                                                                 int nsplit, float* __restrict__ lse) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;   // (layer, b, hq, w) flattened
+  if (i >= queries_total) return;
+  const int b = (int)((i / queries_per_seq) % batch);
+  int S = seq_lens ? seq_lens[b] : max_seq_len;
+  S = S < max_seq_len ? (S < 0 ? 0 : S) : max_seq_len;
+  const int T = (S + SK_KT - 1) / SK_KT;
+  if (T == 0) return;
+  const int tps = (T + nsplit - 1) / nsplit;
+  const int used = (T + tps - 1) / tps;                            // pieces that had tiles
+  const float* pp = part + i * nsplit * 2;
+  float M = SK_NEG;
+  for (int s = 0; s < used; ++s) M = fmaxf(M, pp[2 * s]);
+  float L = 0.f;
+  for (int s = 0; s < used; ++s) L += pp[2 * s + 1] * sk_exp2(pp[2 * s] - M);
+  lse[i] = (M + __builtin_amdgcn_logf(L)) * 0.6931471805599453f;   // log2 units -> natural log
+}
+
+// Split columns: zero-padded moving average of the raw per-key sums, the tail past the sequence, the row maximum.
+__global__ __launch_bounds__(256) void snapkv_pool_kernel(const float* __restrict__ raw, float* __restrict__ scores,
+                                                          int score_stride, const int* __restrict__ seq_lens,
+                                                          int max_seq_len, int W, int ksz, float out_mul,
+                                                          float* __restrict__ row_max) {
+  __shared__ float red[4];
+  const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
+  const long long row = ((long long)l * gridDim.y + b) * gridDim.x + h;
+  int S = seq_lens ? seq_lens[b] : max_seq_len;
+  S = S < max_seq_len ? (S < 0 ? 0 : S) : max_seq_len;
+  const float* in = raw + row * score_stride;
+  float* out = scores + row * score_stride;
+  const int tid = threadIdx.x;
+  if (S <= W) {
+    for (int s = tid; s < score_stride; s += 256) out[s] = s < S ? 0.f : -INFINITY;
+    if (row_max && tid == 0) row_max[row] = -INFINITY;
+    return;
+  }
+  const int SW = S - W, hw = ksz >> 1;
+  float mx = -INFINITY;
+  for (int s = tid; s < score_stride; s += 256) {
+    if (s < SW) {
+      float a = 0.f;
+      for (int x = max(s - hw, 0); x <= min(s + hw, SW - 1); ++x) a += in[x];
+      a *= out_mul;
+      out[s] = a;
+      mx = fmaxf(mx, a);
+    } else if (s >= S) {
+      out[s] = -INFINITY;
+    }
+  }
+  if (row_max) {
+    mx = fc_wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    if (tid == 0) row_max[row] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   }
 }
 
@@ -474,10 +581,10 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
   const char* q = (const char*)queries;
 #define SK_LAUNCH(DT, NWV, FA)                                                                                  \
   do {                                                                                                       \
-    FC_ALLOW_LDS((snapkv_kernel<DT, NWV, FA>), SkCfg<NWV>::LDS);                                              \
-    hipLaunchKernelGGL((snapkv_kernel<DT, NWV, FA>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,       \
+    FC_ALLOW_LDS((snapkv_kernel<DT, NWV, FA, 0>), SkCfg<NWV>::LDS);                                           \
+    hipLaunchKernelGGL((snapkv_kernel<DT, NWV, FA, 0>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,    \
                        num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,    \
-                       row_max, lse);                                                                        \
+                       row_max, lse, 1, (float*)nullptr, (float*)nullptr);                                   \
   } while (0)
 #define SK_DISPATCH2(DT, FA)                 \
   if (waves <= 1) SK_LAUNCH(DT, 1, FA);      \
@@ -513,6 +620,91 @@ extern "C" int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, 
   FC_REQUIRE(lse, FC_EINVAL, "%s: null log-sum-exp pointer", who);
   return snapkv_score_impl(who, keys, queries, num_q_heads, window, kernel_size, causal_window, scale, out_scale,
                            scores, score_stride, row_max, lse, stream);
+}
+
+// ---- split columns ------------------------------------------------------------------------------------
+extern "C" int64_t fc_snapkv_split_workspace_bytes(int32_t num_layers, int32_t batch, int32_t num_q_heads,
+                                                   int32_t num_kv_heads, int32_t window, int32_t score_stride,
+                                                   int32_t nsplit) {
+  if (num_layers <= 0 || batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || window <= 0 || score_stride < 0 ||
+      nsplit <= 0)
+    return -1;
+  const int64_t nq = (int64_t)num_layers * batch * num_q_heads * window;
+  return (nq * nsplit * 2 + nq + (int64_t)num_layers * batch * num_kv_heads * score_stride + 64) * (int64_t)sizeof(float);
+}
+
+extern "C" int fc_snapkv_score_split(const fc_kv_view* keys, const void* queries, const float* lse, int32_t num_q_heads,
+                                     int32_t window, int32_t kernel_size, int32_t causal_window, float scale,
+                                     float out_scale, float* scores, int32_t score_stride, float* row_max,
+                                     int32_t nsplit, void* workspace, int64_t workspace_bytes, void* stream) {
+  const char* who = "fc_snapkv_score_split";
+  int rc = fc_check_view(keys, who);
+  if (rc) return rc;
+  FC_REQUIRE(queries && scores && workspace, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(((uintptr_t)queries & 15) == 0 && ((uintptr_t)workspace & 15) == 0, FC_EINVAL,
+             "%s: queries / workspace not 16-byte aligned", who);
+  FC_REQUIRE(keys->dtype == FC_F16 || keys->dtype == FC_BF16, FC_EUNSUPPORTED,
+             "%s: fp16/bf16 caches only (got dtype %d)", who, keys->dtype);
+  FC_REQUIRE(num_q_heads > 0 && num_q_heads % keys->num_kv_heads == 0, FC_EINVAL,
+             "%s: num_q_heads %d not a multiple of num_kv_heads %d", who, num_q_heads, keys->num_kv_heads);
+  FC_REQUIRE(window > 0, FC_EINVAL, "%s: window must be positive", who);
+  FC_REQUIRE(kernel_size >= 1 && (kernel_size & 1) && kernel_size <= 63, FC_EINVAL,
+             "%s: kernel_size %d must be odd and <= 63", who, kernel_size);
+  FC_REQUIRE(score_stride >= keys->max_seq_len, FC_EINVAL, "%s: score_stride %d < max_seq_len %d", who,
+             score_stride, keys->max_seq_len);
+  FC_REQUIRE(nsplit >= 1 && nsplit <= 256, FC_EINVAL, "%s: nsplit %d out of range [1, 256]", who, nsplit);
+  const int L = keys->num_layers, B = keys->batch, Hkv = keys->num_kv_heads;
+  const int G = num_q_heads / Hkv;
+  const int waves = G * ((window + 31) / 32);
+  KvView kv = fc_make_view(keys);
+  const bool fast = !keys->block_tables ||
+                    (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL);
+  FC_REQUIRE(waves <= 16 && fast, FC_EUNSUPPORTED,
+             "%s: split columns need a query group of at most 16 row blocks (got %d) and pages of 64*2^n tokens or a "
+             "dense view", who, waves);
+  const int64_t need = fc_snapkv_split_workspace_bytes(L, B, num_q_heads, Hkv, window, score_stride, nsplit);
+  FC_REQUIRE(workspace_bytes >= need, FC_EINVAL, "%s: workspace of %lld bytes, %lld needed", who,
+             (long long)workspace_bytes, (long long)need);
+  FC_REQUIRE((long long)Hkv * nsplit <= 2147483647LL && B <= 65535 && L <= 65535, FC_EUNSUPPORTED, "%s: grid too large",
+             who);
+  if (keys->max_seq_len == 0) return FC_OK;
+  const long long nq = (long long)L * B * num_q_heads * window;
+  float* part = (float*)workspace;
+  float* lse_ws = part + nq * nsplit * 2;
+  float* raw = lse_ws + nq;
+  hipStream_t st = (hipStream_t)stream;
+  const float c = scale * 1.4426950408889634f;
+  const float out_mul = out_scale / (float)kernel_size;
+  const char* q = (const char*)queries;
+  dim3 grid(Hkv * nsplit, B, L);
+  const float* lse_use = lse;
+#define SK_SPLIT(DT, NWV, MD)                                                                                      \
+  do {                                                                                                           \
+    FC_ALLOW_LDS((snapkv_kernel<DT, NWV, true, MD>), SkCfg<NWV>::LDS);                                            \
+    hipLaunchKernelGGL((snapkv_kernel<DT, NWV, true, MD>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,     \
+                       num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,        \
+                       row_max, lse_use, nsplit, part, raw);                                                     \
+  } while (0)
+#define SK_SPLIT_NW(DT, MD)                     \
+  if (waves <= 1) SK_SPLIT(DT, 1, MD);          \
+  else if (waves <= 2) SK_SPLIT(DT, 2, MD);     \
+  else if (waves <= 4) SK_SPLIT(DT, 4, MD);     \
+  else if (waves <= 8) SK_SPLIT(DT, 8, MD);     \
+  else SK_SPLIT(DT, 16, MD)
+  if (!lse) {   // pieces' statistics, then their merge into the log-sum-exp
+    if (keys->dtype == FC_BF16) { SK_SPLIT_NW(FC_BF16, 1); } else { SK_SPLIT_NW(FC_F16, 1); }
+    hipLaunchKernelGGL(snapkv_merge_stats_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st,
+                       (const float*)part, nq, num_q_heads * window, B, keys->seq_lens, keys->max_seq_len, nsplit,
+                       lse_ws);
+    lse_use = lse_ws;
+  }
+  if (keys->dtype == FC_BF16) { SK_SPLIT_NW(FC_BF16, 2); } else { SK_SPLIT_NW(FC_F16, 2); }
+#undef SK_SPLIT_NW
+#undef SK_SPLIT
+  hipLaunchKernelGGL(snapkv_pool_kernel, dim3(Hkv, B, L), dim3(256), 0, st, (const float*)raw, scores, score_stride,
+                     keys->seq_lens, keys->max_seq_len, window, kernel_size, out_mul, row_max);
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
 }
 
 extern "C" int fc_snapkv_fill_window(float* scores, int32_t score_stride, int32_t num_layers, int32_t batch,

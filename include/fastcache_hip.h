@@ -125,6 +125,23 @@ int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float
                         float out_scale, float* scores, int32_t score_stride, float* row_max, void* stream);
 
 /*
+ * The same scores with every (layer, sequence, kv head) column cut into `nsplit` key ranges, one workgroup each:
+ * statistics of the pieces, their merge, per-key sums of the pieces, then the moving average across the pieces'
+ * borders.  For launches with too few columns to fill the GPU (one long prompt of a model with few kv heads:
+ * 288 columns of 32768 keys -32 % with 8 pieces); with 1000 or more columns one workgroup per column is faster.
+ * lse: optional log-sum-exp of the window queries as for fc_snapkv_score_lse (NULL = computed here).
+ * Needs a dense view or pages of 64*2^n tokens.
+ * workspace: fc_snapkv_split_workspace_bytes bytes.  No counterpart in the reference (same call sites as
+ * fc_snapkv_score).
+ */
+int64_t fc_snapkv_split_workspace_bytes(int32_t num_layers, int32_t batch, int32_t num_q_heads,
+                                        int32_t num_kv_heads, int32_t window, int32_t score_stride, int32_t nsplit);
+int fc_snapkv_score_split(const fc_kv_view* keys, const void* queries, const float* lse, int32_t num_q_heads,
+                          int32_t window, int32_t kernel_size, int32_t causal_window, float scale, float out_scale,
+                          float* scores, int32_t score_stride, float* row_max, int32_t nsplit, void* workspace,
+                          int64_t workspace_bytes, void* stream);
+
+/*
  * Sets the window entries scores[l][b][h][S_b-W .. S_b) to the maximum over
  * scores[l][:, :, :S_b-W] of the same layer, the way kvpress pads the observation window
  * back in (F.pad(value=scores.max())) so that it always survives selection.

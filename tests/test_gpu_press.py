@@ -346,3 +346,31 @@ def test_snapkv_scores_from_given_log_sum_exp(dev, dtype, Hq, Hkv, S, W, ksz, ca
     torch.testing.assert_close(one_pass, two_pass, rtol=2e-4, atol=tol)
     with pytest.raises(_lib.FastcacheError):
         ops.snapkv_score(kview, q, W, ksz, lse=lse[..., :-1].to(dev))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,S,W,ksz,causal,splits", [(8, 2, 2000, 64, 7, True, 3), (8, 2, 2000, 64, 7, True, 31),
+                                                           (14, 2, 1500, 48, 15, False, 4), (4, 1, 700, 64, 5, True, 2),
+                                                           (16, 4, 1100, 32, 63, True, 5)])
+def test_snapkv_split_columns(dev, dtype, Hq, Hkv, S, W, ksz, causal, splits):
+    """Columns cut into key ranges (one workgroup each, for launches with few columns): same scores as one workgroup
+    per column and as the oracle, ragged lengths included; more pieces than tiles leaves some pieces empty."""
+    L, lens = 2, [S, S - 517, 65]
+    B = len(lens)
+    case = synth.make_paged_case(seed=S + splits, num_layers=L, batch=B, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype,
+                                 num_q_heads=Hq, window=W, keep_dense=True)
+    pool, tab, lens_d = case.kv_cache.to(dev), case.table_tensor(dev), case.lens_tensor(dev)
+    kview = _lib.paged_view(pool[0], tab, lens_d, S)
+    q = case.queries.to(dev)
+    whole = ops.snapkv_score(kview, q, W, ksz, causal_window=causal, reduction="sum", seq_lens=lens_d, splits=1).cpu()
+    cut = ops.snapkv_score(kview, q, W, ksz, causal_window=causal, reduction="sum", seq_lens=lens_d, splits=splits).cpu()
+    for l in range(L):
+        for b, n in enumerate(lens):
+            if n <= W:
+                continue
+            ref = opress.snapkv_score(case.queries[l, b:b + 1], case.dense_k[l][b:b + 1, :, :n], W, ksz, causal, "sum")[0]
+            tol = 1e-3 * float(ref[:, :n - W].abs().mean())
+            # the window entries hold the layer's maximum over all sequences: compared between the two device paths only
+            torch.testing.assert_close(cut[l, b, :, :n - W], ref[:, :n - W], rtol=1e-3, atol=tol)
+            torch.testing.assert_close(cut[l, b, :, :n], whole[l, b, :, :n], rtol=2e-4, atol=tol)
+            assert bool(torch.isinf(cut[l, b, :, n:]).all())
