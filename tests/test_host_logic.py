@@ -326,3 +326,25 @@ def test_checkpoint_layouts_round_trip(tmp_path):
     assert load_checkpoint(m, torch.optim.SGD(m.parameters(), lr=0.1), None, path) == (3, 0.25)
     assert load_checkpoint(m, filename=str(tmp_path / "nope.pth")) == (0, float("inf"))
     assert load_checkpoint_only_model(fresh(), path) and not load_checkpoint_only_model(fresh(), str(tmp_path / "no.pth"))
+
+
+def test_snapkv_split_heuristic():
+    """Key ranges per column: none for launches with a thousand columns or more, up to 8 below, never pieces shorter
+    than 8 key tiles, never for pages that are no multiple of 64 tokens or groups of more than 16 row blocks."""
+    from fastcache_amd import ops
+    from fastcache_amd._lib import FcKvView
+
+    def view(L, B, Hkv, S, block_size=256, paged=True):
+        return FcKvView(base=0, stride_layer=0, stride_block=0, stride_batch=0, stride_token=0, stride_head=0,
+                        block_tables=1 if paged else None, table_stride=0, block_size=block_size, dtype=2,
+                        num_layers=L, batch=B, num_kv_heads=Hkv, head_dim=128, max_seq_len=S, seq_lens=None)
+
+    assert ops.snapkv_splits(view(36, 8, 8, 4096), 32, 64) == 1          # 2304 columns
+    assert ops.snapkv_splits(view(36, 1, 8, 32768), 32, 64) == 8         # 288 columns
+    assert ops.snapkv_splits(view(36, 2, 8, 16384), 32, 64) == 4         # 576 columns
+    assert ops.snapkv_splits(view(28, 1, 4, 32768), 28, 64) == 8         # 112 columns, 14 row blocks
+    assert ops.snapkv_splits(view(36, 1, 8, 1024), 32, 64) == 2          # 16 tiles: at most 2 pieces
+    assert ops.snapkv_splits(view(36, 1, 8, 500), 32, 64) == 1
+    assert ops.snapkv_splits(view(36, 1, 8, 32768, block_size=48), 32, 64) == 1
+    assert ops.snapkv_splits(view(36, 1, 8, 32768, paged=False), 32, 64) == 8
+    assert ops.snapkv_splits(view(4, 1, 1, 32768), 32, 64) == 1          # 64 row blocks per kv head
