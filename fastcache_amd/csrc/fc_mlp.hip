@@ -4,18 +4,21 @@
 //
 // Shape of the work: one workgroup of 8 wavefronts (two per SIMD, so that one multiplies while
 // the other converts, loads or stores) per group of (sequence, head) columns of one
-// layer; a wavefront owns 32 rows of one column per iteration.  The three GEMMs are chained
-// through registers without any transposition:
-//   layer 1 (transposed)  H1^T = W1 * X^T   A = W1 rows from LDS, B = X token rows straight
-//                                           from HBM (16-byte loads, each element read once);
-//   layer 2 (transposed)  H2^T = W2 * H1^T  B = layer 1's accumulators, converted in place;
-//   layer 3               Y = H2 * W3^T     A = layer 2's accumulators, B = W3 rows from LDS.
+// layer; a wavefront owns 32 rows of one column per iteration.  The three GEMMs are transposed
+// (features along the accumulator registers, one token per lane) and chained through registers:
+//   layer 1  H1^T = W1 * X^T   A = W1 rows from LDS, B = X token rows;
+//   layer 2  H2^T = W2 * H1^T  B = layer 1's accumulators, converted in place;
+//   layer 3  Y^T  = W3 * H2^T  B = layer 2's accumulators.
 // A 32x32 accumulator block holds, per lane, 16 values of one token column; taking registers
 // 0..7 and 8..15 as two k-steps gives a complete, if permuted, set of 16 k indices across the two
 // half-waves, so the next layer's weights are stored in LDS with the same permutation
 // ([0-3, 8-11 | 4-7, 12-15] inside every group of 16) and no data moves between lanes.
-// Layer 3's accumulators hold 32 consecutive output features across a half-wave, so its stores
-// are contiguous 64-byte segments.
+//
+// Token rows enter and leave in the layout memory likes, not the one the MFMA wants: four adjacent
+// lanes read (write) 64 contiguous bytes of a row, 16 rows per instruction, and the 32 rows x 64
+// bytes of two k-steps (of one 32-feature block of the output) are re-laid through 2 KB of LDS
+// private to the wavefront.  With one row per lane instead, every 16-byte access of an instruction
+// falls into a cache line of its own and the vector memory pipeline, not HBM, sets the pace.
 //
 // W2 and W3 (permuted) stay in LDS for the life of the workgroup; W1 streams through a double
 // buffer one 128-column chunk (one source token) at a time, shared by the wavefronts; each
@@ -30,17 +33,14 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-#ifndef ML_WAVES
-#define ML_WAVES 8       // wavefronts per workgroup (two per SIMD)
-#endif
-#ifndef ML_TB
-#define ML_TB 1          // 32-row token blocks per wavefront
-#endif
-#define ML_ROWS (32 * ML_TB)
+#define ML_WAVES 8                  // wavefronts per workgroup (two per SIMD)
+#define ML_ROWS 32                  // rows per wavefront and iteration
 #define ML_THREADS (ML_WAVES * 64)
 #define ML_ROWB 272                 // LDS bytes per weight row: 128 elements + 16 bytes of padding
 #define ML_WBYTES (128 * ML_ROWB)   // one 128 x 128 weight block in LDS
-#define ML_TBL 256                  // block-table entries cached per wavefront and view
+#define ML_TBLTOT 768               // block-table entries cached per workgroup and view, divided among its columns
+#define ML_XS 2048                  // per-wavefront LDS bytes for re-laying token rows: 32 rows x 64 bytes
+#define ML_LDS (4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + ML_WAVES * ML_XS)
 // Nothing is scheduled across this point.  Without it the compiler, short of registers, sinks every
 // prefetch (weight fragments from LDS, token rows from memory) to just before its use and the
 // multiplications wait out the full latency each time.
@@ -73,7 +73,7 @@ __device__ __forceinline__ uint4 ml_act_operand(const f32x16& acc, int i0) {
 }
 
 // accumulator block initialised with the bias of its 16 features: register i holds feature
-// fb + (i/4)*8 + lhalf*4 + i%4 (transposed layers: features run along the registers)
+// fb + (i/4)*8 + lhalf*4 + i%4
 __device__ __forceinline__ void ml_bias_init(f32x16& acc, const float* __restrict__ bias, int fb, int lhalf) {
 #pragma unroll
   for (int i4 = 0; i4 < 4; ++i4) {
@@ -83,6 +83,14 @@ __device__ __forceinline__ void ml_bias_init(f32x16& acc, const float* __restric
     acc[i4 * 4 + 2] = bv.z;
     acc[i4 * 4 + 3] = bv.w;
   }
+}
+
+// orders a wavefront's LDS writes before its following LDS reads of other lanes' data (the hardware executes
+// one wavefront's LDS instructions in order; this only keeps the compiler from moving them)
+__device__ __forceinline__ void ml_wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // SRC_T / DST_T: 0 = dense view (no table), 1 = paged view whose table row fits the LDS cache,
@@ -100,11 +108,13 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   char* w2buf = lds + 2 * ML_WBYTES;       // permuted
   char* w3buf = lds + 3 * ML_WBYTES;       // permuted
   float* bias = reinterpret_cast<float*>(lds + 4 * ML_WBYTES);  // [3][128] fp32
-  int* tbls = reinterpret_cast<int*>(lds + 4 * ML_WBYTES + 3 * 128 * sizeof(float));  // [waves][2][ML_TBL]
+  int* tbls = reinterpret_cast<int*>(lds + 4 * ML_WBYTES + 3 * 128 * 4);  // [2 views][columns of the workgroup][tcap]
+  char* xsw = lds + 4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + (threadIdx.x >> 6) * ML_XS;
 
   const int l = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 31, lhalf = lane >> 5;
+  const int lq = lane >> 2, lp = lane & 3;   // memory-side layout: row lq (and 16 + lq), 16-byte piece lp of 64 bytes
   const int cols_per_wg = ML_WAVES / wpc;
   const int col = blockIdx.x * cols_per_wg + wave / wpc;
   const int sub = wave % wpc;
@@ -113,15 +123,19 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   const int b = col_ok ? col / H : 0, h = col_ok ? col - (col / H) * H : 0;
   const int K1 = cf * 128;
 
-  // this wavefront's block-table rows (source and destination), so that no row address waits on a table read
-  int* stbl = tbls + (wave * 2) * ML_TBL;
-  int* dtbl = stbl + ML_TBL;
+  // this column's block-table rows (source and destination), so that no row address waits on a table read;
+  // filled by the wavefronts that share the column
+  const int tcap = ML_TBLTOT / cols_per_wg;
+  int* stbl = tbls + (wave / wpc) * tcap;
+  int* dtbl = stbl + ML_TBLTOT;
   const int s_last = seg_start + c_rows * cf - 1, d_last = dst_start + c_rows - 1;
   // also for a wavefront whose column is past the last one (b = 0): its loads are unconditional and need valid addresses
   if (SRC_T == 1)
-    for (int i = lane; i <= (s_last >> src.block_shift); i += 64) stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
+    for (int i = sub * 64 + lane; i <= (s_last >> src.block_shift); i += 64 * wpc)
+      stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
   if (col_ok && DST_T == 1)
-    for (int i = lane; i <= (d_last >> dst.block_shift); i += 64) dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
+    for (int i = sub * 64 + lane; i <= (d_last >> dst.block_shift); i += 64 * wpc)
+      dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
   auto src_off = [&](int s) -> long long {
     if (SRC_T == 0) return (long long)b * src.stride_batch + (long long)s * src.stride_token;
     if (SRC_T == 1) {
@@ -181,11 +195,11 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   const int rows_per_iter = ML_ROWS * wpc;
   const int n_iter = (c_rows + rows_per_iter - 1) / rows_per_iter;
   const int q_total = n_iter * cf;      // W1 chunk q = (iteration q / cf, token kc = q % cf) sits in buffer q & 1
-  const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lhalf * 16;
-  char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2;
+  const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lp * 16;
+  char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2 + lp * 16;
 
-  // X rows of chunk q for this lane: 2 token blocks x 8 k-steps of 16 bytes
-  auto x_load = [&](uint4 (&xf)[ML_TB][8], int q) {
+  // X rows of chunk q: xf[2*c4 + rh] holds bytes [64*c4 + 16*lp, +16) of the token row of output row 16*rh + lq
+  auto x_load = [&](uint4 (&xf)[8], int q) {
     const int it = q / cf, kc = q - it * cf;
     const int row0 = it * rows_per_iter + sub * ML_ROWS;
     // Every lane always loads (no branch around the loads, so that the compiler keeps exact counts of
@@ -193,32 +207,38 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
     // column past the last one (b = h = 0) and unallocated pages read some valid row instead; what is
     // computed from them is never stored.
 #pragma unroll
-    for (int tb = 0; tb < ML_TB; ++tb) {
-      const int r = min(row0 + tb * 32 + lrow, c_rows - 1);
+    for (int rh = 0; rh < 2; ++rh) {
+      const int r = min(row0 + rh * 16 + lq, c_rows - 1);
       long long off = src_off(seg_start + cf * r + kc);
       off = off < 0 ? 0 : off;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) xf[tb][ks] = *reinterpret_cast<const uint4*>(sbase + off * 2 + ks * 32);
+      for (int c4 = 0; c4 < 4; ++c4) xf[c4 * 2 + rh] = *reinterpret_cast<const uint4*>(sbase + off * 2 + c4 * 64);
     }
   };
+  // Re-laying through this wavefront's 2 KB of LDS: rows of 64 bytes, the four 16-byte pieces of a row XOR-ed
+  // with (row / 4) % 4 so that the memory-side accesses (4 rows per 16 lanes) and the operand-side accesses
+  // (16 rows, same piece, per 16 lanes) each touch every bank once.
+  const unsigned mem_at = (unsigned)lq * 64 + ((lp ^ ((lq >> 2) & 3)) << 4);   // row lq; row 16 + lq is 1024 further
+  const unsigned swz = (lrow >> 2) & 3;
+  const unsigned op_at0 = (unsigned)lrow * 64 + (((0 + lhalf) ^ swz) << 4);    // k-step 0 of the pair: pieces 0, 1
+  const unsigned op_at1 = (unsigned)lrow * 64 + (((2 + lhalf) ^ swz) << 4);    // k-step 1: pieces 2, 3
+  auto relay_put = [&](uint4 lo_rows, uint4 hi_rows) {
+    *reinterpret_cast<uint4*>(xsw + mem_at) = lo_rows;
+    *reinterpret_cast<uint4*>(xsw + mem_at + 1024) = hi_rows;
+    ml_wave_sync();
+  };
+  auto relay_get = [&](int e) { return *reinterpret_cast<const uint4*>(xsw + (e ? op_at1 : op_at0)); };
 
-  f32x16 acc[4][ML_TB];
-#ifdef ML_XD1
-  constexpr int XD = 1;
-#else
-  constexpr int XD = W1R ? 2 : 1;   // prefetch distance in chunks
-#endif
+  f32x16 acc[4];
 
-  // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+XD's rows load into `xnext`.
-  // With W1 resident three register buffers rotate (two chunks always in flight); the streaming
-  // variant needs registers for the W1 copy and keeps two buffers (one chunk in flight);
+  // One pipeline stage: chunk q of layer 1 from `xcur` while chunk q+1's rows load into `xnext`;
   // after the last chunk of an iteration, layers 2 and 3 and the stores.
-  auto stage = [&](uint4 (&xcur)[ML_TB][8], uint4 (&xnext)[ML_TB][8], int q) {
+  auto stage = [&](uint4 (&xcur)[8], uint4 (&xnext)[8], int q) {
     const int it = q / cf, kc = q - it * cf;
     // The prefetches are unconditional (straight-line code keeps the staging registers out of
-    // scratch memory): past the last chunk the X rows are out of range and load nothing, and the
+    // scratch memory): past the last chunk the X rows are clamped to valid ones, and the
     // extra W1 chunk lands in the buffer nobody reads again.
-    x_load(xnext, q + XD);
+    x_load(xnext, q + 1);
     ML_PIN();   // the prefetch stays ahead of this stage's multiplications
     if (!W1R) {
       __syncthreads();  // chunk q is in w1buf[q & 1]; every wavefront is done with chunk q - 1
@@ -227,42 +247,44 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
     {
       const char* wa = w1buf + (W1R ? kc : (q & 1)) * ML_WBYTES + lrow * ML_ROWB + lhalf * 16;
       uint4 af[2][4];      // weight fragments of k-step ks+1 are read while k-step ks multiplies
+      uint4 bop[2][2];     // token operands of two k-steps (64 bytes of every row), re-laid one pair ahead
+      relay_put(xcur[0], xcur[1]);
+      bop[0][0] = relay_get(0);
+      bop[0][1] = relay_get(1);
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) af[0][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
+        if ((ks & 1) == 0 && ks + 2 < 8) {
+          relay_put(xcur[ks + 2], xcur[ks + 3]);
+          bop[((ks >> 1) + 1) & 1][0] = relay_get(0);
+          bop[((ks >> 1) + 1) & 1][1] = relay_get(1);
+        }
         if (ks + 1 < 8) {
 #pragma unroll
           for (int mb = 0; mb < 4; ++mb)
             af[(ks + 1) & 1][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB + (ks + 1) * 32);
         }
-        ML_PIN();   // the four reads of the next k-step are issued before this k-step's multiplications
+        ML_PIN();   // the reads of the next k-step are issued before this k-step's multiplications
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-#pragma unroll
-          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = fc_mfma<DTYPE>(af[ks & 1][mb], xcur[tb][ks], acc[mb][tb]);
-        }
+        for (int mb = 0; mb < 4; ++mb) acc[mb] = fc_mfma<DTYPE>(af[ks & 1][mb], bop[(ks >> 1) & 1][ks & 1], acc[mb]);
         ML_PIN();
       }
     }
     if (!W1R) w1_store((q + 1) & 1);
     if (kc != cf - 1) return;
 
-    // ---- layer 2: H2^T = W2 * H1^T, B operand taken from layer 1's accumulators -------------------
-    uint4 hf[ML_TB][8];
+    // ---- layers 2 and 3: H^T = W * (previous H)^T, B operand taken from the previous layer's accumulators ----
+    uint4 hf[8];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
+    for (int layer = 1; layer < 3; ++layer) {
 #pragma unroll
-      for (int tb = 0; tb < ML_TB; ++tb) {
-        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0);
-        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8);
+      for (int mb = 0; mb < 4; ++mb) {
+        hf[2 * mb] = ml_act_operand<DTYPE>(acc[mb], 0);
+        hf[2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb], 8);
+        ml_bias_init(acc[mb], bias + layer * 128, mb * 32, lhalf);
       }
-      ml_bias_init(acc[mb][0], bias + 128, mb * 32, lhalf);
-#pragma unroll
-      for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
-    }
-    {
-      const char* wa = w2buf + lrow * ML_ROWB + lhalf * 16;
+      const char* wa = (layer == 1 ? w2buf : w3buf) + lrow * ML_ROWB + lhalf * 16;
       uint4 af[2][4];
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) af[0][mb] = *reinterpret_cast<const uint4*>(wa + mb * 32 * ML_ROWB);
@@ -275,102 +297,48 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
         }
         ML_PIN();
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-#pragma unroll
-          for (int tb = 0; tb < ML_TB; ++tb) acc[mb][tb] = fc_mfma<DTYPE>(af[g & 1][mb], hf[tb][g], acc[mb][tb]);
-        }
-        ML_PIN();
-      }
-    }
-    // ---- layer 3: Y = H2 * W3^T, A operand taken from layer 2's accumulators ---------------------
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-#pragma unroll
-      for (int tb = 0; tb < ML_TB; ++tb) {
-        hf[tb][2 * mb] = ml_act_operand<DTYPE>(acc[mb][tb], 0);
-        hf[tb][2 * mb + 1] = ml_act_operand<DTYPE>(acc[mb][tb], 8);
-      }
-      // layer 3 is not transposed: register = token row, lane = feature -> one bias value per lane
-      const float b3v = bias[256 + mb * 32 + lrow];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mb][0][i] = b3v;
-#pragma unroll
-      for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
-    }
-    {
-      // acc[nb][tb] now accumulates Y[tb block rows][nb block features]
-      const char* wb = w3buf + lrow * ML_ROWB + lhalf * 16;
-      uint4 bfr[2][4];
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) bfr[0][nb] = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB);
-#pragma unroll
-      for (int g = 0; g < 8; ++g) {
-        if (g + 1 < 8) {
-#pragma unroll
-          for (int nb = 0; nb < 4; ++nb)
-            bfr[(g + 1) & 1][nb] = *reinterpret_cast<const uint4*>(wb + nb * 32 * ML_ROWB + (g + 1) * 32);
-        }
-        ML_PIN();
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-#pragma unroll
-          for (int tb = 0; tb < ML_TB; ++tb) acc[nb][tb] = fc_mfma<DTYPE>(hf[tb][g], bfr[g & 1][nb], acc[nb][tb]);
-        }
+        for (int mb = 0; mb < 4; ++mb) acc[mb] = fc_mfma<DTYPE>(af[g & 1][mb], hf[g], acc[mb]);
         ML_PIN();
       }
     }
     // every wavefront of the column has consumed this iteration's source rows: stores may alias them
     // (a wavefront that owns its column alone is ordered by its own data dependences)
     if (wpc > 1) __syncthreads();
-    const int row0 = it * rows_per_iter + sub * ML_ROWS;
+    {
+      // The lane owns output row lrow and, per 32-feature block, features (i/4)*8 + lhalf*4 + i%4: four 8-byte
+      // pieces go to the wavefront's LDS rows (64 bytes = one feature block of a row); read back in the
+      // memory-side layout, 16 rows x 64 bytes leave per store instruction.
+      const int row0 = it * rows_per_iter + sub * ML_ROWS;
+      char* rowp[2];
 #pragma unroll
-    for (int tb = 0; tb < ML_TB; ++tb) {
+      for (int rh = 0; rh < 2; ++rh) {
+        const int r = row0 + rh * 16 + lq;
+        long long off = -1;
+        if (col_ok && r < c_rows) off = dst_off(dst_start + r);
+        rowp[rh] = off >= 0 ? dbase + off * 2 : nullptr;
+      }
+      const unsigned y_at = (unsigned)lrow * 64 + lhalf * 8;
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        // registers 4*i4 .. 4*i4+3 are 4 consecutive rows
-        const int r0 = row0 + tb * 32 + i4 * 8 + lhalf * 4;
-        const int t0 = dst_start + r0;
-        // common case: all 4 rows exist and sit in one block (always true for a dense view)
-        const bool together = DST_T == 0 || (dst.block_shift >= 0 && (t0 & (dst.block_size - 1)) + 3 < dst.block_size);
-        if (col_ok && r0 + 3 < c_rows && together) {
-          const long long off0 = dst_off(t0);
-          if (off0 >= 0) {
+      for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              char* rowp = dbase + (off0 + (long long)e * dst.stride_token) * 2 + lrow * 2;
-#pragma unroll
-              for (int nb = 0; nb < 4; ++nb) {
-                const unsigned w = ml_pack2<DTYPE>(acc[nb][tb][i4 * 4 + e], 0.f);
-                *reinterpret_cast<unsigned short*>(rowp + nb * 64) = (unsigned short)(w & 0xffff);
-              }
-            }
-          }
-        } else if (col_ok && r0 < c_rows) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (r0 + e < c_rows) {
-              const long long off = dst_off(t0 + e);
-              if (off >= 0) {
-#pragma unroll
-                for (int nb = 0; nb < 4; ++nb) {
-                  const unsigned w = ml_pack2<DTYPE>(acc[nb][tb][i4 * 4 + e], 0.f);
-                  *reinterpret_cast<unsigned short*>(dbase + off * 2 + (nb * 32 + lrow) * 2) = (unsigned short)(w & 0xffff);
-                }
-              }
-            }
-          }
+        for (int i4 = 0; i4 < 4; ++i4) {
+          uint2 w;
+          w.x = ml_pack2<DTYPE>(acc[mb][i4 * 4 + 0], acc[mb][i4 * 4 + 1]);
+          w.y = ml_pack2<DTYPE>(acc[mb][i4 * 4 + 2], acc[mb][i4 * 4 + 3]);
+          *reinterpret_cast<uint2*>(xsw + y_at + ((i4 ^ swz) << 4)) = w;
         }
+        ml_wave_sync();
+        const uint4 y0 = *reinterpret_cast<const uint4*>(xsw + mem_at);
+        const uint4 y1 = *reinterpret_cast<const uint4*>(xsw + mem_at + 1024);
+        if (rowp[0]) *reinterpret_cast<uint4*>(rowp[0] + mb * 64) = y0;
+        if (rowp[1]) *reinterpret_cast<uint4*>(rowp[1] + mb * 64) = y1;
       }
     }
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-      ml_bias_init(acc[mb][0], bias, mb * 32, lhalf);
-#pragma unroll
-      for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
-    }
+    for (int mb = 0; mb < 4; ++mb) ml_bias_init(acc[mb], bias, mb * 32, lhalf);
   };
 
-  uint4 xa[ML_TB][8], xb[ML_TB][8], xc[ML_TB][8];
+  uint4 xa[8], xb[8];
   w1_load(0);
   w1_store(0);
   if (W1R && cf > 1) {
@@ -379,24 +347,11 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   }
   __syncthreads();   // block tables, biases and the first weights are in LDS
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    ml_bias_init(acc[mb][0], bias, mb * 32, lhalf);
-#pragma unroll
-    for (int tb = 1; tb < ML_TB; ++tb) acc[mb][tb] = acc[mb][0];
-  }
+  for (int mb = 0; mb < 4; ++mb) ml_bias_init(acc[mb], bias, mb * 32, lhalf);
   x_load(xa, 0);
-  if constexpr (XD == 2) {
-    x_load(xb, 1);
-    for (int q = 0; q < q_total; q += 3) {
-      stage(xa, xc, q);
-      if (q + 1 < q_total) stage(xb, xa, q + 1);
-      if (q + 2 < q_total) stage(xc, xb, q + 2);
-    }
-  } else {
-    for (int q = 0; q < q_total; q += 2) {
-      stage(xa, xb, q);
-      if (q + 1 < q_total) stage(xb, xa, q + 1);
-    }
+  for (int q = 0; q < q_total; q += 2) {
+    stage(xa, xb, q);
+    if (q + 1 < q_total) stage(xb, xa, q + 1);
   }
 }
 
@@ -430,11 +385,11 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && ML_ROWS * wpc * 2 <= c) wpc *= 2;
     const int cols_per_wg = ML_WAVES / wpc;
     dim3 grid((ncols + cols_per_wg - 1) / cols_per_wg, src->num_layers);
-    const size_t lds = 4 * ML_WBYTES + 3 * 128 * sizeof(float) + ML_WAVES * 2 * ML_TBL * sizeof(int);
+    const size_t lds = ML_LDS;
     KvView s = fc_make_view(src), d = fc_make_view(dst);
     auto table_mode = [&](const KvView& v, int last_token) {
       if (!v.block_tables) return 0;
-      return (v.block_shift >= 0 && (last_token >> v.block_shift) < ML_TBL) ? 1 : 2;
+      return (v.block_shift >= 0 && (last_token >> v.block_shift) < ML_TBLTOT / cols_per_wg) ? 1 : 2;
     };
     const int sm = table_mode(s, seg_start + c * cf - 1), dm = table_mode(d, dst_start + c - 1);
     // dense/dense, LDS-cached tables, or the general path through global tables
