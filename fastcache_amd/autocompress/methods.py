@@ -1,11 +1,13 @@
 """KV quantisation with the reference's call surface (``QuantizationMethod``,
 nanovllm/autocompress/methods.py:520-757), computed by HIP kernels.
 
-Built: ``int8`` (symmetric, one scale per row of the last dimension), ``int4`` and ``nf4`` (one scale per
-group of ``group_size`` elements, two codes per byte).  Two expressions of the reference do not run as
-written — the int4 packing applies ``|`` to floating tensors (:665) and the NF4 look-up indexes a table
-with ``uint8`` tensors (:725-733) — so for those the packing and look-up they describe are what is built.
-Not built: the fp8 cast variants and asymmetric int8 (``symmetric=False``), which raise.
+Built: ``int8`` (one scale per row of the last dimension; ``symmetric=False`` gives uint8 codes with a
+``(scale, zero point)`` pair per row), ``int4`` and ``nf4`` (one scale per group of ``group_size`` elements, two
+codes per byte), ``fp8`` / ``fp8_e4m3`` / ``fp8_e5m2`` (float8 codes, one scale for the tensor).  Three expressions
+of the reference do not run as written — the int4 packing applies ``|`` to floating tensors (:665), the NF4
+look-up indexes a table with ``uint8`` tensors (:725-733), and de-quantising asymmetric int8 multiplies
+``[..., D]`` codes by the ``[..., 2]`` parameter tensor (:726) — so for the first two the packing and look-up they
+describe are what is built, and the third raises here as it does there.
 """
 from __future__ import annotations
 
@@ -56,12 +58,17 @@ class QuantizationMethod:
             return self._quantize_int4(tensor)
         if t == self.QuantType.NF4:
             return self._quantize_nf4(tensor)
-        raise FastcacheError(f"{self.name}: the fp8 cast variants are not part of this build")
+        return self._quantize_fp8(tensor)
 
     def _quantize_int8(self, tensor: torch.Tensor):
         if not self._symmetric:
-            raise FastcacheError("asymmetric int8 quantisation is not part of this build")
+            return ops.quantize_rows_asym(tensor)       # (uint8 codes, [..., 2] = scale and zero point)
         return ops.quantize_rows(tensor, 8)
+
+    def _quantize_fp8(self, tensor: torch.Tensor):
+        """One scale for the tensor, handed out expanded to ``tensor[..., :1]``'s shape (methods.py:671-680)."""
+        q, scale = ops.quantize_fp8(tensor, e5m2=self._quant_type == self.QuantType.FP8_E5M2)
+        return q, scale.expand(tensor.shape[:-1] + (1,))
 
     def _quantize_int4(self, tensor: torch.Tensor):
         return ops.quantize_group4(tensor, self._group_size, nf4=False)
@@ -72,7 +79,10 @@ class QuantizationMethod:
     def dequantize(self, quantized: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype = torch.float16) -> torch.Tensor:
         t = self._quant_type
         if t == self.QuantType.INT8:
+            if quantized.dtype == torch.uint8:
+                raise FastcacheError("asymmetric int8 codes cannot be de-quantised: the reference's expression "
+                                     "multiplies [..., D] codes by the [..., 2] (scale, zero point) tensor")
             return ops.dequantize_rows(quantized, scale, dtype)
         if t in (self.QuantType.INT4, self.QuantType.NF4):
             return ops.dequantize_group4(quantized, scale, self._group_size, t == self.QuantType.NF4, dtype)
-        raise FastcacheError(f"{self.name}: the fp8 cast variants are not part of this build")
+        return ops.dequantize_fp8(quantized, scale, dtype)

@@ -1,5 +1,6 @@
-// Symmetric quantisation of KV rows: per-row int8 storage (4- or 8-bit range) and back, packed 4-bit
-// groups (integer and NF4), and quantise -> dequantise in one pass with a per-row or whole-tensor scale.
+// Quantisation of KV rows: symmetric per-row int8 storage (4- or 8-bit range) and back, asymmetric 8-bit rows,
+// packed 4-bit groups (integer and NF4), 8-bit floating point codes with one scale for the tensor, and
+// quantise -> dequantise in one pass with a per-row or whole-tensor scale.
 //
 // One wavefront per row of `d` elements.  The arithmetic follows what a tensor library does on a
 // tensor of the row's dtype, step by step: every intermediate (row maximum, scale, quotient) is
@@ -238,6 +239,125 @@ __global__ __launch_bounds__(256) void fake_quant_tensor_kernel(const char* __re
     qz_store<DTYPE>(y, i, qz_fake<DTYPE>(qz_load<DTYPE>(x, i), sc, qmax));
 }
 
+// ---- 8-bit floating point codes ------------------------------------------------------------------
+// Round to nearest even from an fp32 value.  E4M3 (finite-only variant: bias 7, largest value 448, codes 0x7f / 0xff
+// are NaN, no infinity): whatever rounds past 448, infinities and NaN included, becomes NaN.  E5M2 (bias 15, IEEE
+// style): whatever rounds past 57344 becomes infinity, NaN stays NaN.  Values under the smallest normal number are
+// rounded by adding the power of two whose unit in the last place is the target's subnormal spacing.
+template <int E5M2>
+__device__ __forceinline__ unsigned char qz_to_fp8(float f) {
+  unsigned u = __float_as_uint(f);
+  const unsigned sign = (u >> 24) & 0x80u;
+  u &= 0x7fffffffu;
+  unsigned r;
+  if constexpr (!E5M2) {
+    if (u >= (1087u << 20)) {                      // 480 and above
+      r = 0x7f;
+    } else if (u < (121u << 23)) {                 // below 2^-6: multiples of 2^-9
+      r = __float_as_uint(__uint_as_float(u) + __uint_as_float(141u << 23)) - (141u << 23);
+    } else {
+      const unsigned odd = (u >> 20) & 1u;
+      r = (u - (120u << 23) + 0x7ffffu + odd) >> 20;
+    }
+  } else {
+    if (u >= (143u << 23)) {                       // 65536 and above
+      r = u > 0x7f800000u ? 0x7f : 0x7c;
+    } else if (u < (113u << 23)) {                 // below 2^-14: multiples of 2^-16
+      r = __float_as_uint(__uint_as_float(u) + __uint_as_float(134u << 23)) - (134u << 23);
+    } else {
+      const unsigned odd = (u >> 21) & 1u;
+      r = (u - (112u << 23) + 0xfffffu + odd) >> 21;
+    }
+  }
+  return (unsigned char)(r | sign);
+}
+
+template <int E5M2>
+__device__ __forceinline__ float qz_from_fp8(unsigned char c) {
+  const unsigned sign = ((unsigned)c & 0x80u) << 24;
+  const unsigned mag = c & 0x7fu;
+  constexpr int MB = E5M2 ? 2 : 3, BIAS = E5M2 ? 15 : 7;
+  const unsigned e = mag >> MB, m = mag & ((1u << MB) - 1u);
+  float v;
+  if (E5M2 ? (e == 31u) : (mag == 0x7fu)) v = (E5M2 && m == 0u) ? INFINITY : __builtin_nanf("");
+  else if (e == 0u) v = (float)m * (E5M2 ? 1.52587890625e-05f : 0.001953125f);          // m * 2^(1 - BIAS - MB)
+  else v = __uint_as_float(((e + 127u - BIAS) << 23) | (m << (23 - MB)));
+  return __uint_as_float(__float_as_uint(v) | sign);
+}
+
+// scale = clamp(max|x| / 448, min=1e-8) over the whole tensor (both formats divide by 448), code = fp8(x / scale)
+template <int DTYPE, int E5M2>
+__global__ __launch_bounds__(256) void quantize_fp8_kernel(const char* __restrict__ x, long long n,
+                                                           const float* __restrict__ partial, int nparts,
+                                                           unsigned char* __restrict__ q, char* __restrict__ scale) {
+  __shared__ float wm[4];
+  float mx = 0.f;
+  bool has_nan = false;
+  for (int i = threadIdx.x; i < nparts; i += 256) {
+    const float v = partial[i];
+    has_nan |= v != v;
+    mx = fmaxf(mx, v);
+  }
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mx = __builtin_nanf("");
+  if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = wm[0];
+  for (int w = 1; w < 4; ++w) mx = (mx != mx || wm[w] != wm[w]) ? __builtin_nanf("") : fmaxf(mx, wm[w]);
+  float sc = qz_round<DTYPE>(mx / 448.f);
+  sc = qz_round<DTYPE>(sc != sc ? sc : fmaxf(sc, 1e-8f));
+  if (blockIdx.x == 0 && threadIdx.x == 0) qz_store<DTYPE>(scale, 0, sc);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    q[i] = qz_to_fp8<E5M2>(qz_round<DTYPE>(qz_load<DTYPE>(x, i) / sc));
+}
+
+// out = float(code) * scale, rounded to the output dtype (every fp8 value is exact in fp16 and bf16)
+template <int SDT, int ODT, int E5M2>
+__global__ __launch_bounds__(256) void dequantize_fp8_kernel(const unsigned char* __restrict__ q,
+                                                             const char* __restrict__ scale, long long n,
+                                                             char* __restrict__ out) {
+  const float sc = qz_load<SDT>(scale, 0);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    qz_store<ODT>(out, i, qz_from_fp8<E5M2>(q[i]) * sc);
+}
+
+// ---- asymmetric 8-bit rows -----------------------------------------------------------------------
+// scale = clamp((max - min) / 255, 1e-8), zero = clamp(round(-min / scale), 0, 255),
+// code = clamp(round((x - min) / scale), 0, 255); params[row] = (scale, zero) in the dtype of x
+template <int DTYPE>
+__global__ __launch_bounds__(256) void quantize_rows_asym_kernel(const char* __restrict__ x, long long rows, int d,
+                                                                 unsigned char* __restrict__ q,
+                                                                 char* __restrict__ params) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows) return;
+  const long long base = r * d;
+  float mn = INFINITY, mx = -INFINITY;
+  bool has_nan = false;
+  for (int j = lane; j < d; j += 64) {
+    const float v = qz_load<DTYPE>(x, base + j);
+    has_nan |= v != v;
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+  mn = -fc_wave_max(-mn);
+  mx = fc_wave_max(mx);
+  if (__any(has_nan)) mn = mx = __builtin_nanf("");
+  float sc = qz_round<DTYPE>(qz_round<DTYPE>(mx - mn) / 255.f);
+  sc = qz_round<DTYPE>(sc != sc ? sc : fmaxf(sc, 1e-8f));
+  float zp = rintf(qz_round<DTYPE>(-mn / sc));
+  zp = fminf(fmaxf(zp, 0.f), 255.f);
+  if (lane == 0) {
+    qz_store<DTYPE>(params, 2 * r, sc);
+    qz_store<DTYPE>(params, 2 * r + 1, zp);
+  }
+  for (int j = lane; j < d; j += 64) {
+    float t = qz_round<DTYPE>(qz_round<DTYPE>(qz_load<DTYPE>(x, base + j) - mn) / sc);
+    t = fminf(fmaxf(rintf(t), 0.f), 255.f);
+    q[base + j] = (t != t) ? (unsigned char)0 : (unsigned char)(int)t;
+  }
+}
+
 extern "C" int64_t fc_fake_quantize_workspace_bytes(void) { return QZ_PARTS * (int64_t)sizeof(float); }
 
 extern "C" int fc_fake_quantize(const void* x, void* y, int64_t rows, int32_t d, int32_t dtype, int32_t bits,
@@ -321,6 +441,86 @@ extern "C" int fc_dequantize_rows(const int8_t* q, const void* scale, int64_t ro
   else if (out_dtype == FC_F32 && scale_dtype == FC_BF16) DQ(FC_BF16, FC_F32);
   else { fc_set_error("%s: scale dtype %d with output dtype %d", who, scale_dtype, out_dtype); return FC_EUNSUPPORTED; }
 #undef DQ
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_quantize_fp8(const void* x, int64_t n, int32_t dtype, int32_t e5m2, uint8_t* q, void* scale,
+                               void* workspace, int64_t workspace_bytes, void* stream) {
+  const char* who = "fc_quantize_fp8";
+  FC_REQUIRE(x && q && scale, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(n >= 0, FC_EINVAL, "%s: bad size %lld", who, (long long)n);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+  FC_REQUIRE(workspace && workspace_bytes >= fc_fake_quantize_workspace_bytes(), FC_EINVAL,
+             "%s: needs a workspace of %lld bytes", who, (long long)fc_fake_quantize_workspace_bytes());
+  if (n == 0) return FC_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const int nparts = (int)((n + 255) / 256 < QZ_PARTS ? (n + 255) / 256 : QZ_PARTS);
+  const long long want = (n + 1023) / 1024;
+  const unsigned blocks = (unsigned)(want < 8192 ? want : 8192);
+#define F8(DT)                                                                                                       \
+  do {                                                                                                               \
+    hipLaunchKernelGGL((absmax_partial_kernel<DT>), dim3(nparts), dim3(256), 0, st, (const char*)x, (long long)n,   \
+                       (float*)workspace);                                                                           \
+    if (e5m2)                                                                                                        \
+      hipLaunchKernelGGL((quantize_fp8_kernel<DT, 1>), dim3(blocks), dim3(256), 0, st, (const char*)x, (long long)n, \
+                         (const float*)workspace, nparts, (unsigned char*)q, (char*)scale);                          \
+    else                                                                                                             \
+      hipLaunchKernelGGL((quantize_fp8_kernel<DT, 0>), dim3(blocks), dim3(256), 0, st, (const char*)x, (long long)n, \
+                         (const float*)workspace, nparts, (unsigned char*)q, (char*)scale);                          \
+  } while (0)
+  if (dtype == FC_F32) F8(FC_F32); else if (dtype == FC_F16) F8(FC_F16); else F8(FC_BF16);
+#undef F8
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_dequantize_fp8(const uint8_t* q, const void* scale, int64_t n, int32_t e5m2, int32_t scale_dtype,
+                                 int32_t out_dtype, void* out, void* stream) {
+  const char* who = "fc_dequantize_fp8";
+  FC_REQUIRE(q && scale && out, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(n >= 0, FC_EINVAL, "%s: bad size %lld", who, (long long)n);
+  if (n == 0) return FC_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const long long want = (n + 1023) / 1024;
+  const unsigned blocks = (unsigned)(want < 8192 ? want : 8192);
+#define D8(S, O)                                                                                                     \
+  do {                                                                                                               \
+    if (e5m2)                                                                                                        \
+      hipLaunchKernelGGL((dequantize_fp8_kernel<S, O, 1>), dim3(blocks), dim3(256), 0, st, (const unsigned char*)q,  \
+                         (const char*)scale, (long long)n, (char*)out);                                              \
+    else                                                                                                             \
+      hipLaunchKernelGGL((dequantize_fp8_kernel<S, O, 0>), dim3(blocks), dim3(256), 0, st, (const unsigned char*)q,  \
+                         (const char*)scale, (long long)n, (char*)out);                                              \
+  } while (0)
+  // the output dtype is the promotion of the two: equal dtypes, or fp32 when either side is fp32
+  if (scale_dtype == out_dtype) {
+    if (out_dtype == FC_F32) D8(FC_F32, FC_F32);
+    else if (out_dtype == FC_F16) D8(FC_F16, FC_F16);
+    else if (out_dtype == FC_BF16) D8(FC_BF16, FC_BF16);
+    else { fc_set_error("%s: dtype %d", who, out_dtype); return FC_EUNSUPPORTED; }
+  } else if (out_dtype == FC_F32 && scale_dtype == FC_F16) D8(FC_F16, FC_F32);
+  else if (out_dtype == FC_F32 && scale_dtype == FC_BF16) D8(FC_BF16, FC_F32);
+  else { fc_set_error("%s: scale dtype %d with output dtype %d", who, scale_dtype, out_dtype); return FC_EUNSUPPORTED; }
+#undef D8
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_quantize_rows_asym(const void* x, int64_t rows, int32_t d, int32_t dtype, uint8_t* q, void* params,
+                                     void* stream) {
+  const char* who = "fc_quantize_rows_asym";
+  FC_REQUIRE(x && q && params, FC_EINVAL, "%s: null pointer", who);
+  FC_REQUIRE(rows >= 0 && d > 0, FC_EINVAL, "%s: bad sizes rows=%lld d=%d", who, (long long)rows, d);
+  FC_REQUIRE(dtype == FC_F32 || dtype == FC_F16 || dtype == FC_BF16, FC_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (rows == 0) return FC_OK;
+  const long long blocks = (rows + 3) / 4;
+  FC_REQUIRE(blocks <= 2147483647LL, FC_EUNSUPPORTED, "%s: too many rows", who);
+  hipStream_t st = (hipStream_t)stream;
+#define QA(DT) hipLaunchKernelGGL((quantize_rows_asym_kernel<DT>), dim3((unsigned)blocks), dim3(256), 0, st,          \
+                                  (const char*)x, (long long)rows, d, (unsigned char*)q, (char*)params)
+  if (dtype == FC_F32) QA(FC_F32); else if (dtype == FC_F16) QA(FC_F16); else QA(FC_BF16);
+#undef QA
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }

@@ -312,6 +312,58 @@ def fake_quantize(x: torch.Tensor, bits: int, per_tensor: bool, out: Optional[to
     return (y, scale, amax) if return_params else y
 
 
+def quantize_rows_asym(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row asymmetric 8-bit quantisation: ``(q uint8 like x, params x.dtype [..., 2] = (scale, zero point))``."""
+    _lib.require_gpu(x, "x")
+    if x.dim() < 1 or x.numel() == 0:
+        raise FastcacheError("quantize_rows_asym: empty input")
+    xc = x.contiguous()
+    d = xc.shape[-1]
+    rows = xc.numel() // d
+    q = torch.empty(xc.shape, dtype=torch.uint8, device=x.device)
+    params = torch.empty(xc.shape[:-1] + (2,), dtype=x.dtype, device=x.device)
+    check(fn("fc_quantize_rows_asym")(xc.data_ptr(), rows, d, _lib.dtype_code(x.dtype), q.data_ptr(),
+                                      params.data_ptr(), current_stream()), "fc_quantize_rows_asym")
+    return q, params
+
+
+def _fp8_dtype(e5m2: bool) -> torch.dtype:
+    return torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+
+
+def quantize_fp8(x: torch.Tensor, e5m2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(x / scale).to(float8)`` with ``scale = clamp(max|x| / 448, 1e-8)`` over the whole tensor:
+    ``(codes as a float8 tensor like x, scale 0-dim in x.dtype)``."""
+    _lib.require_gpu(x, "x")
+    if x.numel() == 0:
+        raise FastcacheError("quantize_fp8: empty input")
+    xc = x.contiguous()
+    q = torch.empty(xc.shape, dtype=torch.uint8, device=x.device)
+    scale = torch.empty((), dtype=x.dtype, device=x.device)
+    nbytes = int(fn("fc_fake_quantize_workspace_bytes")())
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    check(fn("fc_quantize_fp8")(xc.data_ptr(), xc.numel(), _lib.dtype_code(x.dtype), int(bool(e5m2)), q.data_ptr(),
+                                scale.data_ptr(), ws.data_ptr(), nbytes, current_stream()), "fc_quantize_fp8")
+    return q.view(_fp8_dtype(e5m2)), scale
+
+
+def dequantize_fp8(q: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """``q.to(dtype) * scale`` for float8 codes and one scale for the tensor, with that expression's dtype promotion."""
+    _lib.require_gpu(q, "q")
+    _lib.require_gpu(scale, "scale")
+    if q.dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
+        raise FastcacheError(f"dequantize_fp8: float8 codes expected, got {q.dtype}")
+    # the reference hands the scale out expanded over the leading dimensions: every element is the same number
+    sc = scale.reshape(-1)[:1].contiguous()
+    out_dtype = torch.promote_types(dtype, sc.dtype)
+    qc = q.contiguous()
+    out = torch.empty(qc.shape, dtype=out_dtype, device=q.device)
+    check(fn("fc_dequantize_fp8")(qc.data_ptr(), sc.data_ptr(), qc.numel(), int(q.dtype == torch.float8_e5m2),
+                                  _lib.dtype_code(sc.dtype), _lib.dtype_code(out_dtype), out.data_ptr(),
+                                  current_stream()), "fc_dequantize_fp8")
+    return out
+
+
 def quantize_group4(x: torch.Tensor, group_size: int, nf4: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     """Groups of ``group_size`` consecutive elements -> ``(packed uint8 [..., D/2], scale [..., D/group_size])``."""
     _lib.require_gpu(x, "x")

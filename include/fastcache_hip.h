@@ -275,6 +275,30 @@ int fc_fake_quantize(const void* x, void* y, int64_t rows, int32_t d, int32_t dt
                      void* stream);
 
 /*
+ * 8-bit floating point codes with one scale for the whole tensor of n elements:
+ *   scale = clamp(max|x| / 448, min=1e-8) (448 for both formats, as the reference has it), code = fp8(x / scale),
+ * e5m2 == 0: E4M3, finite-only variant (largest value 448, 0x7f = NaN); e5m2 != 0: E5M2; conversion rounds to
+ * nearest even from the quotient rounded to `dtype`.  scale: one element in `dtype`.  Workspace as for
+ * fc_fake_quantize.  And the inverse, out = float(code) * scale rounded to out_dtype (dtype rules of
+ * fc_dequantize_rows).  Replaces QuantizationMethod._quantize_fp8 and the fp8 branch of dequantize
+ * (nanovllm/autocompress/methods.py:671-680, 735-736).
+ */
+int fc_quantize_fp8(const void* x, int64_t n, int32_t dtype, int32_t e5m2, uint8_t* q, void* scale,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+int fc_dequantize_fp8(const uint8_t* q, const void* scale, int64_t n, int32_t e5m2, int32_t scale_dtype,
+                      int32_t out_dtype, void* out, void* stream);
+
+/*
+ * Asymmetric 8-bit quantisation of rows of `d` elements:
+ *   scale = clamp((max - min) / 255, min=1e-8), zero = clamp(round(-min / scale), 0, 255),
+ *   q = clamp(round((x - min) / scale), 0, 255) as uint8; params[row] = (scale, zero) in the dtype of x;
+ * every intermediate rounded to that dtype.  Replaces the symmetric=False branch of
+ * QuantizationMethod._quantize_int8 (nanovllm/autocompress/methods.py:644-651).
+ */
+int fc_quantize_rows_asym(const void* x, int64_t rows, int32_t d, int32_t dtype, uint8_t* q, void* params,
+                          void* stream);
+
+/*
  * 4-bit quantisation of groups of `group_size` consecutive elements, two codes per byte (element 2j in
  * the low nibble), one scale per group in the dtype of x.
  *   nf4 == 0: scale = clamp(max|x| / 7, 1e-8), code = clamp(round(x / scale), -8, 7) + 8;

@@ -23,6 +23,9 @@ Pinning status (what independent check fixes each restatement; see tests/test_or
                                      forms (zero covariance, identity rotation); the kvpress package itself is
                                      unavailable offline: PARITY UNPINNED beyond the published formula
   presses.fake_quantize               numpy float16 arithmetic step by step, hand-worked rows, idempotence
+  autocompress.quantize_fp8 / quantize_int8_asymmetric
+                                      the float8 cast against a brute-force nearest-code search (ties, both formats),
+                                      hand-worked rows, numpy float16 arithmetic step by step
   blocks.*                           invariants of the free deque / ref counts, hand-worked cases
   attention.decode_attention         float64 loops; flash-attn itself is unavailable offline:
                                      PARITY UNPINNED beyond the mathematical definition

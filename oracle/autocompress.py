@@ -79,6 +79,31 @@ def quantize_int8(tensor: torch.Tensor):
     return (tensor / scale).round().clamp(-128, 127).to(torch.int8), scale
 
 
+def quantize_int8_asymmetric(tensor: torch.Tensor):
+    """methods.py:644-651 (``symmetric=False``): uint8 codes and ``[..., 2]`` = (scale, zero point)."""
+    x_min = tensor.amin(dim=-1, keepdim=True)
+    x_max = tensor.amax(dim=-1, keepdim=True)
+    scale = (x_max - x_min) / 255.0
+    scale = scale.clamp(min=1e-8)
+    zero_point = (-x_min / scale).round().clamp(0, 255)
+    quantized = ((tensor - x_min) / scale).round().clamp(0, 255).to(torch.uint8)
+    return quantized, torch.cat([scale, zero_point], dim=-1)
+
+
+def quantize_fp8(tensor: torch.Tensor, e5m2: bool = False):
+    """methods.py:671-680: one scale for the tensor (448 for both formats), torch's own float8 cast."""
+    dtype = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+    scale = tensor.abs().amax() / 448.0
+    scale = scale.clamp(min=1e-8)
+    quantized = (tensor / scale).to(dtype)
+    return quantized, scale.expand_as(tensor[..., :1])
+
+
+def dequantize_fp8(quantized: torch.Tensor, scale: torch.Tensor, dtype=torch.float16):
+    """methods.py:735-736."""
+    return quantized.to(dtype) * scale
+
+
 def quantize_int4(tensor: torch.Tensor, group_size: int):
     """methods.py:654-669.  The reference packs with ``|`` on the floating ``quantized`` tensor, which torch
     rejects; the packing it describes (low nibble = even element + 8, high nibble = odd element + 8) is done

@@ -168,8 +168,89 @@ def test_quantization_method_bit_exact(dev, dtype, kind):
         rq, rs = (oa.quantize_int4 if kind == "int4" else oa.quantize_nf4)(X, 32)
         assert s.shape == (2, 3, 50, 4) and torch.equal(q.cpu(), rq) and torch.equal(s.cpu(), rs)
         assert torch.equal(qm2.dequantize(q, s, dtype).cpu(), oa.dequantize_4bit(rq, rs, 32, kind == "nf4", dtype))
+
+
+def _fp8_bits(t):
+    return t.view(torch.uint8)
+
+
+@pytest.mark.parametrize("e5m2", [False, True])
+def test_fp8_cast_every_half_and_bfloat_value(dev, e5m2):
+    """Every fp16 and every bf16 bit pattern with |x| <= 448, in a tensor whose largest magnitude is 448 so that the
+    scale is exactly 1: the codes are the float8 cast itself, compared with torch's CPU cast bit for bit
+    (subnormal targets, ties, both signs, zeros)."""
+    for dtype in (torch.float16, torch.bfloat16):
+        allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+        x = allv[allv.float().abs() <= 448]
+        assert float(x.float().abs().max()) == 448.0 and x.numel() > 30000
+        q, s = ops.quantize_fp8(x.to(dev), e5m2=e5m2)
+        rq, rs = oa.quantize_fp8(x, e5m2)
+        assert float(s) == 1.0 and float(rs.reshape(-1)[0]) == 1.0
+        assert q.dtype == rq.dtype and torch.equal(_fp8_bits(q.cpu()), _fp8_bits(rq))
+        # and back: every code times a scale
+        sc = torch.tensor(0.37, dtype=dtype)
+        got = ops.dequantize_fp8(q, sc.to(dev), dtype)
+        assert torch.equal(got.cpu(), oa.dequantize_fp8(rq, sc, dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["fp8", "fp8_e4m3", "fp8_e5m2"])
+def test_quantization_method_fp8_bit_exact(dev, dtype, kind):
+    """QuantizationMethod fp8: float8 codes, the expanded whole-tensor scale and the de-quantised values against
+    the eager expressions on the CPU, bit for bit; fp32 inputs reach the cast unrounded."""
+    g = torch.Generator().manual_seed(len(kind) + 3)
+    X = (torch.randn(2, 3, 50, 128, generator=g) * 1.7).to(dtype)
+    V = (torch.randn(2, 3, 50, 128, generator=g) * torch.logspace(-6, 1, 128)).to(dtype)   # reaches float8 subnormals
+    qm = ac.QuantizationMethod(kind)
+    e5m2 = kind == "fp8_e5m2"
+    (qk, sk), (qv, sv) = qm.compress(X.to(dev), V.to(dev))
+    for x, q, s in ((X, qk, sk), (V, qv, sv)):
+        rq, rs = oa.quantize_fp8(x, e5m2)
+        assert q.dtype == rq.dtype and q.shape == rq.shape and torch.equal(_fp8_bits(q.cpu()), _fp8_bits(rq))
+        assert s.dtype == dtype and s.shape == rs.shape == x.shape[:-1] + (1,) and torch.equal(s.cpu(), rs)
+        for out_dtype in (dtype, torch.float32):
+            got = qm.dequantize(q, s, out_dtype)
+            ref = oa.dequantize_fp8(rq, rs, out_dtype)
+            assert got.dtype == ref.dtype and torch.equal(got.cpu(), ref)
+    assert qm.name == ("quant_fp8_e5m2" if e5m2 else "quant_fp8_e4m3") and qm.compression_ratio == 2.0
+
+
+def test_fp8_special_tensors(dev):
+    """An all-zero tensor (scale floored at 1e-8, or at 0 in fp16 where 1e-8 underflows: 0/0 = NaN codes), a NaN in
+    the tensor (every code NaN), one element."""
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        for x in (torch.zeros(4, 8), torch.tensor([[1.0, float("nan"), -2.0, 0.5]]), torch.tensor([[-3.0]])):
+            x = x.to(dtype)
+            q, s = ops.quantize_fp8(x.to(dev))
+            rq, rs = oa.quantize_fp8(x)
+            assert torch.equal(q.cpu().float().isnan(), rq.float().isnan())
+            ok = ~rq.float().isnan()
+            assert torch.equal(_fp8_bits(q.cpu())[ok], _fp8_bits(rq)[ok])
+            assert torch.equal(s.cpu().reshape(-1)[:1].float().nan_to_num(-1.0), rs.reshape(-1)[:1].float().nan_to_num(-1.0))
     with pytest.raises(FastcacheError):
-        ac.QuantizationMethod("fp8").compress(X.to(dev), V.to(dev))
+        ops.dequantize_fp8(torch.zeros(4, dtype=torch.int8, device=dev), torch.ones((), device=dev), torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 5, 128), (7, 40), (1000, 128), (2, 1)])
+def test_quantization_method_asymmetric_int8_bit_exact(dev, dtype, shape):
+    """symmetric=False: uint8 codes, scale and zero point per row against the eager expression; rows that are
+    constant (scale floored), all positive, all negative."""
+    g = torch.Generator().manual_seed(shape[0])
+    x = (torch.randn(*shape, generator=g) * 2.5 + 0.7).to(dtype)
+    x[0] = 1.25
+    if shape[0] > 2:
+        x[1] = x[1].abs() + 0.5
+        x[2] = -x[2].abs() - 0.5
+    qm = ac.QuantizationMethod("int8", symmetric=False)
+    q, p = qm._quantize(x.to(dev))
+    rq, rp = oa.quantize_int8_asymmetric(x)
+    assert q.dtype == torch.uint8 and q.shape == rq.shape and torch.equal(q.cpu(), rq)
+    assert p.dtype == dtype and p.shape == rp.shape == x.shape[:-1] + (2,)
+    assert torch.equal(p.cpu()[..., 0], rp[..., 0])
+    assert bool((p.cpu()[..., 1].float() == rp[..., 1].float()).all())        # +0 and -0 compare equal
+    with pytest.raises(FastcacheError):
+        qm.dequantize(q, p, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])

@@ -518,3 +518,57 @@ def test_expected_attention_oracle_brute_force_and_closed_forms():
     # without the value norm the scores of the scored keys sum to one per row
     p = op.expected_attention_score(k, v, mu_bf, None, n_sink=n_sink, use_vnorm=False)
     torch.testing.assert_close(p[:, :, n_sink:].sum(-1), torch.ones(B, Hkv), rtol=1e-5, atol=0)
+
+
+def test_fp8_and_asymmetric_int8_oracle_by_brute_force_and_hand():
+    """oracle.autocompress.quantize_fp8 / quantize_int8_asymmetric.  The float8 cast they lean on is pinned against
+    a brute-force search of the nearest representable value (the 256 codes decoded by their bit fields: sign,
+    exponent, mantissa; ties to the even mantissa; past the largest finite value NaN for E4M3, infinity for E5M2);
+    the scale and the asymmetric codes against hand-worked rows and step-by-step numpy float16 arithmetic."""
+    from oracle import autocompress as oa
+    for e5m2 in (False, True):
+        mb, bias = (2, 15) if e5m2 else (3, 7)
+        vals = []
+        for c in range(128):
+            e, m = c >> mb, c & ((1 << mb) - 1)
+            if (e == 31) if e5m2 else (c == 0x7F):
+                vals.append(float("inf") if e5m2 and m == 0 else float("nan"))
+            else:
+                vals.append(m * 2.0 ** (1 - bias - mb) if e == 0 else (1 + m / 2 ** mb) * 2.0 ** (e - bias))
+        finite = np.array([v for v in vals if np.isfinite(v)])
+        g = torch.Generator().manual_seed(3 + e5m2)
+        x = torch.cat([torch.randn(4000, generator=g) * s for s in (448 / 3, 1.0, 2.0 ** -7, 2.0 ** -15)])
+        x = torch.cat([x, torch.tensor(finite[:-1] + np.diff(finite) / 2, dtype=torch.float32)])      # exact ties
+        x = x.float().clamp(-448, 448)
+        x[0] = 448.0                                               # largest magnitude exactly 448 -> scale 1
+        q, s = oa.quantize_fp8(x[:, None], e5m2)
+        assert float(s.reshape(-1)[0]) == 1.0 and s.shape == (x.numel(), 1)
+        codes = q.view(torch.uint8).numpy()[:, 0]
+        for xv, c in zip(x.double().numpy()[::7], codes[::7]):
+            d = np.abs(finite - abs(xv))
+            best = np.flatnonzero(d == d.min())
+            want = best[0] if len(best) == 1 else [b for b in best if b % 2 == 0][0]    # tie: even mantissa
+            assert (c & 0x7F) == want and (c >> 7) == (1 if np.signbit(xv) else 0), (xv, c, want)
+    # scale: 448 for both formats, floor 1e-8, expanded to [..., 1]
+    q, s = oa.quantize_fp8(torch.tensor([[224.0, -1.0], [0.5, 0.0]]), False)
+    assert s.shape == (2, 1) and float(s[0]) == 0.5 and q.float().tolist() == [[448.0, -2.0], [1.0, 0.0]]
+    assert float(oa.quantize_fp8(torch.zeros(2, 2), True)[1].reshape(-1)[0]) == np.float32(1e-8)
+    assert oa.dequantize_fp8(q, s, torch.float32).tolist() == [[224.0, -1.0], [0.5, 0.0]]
+    # asymmetric int8 by hand: row [-1, 0, 1, 4.1] -> scale 5.1/255 = 0.02, zero = 50, codes [0, 50, 100, 255]
+    q, p = oa.quantize_int8_asymmetric(torch.tensor([[-1.0, 0.0, 1.0, 4.1]], dtype=torch.float64))
+    assert q.tolist() == [[0, 50, 100, 255]] and abs(p[0, 0].item() - 0.02) < 1e-12 and p[0, 1].item() == 50.0
+    # a constant row: scale floored, every code 0, zero point clamped to [0, 255]
+    q, p = oa.quantize_int8_asymmetric(torch.full((1, 4), -3.0))
+    assert q.tolist() == [[0, 0, 0, 0]] and p[0, 1].item() == 255.0
+    # float16 rows step by step in numpy
+    g = torch.Generator().manual_seed(21)
+    X = (torch.randn(6, 40, generator=g) * 2 + 0.3).half()
+    q, p = oa.quantize_int8_asymmetric(X)
+    xn = X.numpy()
+    mn, mx = xn.min(-1, keepdims=True), xn.max(-1, keepdims=True)
+    f32, f16 = np.float32, np.float16
+    sc = (f32((f32(mx) - f32(mn)).astype(f16)) / f32(255)).astype(f16)
+    zp = np.clip(np.rint(f32((-f32(mn) / f32(sc)).astype(f16))), 0, 255)
+    codes = np.clip(np.rint(f32((f32((f32(xn) - f32(mn)).astype(f16)) / f32(sc)).astype(f16))), 0, 255)
+    assert np.array_equal(q.numpy(), codes.astype(np.uint8))
+    assert np.array_equal(p[:, 0].numpy(), sc[:, 0]) and np.array_equal(p[:, 1].float().numpy(), zp[:, 0])
