@@ -216,10 +216,12 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
     }
   };
   // Re-laying through this wavefront's 2 KB of LDS: rows of 64 bytes, the four 16-byte pieces of a row XOR-ed
-  // with (row / 4) % 4 so that the memory-side accesses (4 rows per 16 lanes) and the operand-side accesses
-  // (16 rows, same piece, per 16 lanes) each touch every bank once.
-  const unsigned mem_at = (unsigned)lq * 64 + ((lp ^ ((lq >> 2) & 3)) << 4);   // row lq; row 16 + lq is 1024 further
-  const unsigned swz = (lrow >> 2) & 3;
+  // with a 2-bit function of the row number chosen so that the operand-side accesses (consecutive rows, same
+  // piece) touch every bank once whether 8 rows share a 128-byte bank window or 16 rows a 256-byte one:
+  // rows r, r+2, r+4, r+6 and rows r, r+4, r+8, r+12 all get different pieces.
+  auto piece_swz = [](int r) { return (unsigned)((((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1)); };
+  const unsigned mem_at = (unsigned)lq * 64 + ((lp ^ piece_swz(lq)) << 4);   // row lq; row 16 + lq is 1024 further
+  const unsigned swz = piece_swz(lrow);
   const unsigned op_at0 = (unsigned)lrow * 64 + (((0 + lhalf) ^ swz) << 4);    // k-step 0 of the pair: pieces 0, 1
   const unsigned op_at1 = (unsigned)lrow * 64 + (((2 + lhalf) ^ swz) << 4);    // k-step 1: pieces 2, 3
   auto relay_put = [&](uint4 lo_rows, uint4 hi_rows) {
@@ -317,7 +319,10 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
         if (col_ok && r < c_rows) off = dst_off(dst_start + r);
         rowp[rh] = off >= 0 ? dbase + off * 2 : nullptr;
       }
-      const unsigned y_at = (unsigned)lrow * 64 + lhalf * 8;
+      // (a half-wave writes one 8-byte half per row, so rows that share a piece position in a bank window keep
+      // their halves swapped: bit 3 xor bit 4 of the row number)
+      const unsigned y_at = (unsigned)lrow * 64 + (((lhalf ^ (lrow >> 3) ^ (lrow >> 4)) & 1) << 3);
+      const bool swap0 = (lq >> 3) & 1;     // row lq has its halves swapped; row 16 + lq the opposite
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
@@ -330,8 +335,10 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
         ml_wave_sync();
         const uint4 y0 = *reinterpret_cast<const uint4*>(xsw + mem_at);
         const uint4 y1 = *reinterpret_cast<const uint4*>(xsw + mem_at + 1024);
-        if (rowp[0]) *reinterpret_cast<uint4*>(rowp[0] + mb * 64) = y0;
-        if (rowp[1]) *reinterpret_cast<uint4*>(rowp[1] + mb * 64) = y1;
+        if (rowp[0])
+          *reinterpret_cast<uint4*>(rowp[0] + mb * 64) = swap0 ? make_uint4(y0.z, y0.w, y0.x, y0.y) : y0;
+        if (rowp[1])
+          *reinterpret_cast<uint4*>(rowp[1] + mb * 64) = swap0 ? y1 : make_uint4(y1.z, y1.w, y1.x, y1.y);
       }
     }
 #pragma unroll
