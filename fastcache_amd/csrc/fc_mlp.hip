@@ -102,7 +102,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
                                                             const char* __restrict__ b1, const char* __restrict__ w2,
                                                             const char* __restrict__ b2, const char* __restrict__ w3,
                                                             const char* __restrict__ b3, int cf, int seg_start,
-                                                            int c_rows, int dst_start, int wpc, int ncols) {
+                                                            int c_rows, int dst_start, int wpc, int ncols, int ncg) {
   extern __shared__ __align__(16) char lds[];
   char* w1buf = lds;                       // 2 x ML_WBYTES
   char* w2buf = lds + 2 * ML_WBYTES;       // permuted
@@ -112,16 +112,16 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   char* xsw = lds + 4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + (threadIdx.x >> 6) * ML_XS;
 
   const int l = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane & 31, lhalf = lane >> 5;
   const int lq = lane >> 2, lp = lane & 3;   // memory-side layout: row lq (and 16 + lq), 16-byte piece lp of 64 bytes
   const int cols_per_wg = ML_WAVES / wpc;
-  const int col = blockIdx.x * cols_per_wg + wave / wpc;
   const int sub = wave % wpc;
-  const bool col_ok = col < ncols;
   const int H = src.num_kv_heads;
-  const int b = col_ok ? col / H : 0, h = col_ok ? col - (col / H) * H : 0;
   const int K1 = cf * 128;
+  // the column this wavefront works on; a workgroup takes column groups blockIdx.x, blockIdx.x + gridDim.x, ...
+  int col = 0, b = 0, h = 0;
+  bool col_ok = false;
 
   // this column's block-table rows (source and destination), so that no row address waits on a table read;
   // filled by the wavefronts that share the column
@@ -129,13 +129,15 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   int* stbl = tbls + (wave / wpc) * tcap;
   int* dtbl = stbl + ML_TBLTOT;
   const int s_last = seg_start + c_rows * cf - 1, d_last = dst_start + c_rows - 1;
-  // also for a wavefront whose column is past the last one (b = 0): its loads are unconditional and need valid addresses
-  if (SRC_T == 1)
-    for (int i = sub * 64 + lane; i <= (s_last >> src.block_shift); i += 64 * wpc)
-      stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
-  if (col_ok && DST_T == 1)
-    for (int i = sub * 64 + lane; i <= (d_last >> dst.block_shift); i += 64 * wpc)
-      dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
+  auto fill_tables = [&]() {
+    // also for a wavefront whose column is past the last one (b = 0): its loads are unconditional and need valid addresses
+    if (SRC_T == 1)
+      for (int i = sub * 64 + lane; i <= (s_last >> src.block_shift); i += 64 * wpc)
+        stbl[i] = src.block_tables[(long long)b * src.table_stride + i];
+    if (col_ok && DST_T == 1)
+      for (int i = sub * 64 + lane; i <= (d_last >> dst.block_shift); i += 64 * wpc)
+        dtbl[i] = dst.block_tables[(long long)b * dst.table_stride + i];
+  };
   auto src_off = [&](int s) -> long long {
     if (SRC_T == 0) return (long long)b * src.stride_batch + (long long)s * src.stride_token;
     if (SRC_T == 1) {
@@ -195,8 +197,8 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   const int rows_per_iter = ML_ROWS * wpc;
   const int n_iter = (c_rows + rows_per_iter - 1) / rows_per_iter;
   const int q_total = n_iter * cf;      // W1 chunk q = (iteration q / cf, token kc = q % cf) sits in buffer q & 1
-  const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lp * 16;
-  char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2 + lp * 16;
+  const char* sbase = nullptr;   // this lane's piece of token 0 of the column's head, per column group
+  char* dbase = nullptr;
 
   // X rows of chunk q: xf[2*c4 + rh] holds bytes [64*c4 + 16*lp, +16) of the token row of output row 16*rh + lq
   auto x_load = [&](uint4 (&xf)[8], int q) {
@@ -346,20 +348,51 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   };
 
   uint4 xa[8], xb[8];
-  w1_load(0);
-  w1_store(0);
-  if (W1R && cf > 1) {
-    w1_load(1);
-    w1_store(1);
+  if (W1R) {
+    w1_load(0);
+    w1_store(0);
+    if (cf > 1) {
+      w1_load(1);
+      w1_store(1);
+    }
   }
-  __syncthreads();   // block tables, biases and the first weights are in LDS
+  for (int cg = blockIdx.x; cg < ncg; cg += gridDim.x) {
+    if (cg != (int)blockIdx.x) __syncthreads();   // every wavefront is done with the previous group's tables and W1 buffers
+    col = cg * cols_per_wg + wave / wpc;
+    col_ok = col < ncols;
+    b = col_ok ? col / H : 0;
+    h = col_ok ? col - (col / H) * H : 0;
+    sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lp * 16;
+    dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2 + lp * 16;
+    fill_tables();
+    if (!W1R) {
+      w1_load(0);
+      w1_store(0);
+    }
+    __syncthreads();   // block tables, biases and the first weights are in LDS
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) ml_bias_init(acc[mb], bias, mb * 32, lhalf);
-  x_load(xa, 0);
-  for (int q = 0; q < q_total; q += 2) {
-    stage(xa, xb, q);
-    if (q + 1 < q_total) stage(xb, xa, q + 1);
+    for (int mb = 0; mb < 4; ++mb) ml_bias_init(acc[mb], bias, mb * 32, lhalf);
+    x_load(xa, 0);
+    for (int q = 0; q < q_total; q += 2) {
+      stage(xa, xb, q);
+      if (q + 1 < q_total) stage(xb, xa, q + 1);
+    }
+    // the streaming variant is launched with one column group per workgroup (its groups are long, and the
+    // loop would cost it registers it does not have)
+    if (!W1R) break;
   }
+}
+
+// compute units of the current device (0 if the query fails)
+static int ml_compute_units() {
+  static int cus[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus[dev] = n;
+  }
+  return cus[dev];
 }
 
 extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int32_t seg_start, int32_t count,
@@ -391,7 +424,27 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     int wpc = 1;
     while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && ML_ROWS * wpc * 2 <= c) wpc *= 2;
     const int cols_per_wg = ML_WAVES / wpc;
-    dim3 grid((ncols + cols_per_wg - 1) / cols_per_wg, src->num_layers);
+    // One workgroup occupies a compute unit (its LDS), and loading the weights costs it a few microseconds.
+    // When a column group is short work, let each workgroup walk several groups of its layer; pick the number
+    // per workgroup that minimises rounds * (groups * time per group + start-up) in a coarse model.
+    const int ncg = (ncols + cols_per_wg - 1) / cols_per_wg;
+    int gx = ncg;
+    {
+      const int ncu = ml_compute_units();
+      const int n_iter = (c + ML_ROWS * wpc - 1) / (ML_ROWS * wpc);
+      const double t_group = 1.5 * n_iter * (cf + 2), t_start = 4.0;   // microseconds, roughly
+      double best = -1.0;
+      for (int per = 1; cf <= 2 && ncu > 0 && per <= ncg && per <= 64; ++per) {
+        const int g = (ncg + per - 1) / per;
+        const long long rounds = ((long long)g * src->num_layers + ncu - 1) / ncu;
+        const double cost = (double)rounds * (((ncg + g - 1) / g) * t_group + t_start);
+        if (best < 0 || cost < best) {
+          best = cost;
+          gx = g;
+        }
+      }
+    }
+    dim3 grid(gx, src->num_layers);
     const size_t lds = ML_LDS;
     KvView s = fc_make_view(src), d = fc_make_view(dst);
     auto table_mode = [&](const KvView& v, int last_token) {
@@ -406,7 +459,7 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
     FC_ALLOW_LDS((mlp_kernel<DT, ST, DTT, WR>), (int)lds);                                                    \
     hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT, WR>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,   \
                        (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,             \
-                       (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols);                               \
+                       (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols, ncg);                          \
   } while (0)
 #define ML_DISPATCH(DT, WR)                      \
   switch (mode) {                                \
