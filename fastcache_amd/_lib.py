@@ -74,6 +74,8 @@ SIGNATURES = {
     "fc_dequantize_rows": (C.c_int, [_VP, _VP, C.c_int64, _I, _I, _I, _VP, _VP]),
     "fc_fake_quantize_workspace_bytes": (C.c_int64, []),
     "fc_fake_quantize": (C.c_int, [_VP, _VP, C.c_int64, _I, _I, _I, _I, _VP, _VP, _VP, C.c_int64, _VP]),
+    "fc_key_channel_energy": (C.c_int, [_V, _VP, _VP]),
+    "fc_key_channel_zero": (C.c_int, [_V, _VP, _VP]),
     "fc_quantize_fp8": (C.c_int, [_VP, C.c_int64, _I, _I, _VP, _VP, _VP, C.c_int64, _VP]),
     "fc_dequantize_fp8": (C.c_int, [_VP, _VP, C.c_int64, _I, _I, _I, _VP, _VP]),
     "fc_quantize_rows_asym": (C.c_int, [_VP, C.c_int64, _I, _I, _VP, _VP, _VP]),

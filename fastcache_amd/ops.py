@@ -46,6 +46,23 @@ def knorm_mean_score(keys: FcKvView, device, score_stride: Optional[int] = None)
     return out
 
 
+def key_channel_energy(keys: FcKvView, device) -> torch.Tensor:
+    """Sum over each sequence's tokens of ``k^2`` per head-dimension channel -> fp32 ``[L, B, Hkv, 128]``."""
+    out = torch.empty((keys.num_layers, keys.batch, keys.num_kv_heads, keys.head_dim), dtype=torch.float32, device=device)
+    check(fn("fc_key_channel_energy")(C.byref(keys), out.data_ptr(), current_stream()), "fc_key_channel_energy")
+    return out
+
+
+def key_channel_zero(keys: FcKvView, prune: torch.Tensor) -> None:
+    """Zero, in place and for every token, the channels with ``prune[l, b, h, d] != 0`` (uint8 ``[L, B, Hkv, 128]``)."""
+    _lib.require_gpu(prune, "prune")
+    want = (keys.num_layers, keys.batch, keys.num_kv_heads, keys.head_dim)
+    if prune.dtype != torch.uint8 or tuple(prune.shape) != want:
+        raise FastcacheError(f"key_channel_zero: prune must be uint8 {want}, got {prune.dtype} {tuple(prune.shape)}")
+    pc = prune.contiguous()
+    check(fn("fc_key_channel_zero")(C.byref(keys), pc.data_ptr(), current_stream()), "fc_key_channel_zero")
+
+
 def snapkv_splits(keys: FcKvView, num_q_heads: int, window: int) -> int:
     """Key ranges per column for :func:`snapkv_score`.  Measured on MI355X (window 64, group of 4-7 heads): with
     1000 or more (layer, sequence, kv head) columns one workgroup per column is fastest; below that the GPU is not

@@ -305,6 +305,100 @@ class RandomPress(ScorerPress):
         return torch.rand(keys.shape[:3], dtype=torch.float32, device=keys.device, generator=g)
 
 
+@dataclass
+class ThinKPress(ScorerPress):
+    """Prune head-dimension channels of the keys instead of tokens (ThinK): the ``key_channel_compression_ratio``
+    fraction of channels with the lowest ``mean_window(q^2) * mean_tokens(k^2)`` per (batch, kv head) is set to
+    zero for every token, in place; the query statistic is averaged over the query heads of the group.  Values and
+    the cache length are unchanged.  The statistics are formed in fp32 (kvpress forms them in the tensor dtype) and
+    ties go to the lowest channel index."""
+    key_channel_compression_ratio: float = 0.0
+    window_size: int = 32
+
+    def __post_init__(self):
+        assert 0 <= self.key_channel_compression_ratio < 1, "Compression ratio must be between 0 and 1"
+        self.compression_ratio = 0.0
+        self.totalTime = 0
+
+    def channel_scores(self, module, hidden_states, keys, kwargs) -> torch.Tensor:
+        """fp32 ``[B, Hkv, D]``."""
+        B, Hkv, S, D = keys.shape
+        q = SnapKVPress(window_size=self.window_size).window_queries(module, hidden_states, kwargs)   # [B, Hq, W, D]
+        q_energy = q.float().pow(2).mean(dim=2).view(B, Hkv, q.shape[1] // Hkv, D).mean(dim=2)
+        k_energy = ops.key_channel_energy(_lib.dense_view(keys), keys.device)[0] / S
+        return q_energy * k_energy
+
+    def compress(self, module, hidden_states, keys, values, attentions, kwargs):
+        if self.key_channel_compression_ratio == 0:
+            return keys, values
+        B, Hkv, S, D = keys.shape
+        n_pruned = int(D * self.key_channel_compression_ratio)
+        if n_pruned == 0:
+            return keys, values
+        scores = self.channel_scores(module, hidden_states, keys, kwargs)
+        idx = ops.topk_select((-scores).contiguous(), n_pruned).long()             # the lowest scores
+        prune = torch.zeros((B, Hkv, D), dtype=torch.uint8, device=keys.device).scatter_(-1, idx, 1)
+        ops.key_channel_zero(_lib.dense_view(keys), prune[None])
+        return keys, values
+
+
+@dataclass
+class SimLayerKVPress(ScorerPress):
+    """Layer-wise pruning (SimLayerKV): a layer is "lazy" when its last ``n_last`` queries put more than
+    ``lazy_threshold`` of their attention, averaged over batch, heads and those queries, on the first ``n_initial``
+    and the last ``n_recent`` of the other keys; a lazy layer keeps only the first ``n_initial`` tokens and the last
+    ``n_recent - n_last`` ones, other layers keep everything.  ``compression_ratios`` records what each call removed."""
+    lazy_threshold: float = 1.0
+    n_last: int = 1
+    n_recent: int = 1024
+    n_initial: int = 4
+
+    def __post_init__(self):
+        assert 0.0 <= self.lazy_threshold <= 1.0, "lazy_threshold should be in [0, 1]"
+        assert self.n_recent > self.n_last, "n_recent must exceed n_last"
+        self.compression_ratios = []
+        self.totalTime = 0
+
+    @property
+    def compression_ratio(self):
+        if not self.compression_ratios:
+            return 0.0
+        return sum(self.compression_ratios) / len(self.compression_ratios)
+
+    @compression_ratio.setter
+    def compression_ratio(self, value):
+        if isinstance(value, property) or value == 0.0:      # the dataclass default of the base class
+            return
+        raise AttributeError(f"compression ratio cannot be set for {type(self).__name__}")
+
+    def lazy_score(self, module, hidden_states, keys, kwargs) -> float:
+        """Share of the last queries' attention that lands on the initial and the recent keys."""
+        B, Hkv, S, D = keys.shape
+        q = SnapKVPress(window_size=self.n_last).window_queries(module, hidden_states, kwargs)        # [B, Hq, n_last, D]
+        sums = ops.snapkv_score(_lib.dense_view(keys), q.to(keys.dtype), self.n_last, 1, True, "sum",
+                                1.0 / math.sqrt(D))[0][..., :S - self.n_last]                          # [B, Hkv, S - n_last]
+        per_key = sums.sum(dim=(0, 1)) / (B * q.shape[1] * self.n_last)
+        return float(per_key[:self.n_initial].sum() + per_key[-self.n_recent:].sum())
+
+    def compress(self, module, hidden_states, keys, values, attentions, kwargs):
+        B, H, S, D = keys.shape
+        q_len = hidden_states.shape[1] if hidden_states is not None else S
+        if q_len <= self.n_initial + self.n_recent + self.n_last:
+            return keys, values
+        if self.lazy_score(module, hidden_states, keys, kwargs) <= self.lazy_threshold:
+            self.compression_ratios.append(0.0)
+            return keys, values
+        tail = self.n_recent - self.n_last
+        pos = torch.cat([torch.arange(self.n_initial), torch.arange(S - tail, S)]).to(torch.int32)
+        n = pos.numel()
+        idx = pos.to(keys.device).view(1, 1, 1, n).expand(1, B, 1, n).contiguous()                   # one row for all heads
+        out_k = torch.empty((B, H, n, D), dtype=keys.dtype, device=keys.device)
+        out_v = torch.empty_like(out_k)
+        ops.compact(_lib.dense_view(keys), _lib.dense_view(values), _lib.dense_view(out_k), _lib.dense_view(out_v), idx)
+        self.compression_ratios.append((q_len - self.n_initial - self.n_recent + 1) / q_len)
+        return out_k, out_v
+
+
 class SimpleKVQuantizer:
     """Symmetric ``nbits`` quantise-dequantise of every K and V tensor of a cache with ONE scale per tensor
     (utils_ccm/utils_compress.py:117-163).  Used as ``with quantizer(model) as q: q.quantize_cache(pkv)``."""

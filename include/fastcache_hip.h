@@ -275,6 +275,17 @@ int fc_fake_quantize(const void* x, void* y, int64_t rows, int32_t d, int32_t dt
                      void* stream);
 
 /*
+ * Key-channel statistics and pruning for the ThinK press (kvpress.ThinKPress, which the reference registers at
+ * nanovllm/autocompress/methods.py:422 and constructs at :432-436):
+ *   energy[l][b][h][d] = sum over the tokens s < len(b) of keys[l][b][h][s][d]^2   (fp32, [L][B][Hkv][128]);
+ *   fc_key_channel_zero sets keys[l][b][h][s][d] = 0 for every token of the sequence and every channel d with
+ *   prune[l][b][h][d] != 0 (uint8, [L][B][Hkv][128]), in place.
+ * The press multiplies the energies with those of the window queries, picks the channels and calls the second.
+ */
+int fc_key_channel_energy(const fc_kv_view* keys, float* energy, void* stream);
+int fc_key_channel_zero(const fc_kv_view* keys, const uint8_t* prune, void* stream);
+
+/*
  * 8-bit floating point codes with one scale for the whole tensor of n elements:
  *   scale = clamp(max|x| / 448, min=1e-8) (448 for both formats, as the reference has it), code = fp8(x / scale),
  * e5m2 == 0: E4M3, finite-only variant (largest value 448, 0x7f = NaN); e5m2 != 0: E5M2; conversion rounds to

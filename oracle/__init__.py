@@ -22,6 +22,9 @@ Pinning status (what independent check fixes each restatement; see tests/test_or
   presses.expected_attention_*        float64 loops over tokens / keys for the statistics and the score, closed
                                      forms (zero covariance, identity rotation); the kvpress package itself is
                                      unavailable offline: PARITY UNPINNED beyond the published formula
+  presses.think_* / simlayer_*        loops over heads, tokens, queries with the causal rule written out, hand-worked
+                                     rows; kvpress itself is unavailable offline: PARITY UNPINNED beyond the
+                                     published description of ThinK and SimLayerKV
   presses.fake_quantize               numpy float16 arithmetic step by step, hand-worked rows, idempotence
   autocompress.quantize_fp8 / quantize_int8_asymmetric
                                       the float8 cast against a brute-force nearest-code search (ties, both formats),

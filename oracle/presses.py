@@ -302,3 +302,44 @@ def fake_quantize(x: torch.Tensor, nbits: int, per_tensor: bool):
     x_quant = torch.round(x / scale)
     x_quant = torch.clamp(x_quant, -2 ** (nbits - 1), 2 ** (nbits - 1) - 1)
     return x_quant * scale, scale, max_val
+
+
+# ---- ThinK and SimLayerKV (kvpress presses the reference registers at nanovllm/autocompress/methods.py:422-423) ----
+def think_channel_scores(keys: torch.Tensor, queries: torch.Tensor) -> torch.Tensor:
+    """ThinK: ``mean over the window of q^2`` (then over the query heads of a kv group) times ``mean over the tokens of
+    k^2`` -> ``[B, Hkv, D]`` (float64).  keys ``[B, Hkv, S, D]``, queries ``[B, Hq, W, D]``."""
+    B, Hkv, S, D = keys.shape
+    qn = queries.double().pow(2).mean(dim=2).view(B, Hkv, queries.shape[1] // Hkv, D).mean(dim=2)
+    kn = keys.double().pow(2).mean(dim=2)
+    return qn * kn
+
+
+def think_prune(keys: torch.Tensor, queries: torch.Tensor, ratio: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Keys with the ``int(D * ratio)`` lowest-scored channels of every (batch, kv head) zeroed, and the sorted pruned
+    channel indices ``[B, Hkv, n]``; ties to the lowest channel."""
+    B, Hkv, S, D = keys.shape
+    n = int(D * ratio)
+    scores = think_channel_scores(keys, queries)
+    idx = topk_lowest_index(-scores, n)
+    out = keys.clone()
+    if n:
+        out.scatter_(-1, idx[:, :, None, :].expand(B, Hkv, S, n), 0)
+    return out, idx
+
+
+def simlayer_lazy_score(keys: torch.Tensor, queries: torch.Tensor, n_initial: int, n_recent: int) -> float:
+    """SimLayerKV: softmax of the last ``n_last`` queries over all keys (causal among themselves), the window's own
+    columns dropped, averaged over batch, heads and queries; sum over the first ``n_initial`` and the last
+    ``n_recent`` remaining keys.  keys ``[B, Hkv, S, D]``, queries ``[B, Hq, n_last, D]``."""
+    B, Hkv, S, D = keys.shape
+    Hq, W = queries.shape[1], queries.shape[2]
+    k = keys.double().repeat_interleave(Hq // Hkv, dim=1)
+    logits = torch.matmul(queries.double(), k.transpose(2, 3)) / math.sqrt(D)
+    logits = logits + torch.triu(torch.full((W, S), float("-inf"), dtype=torch.float64), diagonal=S - W + 1)
+    attn = torch.softmax(logits, dim=-1)[..., :S - W].mean(dim=(0, 1, 2))
+    return float(attn[:n_initial].sum() + attn[-n_recent:].sum())
+
+
+def simlayer_keep_positions(S: int, n_initial: int, n_recent: int, n_last: int) -> torch.Tensor:
+    """Token positions a lazy layer keeps: the first ``n_initial`` and the last ``n_recent - n_last``."""
+    return torch.cat([torch.arange(n_initial), torch.arange(S - (n_recent - n_last), S)])

@@ -3,6 +3,7 @@ import pytest
 import torch
 
 from fastcache_amd import _lib, ops, synth
+from fastcache_amd.presses import SimLayerKVPress, ThinKPress
 from oracle import paged as opaged
 from oracle import presses as opress
 
@@ -374,3 +375,104 @@ def test_snapkv_split_columns(dev, dtype, Hq, Hkv, S, W, ksz, causal, splits):
             torch.testing.assert_close(cut[l, b, :, :n - W], ref[:, :n - W], rtol=1e-3, atol=tol)
             torch.testing.assert_close(cut[l, b, :, :n], whole[l, b, :, :n], rtol=2e-4, atol=tol)
             assert bool(torch.isinf(cut[l, b, :, n:]).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hq,Hkv,S,W,ratio", [(2, 8, 2, 700, 32, 0.5), (1, 4, 4, 33, 16, 0.25), (3, 6, 3, 1300, 8, 0.9)])
+def test_think_press_channel_energy_and_pruning(dev, dtype, B, Hq, Hkv, S, W, ratio):
+    """ThinK: channel energies of K within fp32 summation error of the float64 oracle; the pruned channel set equals
+    the oracle's wherever the channel scores are not within 1e-5 (relative) of the selection threshold; pruned
+    channels are zero for every token, every other element and V are untouched bit for bit."""
+    g = torch.Generator().manual_seed(S + W)
+    k = (torch.randn(B, Hkv, S, 128, generator=g) * torch.linspace(0.2, 2.0, 128)).to(dtype)
+    v = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    q = torch.randn(B, Hq, W, 128, generator=g).to(dtype)
+    kd, vd = k.to(dev), v.to(dev)
+    energy = ops.key_channel_energy(_lib.dense_view(kd), dev)[0].cpu()
+    torch.testing.assert_close(energy.double(), k.double().pow(2).sum(2), rtol=1e-5, atol=1e-6)
+    press = ThinKPress(key_channel_compression_ratio=ratio, window_size=W)
+    ok, ov = press.compress(None, None, kd, vd, None, {"queries": q.to(dev)})
+    assert ok.data_ptr() == kd.data_ptr() and torch.equal(ov.cpu(), v)
+    ref_k, ref_idx = opress.think_prune(k, q, ratio)
+    scores = opress.think_channel_scores(k, q)
+    n = int(128 * ratio)
+    got = ok.cpu()
+    zeroed = (got == 0).all(dim=2)                                   # [B, Hkv, 128]: channels that are zero everywhere
+    for b in range(B):
+        for h in range(Hkv):
+            srt = scores[b, h].sort().values
+            thr_lo, thr_hi = srt[n - 1], srt[n]
+            near = ((scores[b, h] - thr_lo).abs() <= 1e-5 * thr_lo.abs()) | ((scores[b, h] - thr_hi).abs() <= 1e-5 * thr_hi.abs())
+            want = torch.zeros(128, dtype=torch.bool)
+            want[ref_idx[b, h]] = True
+            assert int(zeroed[b, h].sum()) == n
+            assert torch.equal(zeroed[b, h][~near], want[~near])
+            kept = ~zeroed[b, h]
+            assert torch.equal(got[b, h][:, kept], k[b, h][:, kept])
+
+
+def test_think_press_paged_ragged_and_no_ops(dev):
+    """The two kernels on a paged pool with ragged lengths (energies per sequence, zeroing limited to the sequence's
+    own tokens); ratio 0 and a ratio below one channel leave the keys alone."""
+    L, H, lens = 2, 2, [300, 17, 129]
+    case = synth.make_paged_case(seed=3, num_layers=L, batch=len(lens), num_kv_heads=H, seq_lens=lens, dtype=torch.float16,
+                                 keep_dense=True, block_size=64, fill_value=3.0)
+    pool, tab, lens_d = case.kv_cache.to(dev), case.table_tensor(dev), case.lens_tensor(dev)
+    view = _lib.paged_view(pool[0], tab, lens_d, max(lens))
+    energy = ops.key_channel_energy(view, dev).cpu()
+    for l in range(L):
+        for b, n in enumerate(lens):
+            torch.testing.assert_close(energy[l, b].double(), case.dense_k[l][b, :, :n].double().pow(2).sum(1), rtol=1e-5, atol=1e-6)
+    prune = torch.zeros(L, len(lens), H, 128, dtype=torch.uint8)
+    prune[..., 5] = 1
+    prune[1, 2, 1, 64:] = 1
+    ops.key_channel_zero(view, prune.to(dev))
+    after = pool.cpu()
+    used = set()
+    for b, n in enumerate(lens):
+        used.update(case.block_tables[b])
+        for l in range(L):
+            rows = torch.cat([after[0, l, blk] for blk in case.block_tables[b]])           # [tokens, H, D]
+            want = case.dense_k[l][b, :, :n].clone().permute(1, 0, 2)
+            want[..., 5] = 0
+            if (l, b) == (1, 2):
+                want[:, 1, 64:] = 0
+            assert torch.equal(rows[:n], want)
+            assert bool((rows[n:] == 3.0).all())                                            # slots past the sequence end
+    assert torch.equal(after[1], case.kv_cache[1])
+    spare = [i for i in range(after.shape[2]) if i not in used]
+    assert bool((after[0][:, spare] == 3.0).all())
+    k = torch.randn(1, 2, 40, 128).half().to(dev)
+    for ratio in (0.0, 0.005):
+        out, _ = ThinKPress(key_channel_compression_ratio=ratio).compress(None, None, k.clone(), k, None, {"queries": k[:, :, :32]})
+        assert torch.equal(out, k)
+    with pytest.raises(_lib.FastcacheError):
+        ops.key_channel_zero(view, prune.to(dev)[..., :64])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n_last,n_recent,n_initial", [(1, 64, 4), (8, 100, 2)])
+def test_simlayer_press(dev, dtype, n_last, n_recent, n_initial):
+    """SimLayerKV: the lazy score against the float64 oracle (1e-3); below the threshold the layer is left alone,
+    above it only the initial and the recent tokens survive, bit for bit; short inputs are never touched."""
+    B, Hq, Hkv, S = 2, 8, 2, 900
+    g = torch.Generator().manual_seed(n_recent)
+    k = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    q = (torch.randn(B, Hq, n_last, 128, generator=g) * 0.5).to(dtype)
+    kd, vd, kw = k.to(dev), v.to(dev), {"queries": q.to(dev)}
+    ref = opress.simlayer_lazy_score(k, q, n_initial, n_recent)
+    press = SimLayerKVPress(lazy_threshold=1.0, n_last=n_last, n_recent=n_recent, n_initial=n_initial)
+    got = press.lazy_score(None, None, kd, kw)
+    assert abs(got - ref) <= 1e-3 * ref and 0.0 < ref < 1.0
+    ok, ov = press.compress(None, None, kd, vd, None, kw)                 # threshold 1: never lazy
+    assert ok.data_ptr() == kd.data_ptr() and press.compression_ratios == [0.0]
+    lazy = SimLayerKVPress(lazy_threshold=ref / 2, n_last=n_last, n_recent=n_recent, n_initial=n_initial)
+    ok, ov = lazy.compress(None, None, kd, vd, None, kw)
+    pos = opress.simlayer_keep_positions(S, n_initial, n_recent, n_last)
+    assert ok.shape == (B, Hkv, pos.numel(), 128)
+    assert torch.equal(ok.cpu(), k[:, :, pos]) and torch.equal(ov.cpu(), v[:, :, pos])
+    assert lazy.compression_ratios == [(S - n_initial - n_recent + 1) / S] and lazy.compression_ratio == lazy.compression_ratios[0]
+    short = kd[:, :, :n_initial + n_recent + n_last]
+    ok, _ = lazy.compress(None, None, short, short, None, kw)
+    assert ok.data_ptr() == short.data_ptr() and len(lazy.compression_ratios) == 1

@@ -572,3 +572,54 @@ def test_fp8_and_asymmetric_int8_oracle_by_brute_force_and_hand():
     codes = np.clip(np.rint(f32((f32((f32(xn) - f32(mn)).astype(f16)) / f32(sc)).astype(f16))), 0, 255)
     assert np.array_equal(q.numpy(), codes.astype(np.uint8))
     assert np.array_equal(p[:, 0].numpy(), sc[:, 0]) and np.array_equal(p[:, 1].float().numpy(), zp[:, 0])
+
+
+def test_think_and_simlayer_oracle_by_loops_and_hand():
+    """oracle.presses.think_channel_scores / think_prune / simlayer_lazy_score / simlayer_keep_positions against
+    plain loops and hand-worked cases.  What the third-party kvpress package does beyond the published description
+    of the two methods cannot be checked offline: PARITY UNPINNED for those choices (statistics in which dtype,
+    how many recent tokens a lazy layer keeps)."""
+    import math
+    from oracle import presses as op
+    g = torch.Generator().manual_seed(31)
+    B, Hq, Hkv, S, W, D = 2, 4, 2, 9, 3, 128
+    k = torch.randn(B, Hkv, S, D, generator=g)
+    q = torch.randn(B, Hq, W, D, generator=g)
+    sc = op.think_channel_scores(k, q)
+    G = Hq // Hkv
+    for b in range(B):
+        for h in range(Hkv):
+            for d in (0, 1, 77, 127):
+                qe = sum(float(q[b, h * G + j, w, d]) ** 2 for j in range(G) for w in range(W)) / (G * W)
+                ke = sum(float(k[b, h, s, d]) ** 2 for s in range(S)) / S
+                assert abs(float(sc[b, h, d]) - qe * ke) <= 1e-12 * max(1.0, qe * ke)
+    # by hand: channel d of the keys scaled by (d + 1), queries all ones -> the lowest-energy channels are 0 .. n-1
+    kk = torch.ones(1, 1, 5, D) * torch.arange(1, D + 1)
+    out, idx = op.think_prune(kk, torch.ones(1, 1, 2, D), 0.25)
+    assert idx[0, 0].tolist() == list(range(32))
+    assert bool((out[..., :32] == 0).all()) and torch.equal(out[..., 32:], kk[..., 32:])
+    # equal scores: ties go to the lowest channel; ratio below one channel prunes nothing
+    out, idx = op.think_prune(torch.ones(1, 1, 3, D), torch.ones(1, 1, 2, D), 0.5)
+    assert idx[0, 0].tolist() == list(range(64))
+    assert torch.equal(op.think_prune(kk, torch.ones(1, 1, 2, D), 0.005)[0], kk)
+    # SimLayerKV: loops over queries and keys with the causal rule written out
+    n_last, n_initial, n_recent = 2, 2, 3
+    ql = q[:, :, :n_last]
+    got = op.simlayer_lazy_score(k, ql, n_initial, n_recent)
+    acc = [0.0] * (S - n_last)
+    for b in range(B):
+        for hq in range(Hq):
+            for w in range(n_last):
+                visible = S - n_last + w + 1                 # query w sees the prefix and window keys 0 .. w
+                logit = [float(torch.dot(ql[b, hq, w].double(), k[b, hq // G, s].double())) / math.sqrt(D) for s in range(visible)]
+                m = max(logit)
+                e = [math.exp(x - m) for x in logit]
+                z = sum(e)
+                for s in range(S - n_last):
+                    acc[s] += e[s] / z / (B * Hq * n_last)
+    want = sum(acc[:n_initial]) + sum(acc[-n_recent:])
+    assert abs(got - want) <= 1e-12
+    # all of the probability mass outside the window counted once when initial + recent cover every key
+    total = op.simlayer_lazy_score(k, ql, 0, S - n_last)
+    assert abs(total - sum(acc)) <= 1e-12 and total < 1.0
+    assert op.simlayer_keep_positions(20, 4, 6, 1).tolist() == [0, 1, 2, 3, 15, 16, 17, 18, 19]
