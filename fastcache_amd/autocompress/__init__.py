@@ -5,4 +5,4 @@ from .context import GPUArch, HardwareProfile, WorkloadContext, detect_hardware,
 from .execution import StreamManager, get_stream_manager  # noqa: F401
 from .kernels import (KernelConfig, TileLangKernelGenerator, get_kernel_generator, get_mlp_kernel,  # noqa: F401
                       get_quantize_kernels, get_sparse_gather_kernel)
-from .methods import QuantizationMethod  # noqa: F401
+from .methods import KVPressMethod, QuantizationMethod  # noqa: F401

@@ -1,5 +1,7 @@
-"""KV quantisation with the reference's call surface (``QuantizationMethod``,
-nanovllm/autocompress/methods.py:520-757), computed by HIP kernels.
+"""The compression-method adapters of the reference that carry device work: ``KVPressMethod``
+(nanovllm/autocompress/methods.py:227-495, a press by name with ``compress(keys, values, **kwargs)``) and
+``QuantizationMethod`` (:520-757), computed by HIP kernels.  The cost profiles and timing heuristics the
+reference attaches to them (A100 constants for its scheduler) are not carried over.
 
 Built: ``int8`` (one scale per row of the last dimension; ``symmetric=False`` gives uint8 codes with a
 ``(scale, zero point)`` pair per row), ``int4`` and ``nf4`` (one scale per group of ``group_size`` elements, two
@@ -86,3 +88,53 @@ class QuantizationMethod:
         if t in (self.QuantType.INT4, self.QuantType.NF4):
             return ops.dequantize_group4(quantized, scale, self._group_size, t == self.QuantType.NF4, dtype)
         return ops.dequantize_fp8(quantized, scale, dtype)
+
+
+class KVPressMethod:
+    """A press chosen by name, called outside a model (methods.py:227-495).  The press runs on the HIP kernels of
+    ``fastcache_amd.presses``; ``compress`` forwards ``module`` / ``hidden_states`` / ``attentions`` from the keyword
+    arguments and hands all of them on as the press's ``kwargs`` (``queries``, ``position_embeddings``, ...)."""
+
+    @staticmethod
+    def _press_map():
+        from .. import presses
+        return {"snapkv": presses.SnapKVPress, "streaming_llm": presses.StreamingLLMPress,
+                "observed_attention": presses.ObservedAttentionPress,
+                "expected_attention": presses.ExpectedAttentionPress, "knorm": presses.KnormPress,
+                "tova": presses.TOVAPress, "think": presses.ThinKPress, "simlayer": presses.SimLayerKVPress,
+                "random": presses.RandomPress}
+
+    def __init__(self, method_name: str, compression_ratio: float = 0.5, **method_kwargs):
+        self._method_name = method_name.lower()
+        self._compression_ratio = compression_ratio
+        self._method_kwargs = method_kwargs
+        self._press = None
+
+    def _init_press(self):
+        if self._press is not None:
+            return
+        press_class = self._press_map().get(self._method_name)
+        if press_class is None:
+            raise ValueError(f"Unknown kvpress method: {self._method_name}")
+        if self._method_name == "think":
+            self._press = press_class(key_channel_compression_ratio=self._compression_ratio, **self._method_kwargs)
+        elif self._method_name == "simlayer":
+            # the reference passes compression_ratio= here as well, which this press (like kvpress's) cannot take:
+            # its ratio is an outcome of the lazy-layer test
+            self._press = press_class(**self._method_kwargs)
+        else:
+            self._press = press_class(compression_ratio=self._compression_ratio, **self._method_kwargs)
+
+    @property
+    def name(self) -> str:
+        return f"kvpress_{self._method_name}"
+
+    @property
+    def press(self):
+        self._init_press()
+        return self._press
+
+    def compress(self, keys: torch.Tensor, values: torch.Tensor, **kwargs) -> Tuple[torch.Tensor, torch.Tensor]:
+        self._init_press()
+        return self._press.compress(module=kwargs.get("module"), hidden_states=kwargs.get("hidden_states"),
+                                    keys=keys, values=values, attentions=kwargs.get("attentions"), kwargs=kwargs)

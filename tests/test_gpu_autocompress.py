@@ -321,3 +321,28 @@ def test_fake_quantize_odd_shapes(dev, shape, bits):
         ref = op.fake_quantize(x, bits, per_tensor)[0]
         got = ops.fake_quantize(x.to(dev), bits, per_tensor).cpu()
         assert torch.equal(torch.nan_to_num(got, nan=-7.0), torch.nan_to_num(ref, nan=-7.0)), per_tensor
+
+
+def test_kvpress_method_adapter(dev):
+    """KVPressMethod: a press by name, called on bare tensors; every name of the reference's table resolves, the
+    results equal the press called directly, unknown names raise as there."""
+    from fastcache_amd import presses
+    g = torch.Generator().manual_seed(9)
+    k = torch.randn(2, 2, 300, 128, generator=g).half().to(dev)
+    v = torch.randn(2, 2, 300, 128, generator=g).half().to(dev)
+    q = torch.randn(2, 8, 64, 128, generator=g).half().to(dev)
+    m = ac.KVPressMethod("SnapKV", compression_ratio=0.5, window_size=64, kernel_size=7)
+    assert m.name == "kvpress_snapkv"
+    ck, cv = m.compress(k, v, queries=q)
+    rk, rv = presses.SnapKVPress(compression_ratio=0.5, window_size=64, kernel_size=7).compress(None, None, k, v, None, {"queries": q})
+    assert ck.shape == (2, 2, 150, 128) and torch.equal(ck, rk) and torch.equal(cv, rv)
+    ck, cv = ac.KVPressMethod("knorm", 0.25).compress(k, v)
+    assert ck.shape == (2, 2, 225, 128)
+    tk, _ = ac.KVPressMethod("think", 0.5, window_size=32).compress(k.clone(), v, queries=q[:, :, -32:])
+    assert int((tk == 0).all(dim=2).sum()) == 2 * 2 * 64
+    sk, _ = ac.KVPressMethod("simlayer", 0.5, lazy_threshold=0.0, n_recent=100).compress(k, v, queries=q[:, :, -1:])
+    assert sk.shape == (2, 2, 4 + 99, 128)
+    for name in ("streaming_llm", "observed_attention", "expected_attention", "tova", "random"):
+        assert ac.KVPressMethod(name, 0.3).press.compression_ratio == 0.3
+    with pytest.raises(ValueError):
+        ac.KVPressMethod("h2o").compress(k, v)
