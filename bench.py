@@ -446,6 +446,7 @@ WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkl
 _FETCH_SCALE = 524288 / 2.623e5
 _WRITE_SCALE = 524288 / 5.244e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
+    "cfg1-knorm-llama-7b": (2.642e5, 5.263e5),
     "cfg2-snapkv-qwen3-8b": (2.391e6, 3.636e4),
     "cfg3-ccm-linear-decouple-llava-1.5-7b": (1.861e6, 1.845e6),      # mean over the 4 launches of a step
 }
