@@ -29,7 +29,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
                                                           const int* __restrict__ n_kept,
                                                           int* __restrict__ indices, int index_stride) {
   constexpr int TK_WAVES = TK_THREADS / FC_WAVE;
-  extern __shared__ unsigned lds_keys[];
+  extern __shared__ __align__(16) unsigned lds_keys[];
   __shared__ unsigned hist[TK_BINS];
   __shared__ unsigned wave_tot[TK_BINS / FC_WAVE];
   __shared__ unsigned sel_bin, sel_remaining;
@@ -53,7 +53,25 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
   }
 
   if (LDS_KEYS) {
-    for (int i = tid; i < n; i += TK_THREADS) lds_keys[i] = tk_key(row[i]);
+    // 16-byte loads, four per thread in flight, when the row starts on a 16-byte boundary
+    int done = 0;
+    if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+      const float4* row4 = reinterpret_cast<const float4*>(row);
+      uint4* keys4 = reinterpret_cast<uint4*>(lds_keys);
+      const int n4 = n >> 2;
+      for (int i0 = 0; i0 < n4; i0 += 4 * TK_THREADS) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = row4[min(i0 + u * TK_THREADS + tid, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * TK_THREADS + tid;
+          if (i < n4) keys4[i] = make_uint4(tk_key(v[u].x), tk_key(v[u].y), tk_key(v[u].z), tk_key(v[u].w));
+        }
+      }
+      done = n4 << 2;
+    }
+    for (int i = done + tid; i < n; i += TK_THREADS) lds_keys[i] = tk_key(row[i]);
   }
   auto key_at = [&](int i) -> unsigned { return LDS_KEYS ? lds_keys[i] : tk_key(row[i]); };
 
