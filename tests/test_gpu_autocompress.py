@@ -346,3 +346,56 @@ def test_kvpress_method_adapter(dev):
         assert ac.KVPressMethod(name, 0.3).press.compression_ratio == 0.3
     with pytest.raises(ValueError):
         ac.KVPressMethod("h2o").compress(k, v)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [128, 64, 256, 40])
+def test_quantisers_special_rows_all_row_lengths(dev, dtype, d):
+    """Rows of 128 / 256 / 512 bytes take the 16-bytes-per-lane kernels, other lengths the generic ones: both against
+    the eager expressions bit for bit, on random rows plus an all-zero row, a row with a NaN, a row with an infinity,
+    a constant row, a one-hot row and a row of tiny values; row counts that leave the last block partly empty."""
+    g = torch.Generator().manual_seed(d)
+    x = (torch.randn(37, d, generator=g) * 3).to(dtype)
+    x[1] = 0
+    x[2, 5] = float("nan")
+    x[3, 7] = float("inf")
+    x[4] = -1.75
+    x[5] = 0
+    x[5, d - 1] = 2.5
+    x[6] = x[6] * 1e-6
+    xd = x.to(dev)
+
+    def same(a, b):
+        a, b = a.cpu(), b
+        assert a.dtype == b.dtype and a.shape == b.shape
+        if a.is_floating_point():
+            assert torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(7.0), b.nan_to_num(7.0))
+        else:
+            assert torch.equal(a, b)
+
+    q, s = ops.quantize_rows(xd, 8)
+    rq, rs = oa.quantize_int8(x)
+    same(s, rs)
+    same(q, rq)                                  # NaN quotients (NaN row, 0/0 of a zero row in fp16, inf/inf) give code 0
+    ok_rows = ~x.isnan().any(-1)
+    q, p = ops.quantize_rows_asym(xd)
+    rq, rp = oa.quantize_int8_asymmetric(x)
+    ok_asym = ok_rows & ~x.isinf().any(-1)       # inf - inf inside the row gives NaN codes
+    assert torch.equal(q.cpu()[ok_asym], rq[ok_asym])
+    same(p[..., 0], rp[..., 0])
+    assert bool((p.cpu()[..., 1].float().nan_to_num(-1) == rp[..., 1].float().nan_to_num(-1)).all())
+    if d % 8 == 0:
+        for nf4 in (False, True):
+            q, s = ops.quantize_group4(xd, d, nf4)
+            rq, rs = (oa.quantize_nf4 if nf4 else oa.quantize_int4)(x, d)
+            same(s, rs)
+            same(q, rq)                          # NaN quotients: integer 0 + 8 (int4), first level (nf4)
+    for bits in (4, 8):
+        y, sc, mx = ops.fake_quantize(xd, bits, per_tensor=False, return_params=True)
+        qmax = 2 ** (bits - 1) - 1
+        rmx = x.abs().amax(dim=-1, keepdim=True)
+        rsc = rmx / qmax
+        ry = (x / rsc).round().clamp(-qmax - 1, qmax) * rsc
+        same(mx, rmx)
+        same(sc, rsc)
+        same(y, ry)
