@@ -198,6 +198,14 @@ __device__ __forceinline__ unsigned fc_lds_addr(const void* p) {
   return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
 }
 
+// 16 bytes from an absolute LDS address (what fc_lds_addr returns, plus offsets): one ds_read_b128 with the
+// address taken as it is, no base added
+__device__ __forceinline__ uint4 fc_lds_read128(unsigned addr) {
+  typedef unsigned fc_u32x4 __attribute__((ext_vector_type(4)));
+  const fc_u32x4 v = *reinterpret_cast<const __attribute__((address_space(3))) fc_u32x4*>((size_t)addr);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16 (lds_base is
 // wave-uniform).  The load is counted in vmcnt; the compiler does not know it writes LDS, so
 // every consumer sits behind an explicit wait (fc_wait_barrier, fc_wait_vm).

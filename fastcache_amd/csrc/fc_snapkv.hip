@@ -43,7 +43,8 @@ __device__ __forceinline__ float sk_exp2(float x) { return __builtin_amdgcn_exp2
 template <int NW>
 struct SkCfg {
   static constexpr int ST = NW >= 8 ? 4 : 3;   // key tiles resident or in flight per workgroup
-  static constexpr int LDS = ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4 + SK_TBL * 4;
+  // + 256: the key tiles start on a 256-byte LDS address (see the operand reads)
+  static constexpr int LDS = ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4 + SK_TBL * 4 + 256;
 };
 
 // MODE 0: the whole kernel for one (layer, sequence, kv head) column.
@@ -61,7 +62,10 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   constexpr int ST = SkCfg<NW>::ST;
   constexpr int LPW = 16 / NW;   // 1 KB wave-loads (4 key rows) per wavefront and tile
   static_assert(LPW * NW == 16, "NW must divide 16");
-  extern __shared__ __align__(16) char smem[];
+  extern __shared__ __align__(16) char smem_raw[];
+  // The key tiles start on a multiple of 256 in LDS address terms, so that the LDS base can be folded into a lane's
+  // operand address before the XOR that picks the 16-byte chunk (which touches address bits 4..7 only).
+  char* smem = smem_raw + ((256u - (fc_lds_addr(smem_raw) & 255u)) & 255u);
   char* kbuf = smem;
   float(*vpart)[NW][SK_KT] = reinterpret_cast<float(*)[NW][SK_KT]>(smem + ST * SK_TILEB);
   float(*vraw)[SK_KT] = reinterpret_cast<float(*)[SK_KT]>(smem + ST * SK_TILEB + 4 * NW * SK_KT * 4);
@@ -174,18 +178,19 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     if (MODE == 2) return te - 1 - pos;    // descending
     return pos < T ? pos : 2 * T - 1 - pos;
   };
-  int kc = 0, m = 0;
+  unsigned kc = 0;   // unsigned: kc % ST is a mask for ST = 4
+  int m = 0;
   auto prologue = [&](int first) {   // first = 0: both sweeps; first = T: the second sweep alone
     m = first;
-    for (int i = 0; i < ST - 1 && first + i < P; ++i) issue(plan_tile(first + i), (kc + i) % ST);
+    for (int i = 0; i < ST - 1 && first + i < P; ++i) issue(plan_tile(first + i), (int)((kc + (unsigned)i) % ST));
   };
   // top of a tile iteration: tile position m has landed for every wave, the stage consumed by the
   // previous iteration is free and receives position m+ST-1; returns the stage to read
   auto acquire = [&]() {
     if (m + ST - 2 < P) fc_wait_barrier<LPW*(ST - 2)>(); else fc_wait_barrier<0>();
     const int nx = m + ST - 1;
-    if (nx < P) issue(plan_tile(nx), (kc + ST - 1) % ST);
-    return kc % ST;
+    if (nx < P) issue(plan_tile(nx), (int)((kc + ST - 1) % ST));
+    return (int)(kc % ST);
   };
 
   const bool always_general = SW < SK_KT;
@@ -194,7 +199,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // LDS address of the lane's fragment of k-slice ks of a 32-key block: the row base plus the
   // swizzled chunk ((ks*2 + lhalf) ^ swz) * 16.  ks*32, lhalf*16 and the row base occupy disjoint
   // bits, so this is (row base + xs) ^ (ks*32).
-  const unsigned xs = (unsigned)((lhalf ^ swz) << 4) + lrow * 256;
+  const unsigned xs = (unsigned)((lhalf ^ swz) << 4) + lrow * 256 + kbuf_lds;   // an absolute LDS address
   // 32 keys x 32 queries of logits.  KEYS_ROWS: C[key][query] (the lane owns one query and 16
   // keys), otherwise C[query][key] (the lane owns one key and 16 queries).
   auto mfma_block = [&](bool keys_rows, int stage, int cb, f32x16& acc) {
@@ -203,7 +208,24 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     const unsigned a0 = (unsigned)(stage * SK_TILEB + cb * 8192) + xs;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      const uint4 kf = *reinterpret_cast<const uint4*>(kbuf + (a0 ^ (unsigned)(ks * 32)));
+      const uint4 kf = fc_lds_read128(a0 ^ (unsigned)(ks * 32));
+      acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc) : fc_mfma<DTYPE>(qf[ks], kf, acc);
+    }
+  };
+  // The same for the loops that walk whole tiles: the eight fragment addresses of a tile's first block are
+  // formed once per tile (tile_addr) and the second block reads 8192 bytes further, which the read instruction
+  // adds by itself.
+  unsigned adr[8];
+  auto tile_addr = [&](int stage) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) adr[ks] = ((unsigned)(stage * SK_TILEB) + xs) ^ (unsigned)(ks * 32);
+  };
+  auto mfma_tile_block = [&](bool keys_rows, int cb, f32x16& acc) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const uint4 kf = fc_lds_read128(adr[ks] + (unsigned)(cb * 8192));
       acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc) : fc_mfma<DTYPE>(qf[ks], kf, acc);
     }
   };
@@ -274,20 +296,20 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // with the exponentials of the block before it
   auto sweep1_piped = [&](int t0, int t1) {
     f32x16 acc_a, acc_b;
-    int stage = acquire();
-    mfma_block(true, stage, 0, acc_a);
+    tile_addr(acquire());
+    mfma_tile_block(true, 0, acc_a);
     for (int t = t0; t < t1 - 1; ++t) {
-      mfma_block(true, stage, 1, acc_b);
+      mfma_tile_block(true, 1, acc_b);
       stats_fast(acc_a);
       interleave();
       ++m;
       ++kc;
-      stage = acquire();
-      mfma_block(true, stage, 0, acc_a);
+      tile_addr(acquire());
+      mfma_tile_block(true, 0, acc_a);
       stats_fast(acc_b);
       interleave();
     }
-    mfma_block(true, stage, 1, acc_b);
+    mfma_tile_block(true, 1, acc_b);
     stats_fast(acc_a);
     interleave();
     stats_fast(acc_b);
@@ -312,7 +334,17 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       sweep1_plain(max(tf_end, tb + 1), te, false);
     }
     const bool bad = !(lsq <= 3.0e38f);   // inf or NaN
-    if (attempt == 1 || !__builtin_amdgcn_readfirstlane(__syncthreads_or(bad))) break;
+    if (attempt == 1) break;
+    // Did any lane of the workgroup overflow?  Through the (still unused) per-key sum area rather than
+    // __syncthreads_or, whose static LDS word would move the key tiles off LDS address 0 and cost every
+    // operand read an extra address addition.
+    const bool wave_bad = __any(bad);
+    if (lane == 0) vpart[0][wave][0] = wave_bad ? 1.f : 0.f;
+    __syncthreads();
+    float any_bad = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) any_bad += vpart[0][w][0];
+    if (!__builtin_amdgcn_readfirstlane(any_bad > 0.f)) break;
     fc_wait_barrier<0>();   // the tiles prefetched for sweep 2 land before their stages are reused
     mref = SK_NEG;
     lsq = 0.f;
@@ -382,24 +414,24 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   };
   {
     f32x16 acc_a, acc_b;
-    int stage = acquire();
-    mfma_block(false, stage, 0, acc_a);
+    tile_addr(acquire());
+    mfma_tile_block(false, 0, acc_a);
     for (int u = 0; u < P2 - 1; ++u) {
-      mfma_block(false, stage, 1, acc_b);
+      mfma_tile_block(false, 1, acc_b);
       probs(acc_a, u, 0);
       interleave();
       ++m;
       ++kc;
-      stage = acquire();
+      tile_addr(acquire());
       // the sums of the tile processed before this one are complete: fold them; tile T-u+2 had
       // both neighbours folded (by other wavefronts) before the barrier just passed
       if (u >= 1) fold(u - 1);
       if (MODE == 0 && u >= 3) emit_tile(T - u + 2);
-      mfma_block(false, stage, 0, acc_a);
+      mfma_tile_block(false, 0, acc_a);
       probs(acc_b, u, 1);
       interleave();
     }
-    mfma_block(false, stage, 1, acc_b);
+    mfma_tile_block(false, 1, acc_b);
     probs(acc_a, P2 - 1, 0);
     interleave();
     probs(acc_b, P2 - 1, 1);
