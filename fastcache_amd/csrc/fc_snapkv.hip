@@ -136,6 +136,12 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   // FAST: a tile lies inside one page (or the view is dense), so a load is a wave-uniform tile base
   // plus a per-lane byte offset; the offset is recomputed per load rather than kept in registers.
   const unsigned tok_bytes = (unsigned)kv.stride_token * 2;
+  unsigned lofs[LPW];   // byte offset of this lane's 16 bytes inside a tile, per wave-load
+#pragma unroll
+  for (int u = 0; u < LPW; ++u) {
+    const int r = 4 * (wave * LPW + u) + (lane >> 4);
+    lofs[u] = (unsigned)r * tok_bytes + (((lane & 15) ^ (r & 15)) << 4);
+  }
   auto issue = [&](int tile, int stage) {
     if constexpr (FAST) {
       const int s0 = tile * SK_KT;
@@ -146,15 +152,22 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       } else {
         tb = (long long)b * kv.stride_batch + (long long)s0 * kv.stride_token;
       }
-      const char* g = kbase + tb * 2;
+      // (wave-uniform by construction; said again so that it stays in scalar registers across the branch below)
+      const unsigned long long gu = (unsigned long long)(kbase + tb * 2);
+      const char* g = reinterpret_cast<const char*>(
+          ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(gu >> 32)) << 32) |
+          (unsigned)__builtin_amdgcn_readfirstlane((int)(gu & 0xffffffffu)));
       const int rmax = S - 1 - s0;   // rows past the end re-read the last row
+      if (rmax >= SK_KT - 1) {       // a whole tile: the lane offsets are the ones prepared before the loops
 #pragma unroll
-      for (int u = 0; u < LPW; ++u) {
-        int ln = lane;
-        asm volatile("" : "+v"(ln));
-        const int r = 4 * (wave * LPW + u) + (ln >> 4);
-        const unsigned lo = (unsigned)min(r, rmax) * tok_bytes + (((ln & 15) ^ (r & 15)) << 4);
-        fc_load_lds(g, lo, kbuf_lds + stage * SK_TILEB + (wave * LPW + u) * 1024);
+        for (int u = 0; u < LPW; ++u) fc_load_lds(g, lofs[u], kbuf_lds + stage * SK_TILEB + (wave * LPW + u) * 1024);
+      } else {
+#pragma unroll
+        for (int u = 0; u < LPW; ++u) {
+          const int r = 4 * (wave * LPW + u) + (lane >> 4);
+          const unsigned lo = (unsigned)min(r, rmax) * tok_bytes + (((lane & 15) ^ (r & 15)) << 4);
+          fc_load_lds(g, lo, kbuf_lds + stage * SK_TILEB + (wave * LPW + u) * 1024);
+        }
       }
     } else {
 #pragma unroll 1
