@@ -278,10 +278,8 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     mref = mnew;
   };
   auto stats_fast = [&](const f32x16& acc) {
-    float bs = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) bs += sk_exp2(fmaf(acc[i], c, nmq));
-    lsq += bs;
+    for (int i = 0; i < 16; ++i) lsq += sk_exp2(fmaf(acc[i], c, nmq));
   };
   // tiles [t0, t1) one block at a time, with masking; fixed offset unless `general`
   auto sweep1_plain = [&](int t0, int t1, bool general) {
@@ -411,17 +409,22 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
   auto emit_tile = [&](int e) {   // moving average of tile e, whose neighbours are folded
     const int s = e * SK_KT + fkey;
     float a = 0.f;
-    for (int j = fp; j < ksz; j += NW) {
-      const int x = s + j - hw;
-      if (x >= 0 && x < SW) a += vraw[(x / SK_KT) & 3][x % SK_KT];
+    if (ksz <= NW) {   // the usual case: at most one term per lane, no loop
+      const int x = s + fp - hw;
+      if (fp < ksz && x >= 0 && x < SW) a = vraw[(x >> 6) & 3][x & (SK_KT - 1)];
+    } else {
+      for (int j = fp; j < ksz; j += NW) {
+        const int x = s + j - hw;
+        if (x >= 0 && x < SW) a += vraw[(x / SK_KT) & 3][x % SK_KT];
+      }
     }
     a = fc_group_sum<NW>(a);
     if (fp == 0 && s < SW) out_row[s] = a * out_mul;
   };
   auto probs = [&](const f32x16& acc, int u, int cb) {
-    float vs = 0.f;
+    float vs = sk_exp2(fmaf(acc[0], c, nm[0]));
 #pragma unroll
-    for (int i = 0; i < 16; ++i) vs += sk_exp2(fmaf(acc[i], c, nm[i]));
+    for (int i = 1; i < 16; ++i) vs += sk_exp2(fmaf(acc[i], c, nm[i]));
     vs += __shfl_xor(vs, 32, 64);
     if (lane < 32) vpart[u & 3][wave][cb * 32 + lane] = vs;
   };
