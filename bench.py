@@ -5,7 +5,8 @@
 hot path over one batch of synthetic input that is already resident in HBM.  The default workload
 is configuration 2 (SnapKV press over a Qwen3-8B-shaped paged pool: score -> window fill -> top-k
 -> in-place compaction, all 36 layers, batch 8, 4096 tokens per sequence).  ``--workload`` selects
-the other configurations (knorm, ccm, decode, hybrid; decode-eager = the decode launches without a
+the other configurations (knorm, ccm, decode, hybrid, hybrid-decode = the 64 decode steps of
+configuration 5; decode-eager = the decode launches without a
 graph, for the profiler; snapkv-lse = cfg2 with the window queries' log-sum-exp given, single pass over K); they are measured the same way.
 
 Extra objects on the line:
@@ -328,20 +329,29 @@ class DecodeWorkload(Workload):
     metric = "decode tokens/sec"
     unit = "tokens/s"
 
-    def __init__(self, seed, device, graph_steps=128, eager=False):
+    def __init__(self, seed, device, graph_steps=128, eager=False, hybrid=False):
         super().__init__()
         from fastcache_amd import synth
         from fastcache_amd.engine.decode_graph import DecodeGraph
-        self.L, self.B, self.Hq, self.Hkv, self.T = 32, 90, 32, 32, graph_steps
         self.eager = eager
         self.device = device
-        self.case = synth.decode_case(seed=seed, steps=self.T, device=device, device_draw=True)
+        if hybrid:   # the decode half of configuration 5: 16 caches compressed to 3280 tokens, 7 query heads per kv head
+            self.name, self.dtype_name = "cfg5-decode-after-hybrid-minicpm-v-2.6", "bf16"
+            self.L, self.B, self.Hq, self.Hkv, self.T, dtype = 28, 16, 28, 4, graph_steps, torch.bfloat16
+            self.lens_text = "3280 (16384 compressed to 20 %)"
+            self.case = synth.decode_case(seed=seed, num_layers=self.L, batch=self.B, num_kv_heads=self.Hkv,
+                                          min_len=3280, max_len=3280, steps=self.T, dtype=dtype, device=device,
+                                          device_draw=True)
+        else:
+            self.L, self.B, self.Hq, self.Hkv, self.T, dtype = 32, 90, 32, 32, graph_steps, torch.float16
+            self.lens_text = "uniform[128, 2048]"
+            self.case = synth.decode_case(seed=seed, steps=self.T, device=device, device_draw=True)
         self.tables = self.case.table_tensor(device)
         self.lens0 = self.case.lens_tensor(device)
         self.lens = self.lens0.clone()
         g = torch.Generator(device=device).manual_seed(seed + 1)
         mk = lambda h: torch.randn((self.T, self.L, self.B, h, D), generator=g, device=device,
-                                   dtype=torch.float32).to(torch.float16)
+                                   dtype=torch.float32).to(dtype)
         self.dg = DecodeGraph(self.case.kv_cache, self.tables, self.lens, mk(self.Hq), mk(self.Hkv), mk(self.Hkv),
                               D ** -0.5)
         if not eager:
@@ -358,7 +368,7 @@ class DecodeWorkload(Workload):
 
     def config(self):
         return {"workload": self.name, "layers": self.L, "batch": self.B, "q_heads": self.Hq, "kv_heads": self.Hkv,
-                "head_dim": D, "context_lens": "uniform[128, 2048]", "sum_context_lens": sum(self.case.seq_lens),
+                "head_dim": D, "context_lens": self.lens_text, "sum_context_lens": sum(self.case.seq_lens),
                 "block_size": 256, "decode_steps_per_graph": self.T,
                 "graph": "none (eager launches, for the profiler)" if self.eager else "one hipGraph of all steps and layers"}
 
@@ -435,7 +445,10 @@ WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkl
              # cfg2 with the window queries' log-sum-exp handed in (not the BASELINE metric: the reference has no such input)
              "snapkv-lse": lambda seed, dev: SnapKVWorkload(seed, dev, given_lse=True),
              # the decode launches without a graph, 4 steps per bracket: rocprofv3 cannot walk the 128-step graph
-             "decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True)}
+             "decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True),
+             # the 64 decode steps that follow the compression in configuration 5, in one graph
+             "hybrid-decode": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=64, hybrid=True),
+             "hybrid-decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True, hybrid=True)}
 
 
 # HBM-side bytes per launch of a workload's dominant kernel, from two rocprofv3 counter runs
