@@ -528,7 +528,8 @@ extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cac
     FC_REQUIRE(Hkv * gtiles <= 65535 && B <= 65535, FC_EUNSUPPORTED, "%s: grid too large", who);
     dim3 grid(splits, Hkv * gtiles, B);
     const auto tile_in_page = [](const fc_kv_view* v, const KvView& d) {
-      return v->block_tables == nullptr || (d.block_shift >= 5);
+      return v->stride_token >= 0 && v->stride_token < (1 << 24) &&   // a tile's byte offsets fit 32 bits
+             (v->block_tables == nullptr || (d.block_shift >= 5));
     };
     const bool fast = tile_in_page(k_cache, k) && tile_in_page(v_cache, v);
 #define DA_LAUNCH(DT, GTV, FA)                                                                                   \

@@ -643,8 +643,9 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
 #define SK_DISPATCH(DT) \
   if (fast) { SK_DISPATCH2(DT, true); } else { SK_DISPATCH2(DT, false); }
   // a key tile lies inside one page (whose table row fits the LDS copy), or the view is dense
-  const bool fast = !keys->block_tables ||
-                    (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL);
+  const bool fast = keys->stride_token >= 0 && keys->stride_token < (1 << 24) &&   // a tile's byte offsets fit 32 bits
+                    (!keys->block_tables ||
+                     (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL));
   if (keys->dtype == FC_BF16) { SK_DISPATCH(FC_BF16); } else { SK_DISPATCH(FC_F16); }
 #undef SK_DISPATCH2
 #undef SK_DISPATCH
@@ -705,8 +706,9 @@ extern "C" int fc_snapkv_score_split(const fc_kv_view* keys, const void* queries
   const int G = num_q_heads / Hkv;
   const int waves = G * ((window + 31) / 32);
   KvView kv = fc_make_view(keys);
-  const bool fast = !keys->block_tables ||
-                    (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL);
+  const bool fast = keys->stride_token >= 0 && keys->stride_token < (1 << 24) &&   // a tile's byte offsets fit 32 bits
+                    (!keys->block_tables ||
+                     (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL));
   FC_REQUIRE(waves <= 16 && fast, FC_EUNSUPPORTED,
              "%s: split columns need a query group of at most 16 row blocks (got %d) and pages of 64*2^n tokens or a "
              "dense view", who, waves);
