@@ -313,9 +313,13 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       mfma_tile_block(true, 1, acc_b);
       stats_fast(acc_a);
       interleave();
+      asm volatile("" : "+v"(lsq));   // ... nor sink acc_a's exponentials below it
       ++m;
       ++kc;
       tile_addr(acquire());
+      // acc_b's exponentials are pure register arithmetic, which the compiler would otherwise move ahead of the
+      // barrier in acquire() and leave the MFMAs below without vector work to overlap
+      asm volatile("" : "+v"(acc_b));
       mfma_tile_block(true, 0, acc_a);
       stats_fast(acc_b);
       interleave();
