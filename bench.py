@@ -461,6 +461,7 @@ _WRITE_SCALE = 524288 / 5.244e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
     "cfg1-knorm-llama-7b": (2.642e5, 5.263e5),
     "cfg2-snapkv-qwen3-8b": (2.391e6, 3.636e4),
+    "cfg2-snapkv-qwen3-8b+given-lse": (1.273e6, 3.636e4),           # one sweep: K is read once
     "cfg3-ccm-linear-decouple-llava-1.5-7b": (1.861e6, 1.845e6),      # mean over the 4 launches of a step
     "cfg5-ccm-hybrid-minicpm-v-2.6": (3.919e6, 1.468e6),
     # The decode launches were counted without the graph, 4 steps per bracket (the profiler cannot walk the long
