@@ -348,3 +348,28 @@ def test_snapkv_split_heuristic():
     assert ops.snapkv_splits(view(36, 1, 8, 32768, block_size=48), 32, 64) == 1
     assert ops.snapkv_splits(view(36, 1, 8, 32768, paged=False), 32, 64) == 8
     assert ops.snapkv_splits(view(4, 1, 1, 32768), 32, 64) == 1          # 64 row blocks per kv head
+
+
+def test_bench_counter_table_names_real_workloads():
+    """The HBM-counter table of bench.py is keyed by workload name: a key that no workload carries would silently
+    turn that workload's ``roofline.traffic`` into null.  Also the refusal of more than one GPU."""
+    import ast
+    import pathlib
+    import subprocess
+    import sys
+    root = pathlib.Path(__file__).resolve().parents[1]
+    src = (root / "bench.py").read_text()
+    names = {n.value for n in ast.walk(ast.parse(src))
+             if isinstance(n, ast.Constant) and isinstance(n.value, str) and n.value.startswith("cfg")}
+    names |= {n + "+given-lse" for n in names}
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_under_test", root / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert set(bench._COUNTER_KIB) <= names
+    for key, kib in bench._COUNTER_KIB.items():
+        t = bench._measured_traffic(key, kib[2] if len(kib) > 2 else 1)
+        assert t is not None and t > 0
+    assert bench._measured_traffic("no such workload", 1) is None
+    res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0 and "ONE GPU" in (res.stdout + res.stderr)
