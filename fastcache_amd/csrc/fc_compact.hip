@@ -60,8 +60,12 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   const KvView& dst = is_v ? dv : dk;
   const int tid = threadIdx.x, sub = tid % LPR, rg = tid / LPR;
   const int S = fc_seq_len(src, b);
+  // A count read from device memory is never trusted beyond what the host validated: the index row holds
+  // index_stride entries, and the destination (its block table included) max_seq_len tokens.
   int n = n_kept ? n_kept[b] : k;
-  if (!GATHER) n = min(n, S - src_start);
+  if (GATHER) n = min(n, index_stride);
+  else n = min(n, S - src_start);
+  n = min(n, dst.max_seq_len - dst_start);
   if (n <= 0) return;
 
   // block-table rows of this sequence (source and destination views may differ)

@@ -148,7 +148,7 @@ def topk_select(scores: torch.Tensor, k: int, row_lens: Optional[torch.Tensor] =
     """Indices of the ``k`` largest entries per row of ``scores[..., S]`` (fp32): ties to the lowest
     index, output ascending, int32 ``[..., k]``.  With ``row_lens``/``n_kept`` (int32 ``[B]``) rows
     ordered (..., b, head) take their valid length and kept count from entry ``b``
-    (``rows_per_len`` = heads per b); entries past a row's kept count are left at -1."""
+    (``rows_per_len`` = heads per b); entries past a row's kept count (or valid length) are -1."""
     _lib.require_gpu(scores, "scores")
     if scores.dtype != torch.float32 or scores.stride(-1) != 1:
         raise FastcacheError("scores must be fp32 with a contiguous last axis")
@@ -171,7 +171,7 @@ def topk_select(scores: torch.Tensor, k: int, row_lens: Optional[torch.Tensor] =
     n_kept = _i32(n_kept, "n_kept", dev)
     per_row = row_lens is not None or n_kept is not None
     mod = (row_lens if row_lens is not None else n_kept).numel() if per_row else 1
-    if n_kept is not None:
+    if per_row:
         out = torch.full((*scores.shape[:-1], k), -1, dtype=torch.int32, device=dev)
     else:
         out = torch.empty((*scores.shape[:-1], k), dtype=torch.int32, device=dev)
@@ -482,3 +482,4 @@ def decode_attn(k_cache: FcKvView, v_cache: FcKvView, layer: int, q: torch.Tenso
                                context_lens.data_ptr(), scale, workspace.data_ptr(), workspace.numel(),
                                current_stream()), "fc_decode_attn")
     return out
+

@@ -120,6 +120,52 @@ def test_compact_paged_in_place_with_kept_counts(dev, dtype, block_size):
     assert bool((after[:, :, spare] == 7.0).all())
 
 
+@pytest.mark.parametrize("paged", [True, False])
+def test_compact_clamps_device_side_kept_counts(dev, paged):
+    """A kept count in device memory that exceeds the index row (or the destination) is cut to what the host
+    validated: rows past the index stride, other sequences' pages and spare pages keep their bytes."""
+    L, H, lens, K = 1, 2, [300, 280], 40
+    B = len(lens)
+    case = synth.make_paged_case(seed=9, num_layers=L, batch=B, num_kv_heads=H, seq_lens=lens, dtype=torch.bfloat16,
+                                 keep_dense=True, fill_value=3.0)
+    g = torch.Generator().manual_seed(2)
+    idx = torch.stack([torch.sort(torch.randperm(280, generator=g)[:K]).values.int() for _ in range(L * B * H)])
+    idx = idx.view(L, B, H, K)
+    bogus = torch.tensor([K + 100000, 2 ** 31 - 1], dtype=torch.int32, device=dev)   # far beyond the index rows
+    if paged:
+        pool = case.kv_cache.to(dev)
+        before = pool.cpu().clone()
+        tab, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+        views = [_lib.paged_view(pool[p], tab, lens_d, max(lens)) for p in range(2)]
+        ops.compact(views[0], views[1], views[0], views[1], idx.to(dev), n_kept=bogus)
+        torch.cuda.synchronize()
+        after = pool.cpu()
+        for b in range(B):
+            blocks = case.block_tables[b]
+            for p, dense in enumerate((case.dense_k, case.dense_v)):
+                rows = torch.cat([after[p, 0, blk] for blk in blocks])                      # [tokens, H, D]
+                want = opress.gather_tokens(dense[0][b:b + 1, :, :lens[b]], idx[0, b:b + 1].long())[0]
+                assert torch.equal(rows[:K].permute(1, 0, 2), want), (b, p)
+                old = torch.cat([before[p, 0, blk] for blk in blocks])
+                assert torch.equal(rows[K:], old[K:]), "rows past the index stride were touched"
+        used = {blk for t in case.block_tables for blk in t}
+        spare = [i for i in range(after.shape[2]) if i not in used]
+        assert bool((after[:, :, spare] == 3.0).all())
+    else:
+        k = case.dense_k[0].to(dev).contiguous()          # [B, H, S, D]
+        v = case.dense_v[0].to(dev).contiguous()
+        src = [_lib.dense_view(k), _lib.dense_view(v)]
+        guard = torch.full((2, B, H, K + 8, 128), 5.0, dtype=torch.bfloat16, device=dev)
+        dst = [_lib.dense_view(guard[p, :, :, :K]) for p in range(2)]                       # K rows, 8 guard rows behind
+        ops.compact(src[0], src[1], dst[0], dst[1], idx.to(dev), n_kept=bogus)
+        torch.cuda.synchronize()
+        out = guard.cpu()
+        assert bool((out[:, :, :, K:] == 5.0).all()), "rows past the destination were written"
+        for p, dense in enumerate((case.dense_k, case.dense_v)):
+            want = opress.gather_tokens(dense[0][:, :, :280], idx[0].long())
+            assert torch.equal(out[p, :, :, :K], want)
+
+
 def test_compact_rejects_bad_arguments(dev):
     k = torch.zeros(1, 1, 2, 8, 128, device=dev)
     view = _lib.dense_view(k)
