@@ -91,6 +91,8 @@ SIGNATURES = {
     "fc_advance_lens": (C.c_int, [_VP, _I, _I, _VP]),
     "fc_decode_attn_workspace_bytes": (C.c_int64, [_I, _I, _I]),
     "fc_decode_attn": (C.c_int, [_V, _V, _I, _VP, _VP, _I, _VP, _F, _VP, C.c_int64, _VP]),
+    "fc_decode_attn_static_capacity": (C.c_int64, []),
+    "fc_decode_attn_static": (C.c_int, [_V, _V, _I, _VP, _VP, _I, _VP, _F, _VP]),
 }
 
 

@@ -493,10 +493,10 @@ extern "C" int64_t fc_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_h
   return (int64_t)batch * num_q_heads * (splits > 0 ? splits : 1) * (FC_HEAD_DIM + 2) * (int64_t)sizeof(float);
 }
 
-extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer, const void* q,
-                              void* out, int32_t num_q_heads, const int32_t* context_lens, float scale,
-                              void* workspace, int64_t workspace_bytes, void* stream) {
-  const char* who = "fc_decode_attn";
+// Checks and launches shared by the entry points; `workspace` is a device address.
+static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer,
+                      const void* q, void* out, int32_t num_q_heads, const int32_t* context_lens, float scale,
+                      void* workspace, int64_t workspace_bytes, void* stream) {
   int rc;
   if ((rc = fc_check_view(k_cache, who)) || (rc = fc_check_view(v_cache, who))) return rc;
   FC_REQUIRE(k_cache->dtype == v_cache->dtype && k_cache->num_layers == v_cache->num_layers &&
@@ -562,4 +562,47 @@ extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cac
                        k_cache->max_seq_len, num_q_heads, splits, (char*)out);
   FC_CHECK_LAUNCH(who);
   return FC_OK;
+}
+
+extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer, const void* q,
+                              void* out, int32_t num_q_heads, const int32_t* context_lens, float scale,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
+  return da_enqueue("fc_decode_attn", k_cache, v_cache, layer, q, out, num_q_heads, context_lens, scale, workspace,
+                    workspace_bytes, stream);
+}
+
+// ---- the same attention for callers that cannot allocate -------------------------------------------------
+// The chunk partials live in a file-scope device array instead of a caller workspace.  `scratch` below is the
+// host-side handle of that array, not a device address: its address on the current device is looked up once
+// per device (every GPU holds its own copy) and only that address is ever handed to a kernel.
+#define DA_STATIC_BYTES (16ll << 20)
+static __device__ __align__(256) unsigned char scratch[DA_STATIC_BYTES];
+
+#define DA_MAX_DEVICES 64
+static void* da_scratch_ptr[DA_MAX_DEVICES];   // filled per device on first use; a repeated look-up gives the same value
+
+extern "C" int64_t fc_decode_attn_static_capacity(void) { return DA_STATIC_BYTES; }
+
+extern "C" int fc_decode_attn_static(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer,
+                                     const void* q, void* out, int32_t num_q_heads, const int32_t* context_lens,
+                                     float scale, void* stream) {
+  const char* who = "fc_decode_attn_static";
+  FC_REQUIRE(k_cache && num_q_heads > 0, FC_EINVAL, "%s: null view or bad head count", who);
+  const int64_t need = fc_decode_attn_workspace_bytes(k_cache->batch, num_q_heads, k_cache->max_seq_len);
+  FC_REQUIRE(need > 0, FC_EINVAL, "%s: bad sizes", who);
+  FC_REQUIRE(need <= DA_STATIC_BYTES, FC_EUNSUPPORTED,
+             "%s: batch %d x %d query heads x max_seq_len %d needs %lld bytes of chunk partials, the built-in "
+             "buffer holds %lld; use fc_decode_attn with a workspace",
+             who, k_cache->batch, num_q_heads, k_cache->max_seq_len, (long long)need, (long long)DA_STATIC_BYTES);
+  int dev = -1;
+  FC_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < DA_MAX_DEVICES, FC_EUNSUPPORTED,
+             "%s: no current device below %d", who, DA_MAX_DEVICES);
+  void* ws = da_scratch_ptr[dev];
+  if (!ws) {
+    const hipError_t e = hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch));
+    FC_REQUIRE(e == hipSuccess && ws, FC_ELAUNCH, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+    da_scratch_ptr[dev] = ws;
+  }
+  return da_enqueue(who, k_cache, v_cache, layer, q, out, num_q_heads, context_lens, scale, ws, DA_STATIC_BYTES,
+                    stream);
 }

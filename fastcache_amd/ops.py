@@ -483,3 +483,20 @@ def decode_attn(k_cache: FcKvView, v_cache: FcKvView, layer: int, q: torch.Tenso
                                current_stream()), "fc_decode_attn")
     return out
 
+
+
+def decode_attn_static(k_cache: FcKvView, v_cache: FcKvView, layer: int, q: torch.Tensor,
+                       context_lens: torch.Tensor, scale: float, out: torch.Tensor) -> torch.Tensor:
+    """``decode_attn`` with the chunk partials in the library's built-in device buffer: the call allocates
+    nothing (``out`` is the caller's).  Calls that overlap on one GPU share that buffer and race."""
+    _lib.require_gpu(q, "q")
+    if q.dim() != 3 or not q.is_contiguous() or _lib.dtype_code(q.dtype) != k_cache.dtype:
+        raise FastcacheError("q must be contiguous [B, Hq, D] in the cache dtype")
+    if out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+        raise FastcacheError("out must be a contiguous tensor shaped and typed like q")
+    _lib.require_gpu(out, "out")
+    _i32(context_lens, "context_lens", q.device)
+    check(fn("fc_decode_attn_static")(C.byref(k_cache), C.byref(v_cache), layer, q.data_ptr(), out.data_ptr(),
+                                      q.shape[1], context_lens.data_ptr(), scale, current_stream()),
+          "fc_decode_attn_static")
+    return out

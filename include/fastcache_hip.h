@@ -372,6 +372,21 @@ int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t
                    const void* q, void* out, int32_t num_q_heads, const int32_t* context_lens,
                    float scale, void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * fc_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the chunk partials go to a buffer built into the library, a
+ * file-scope device array of fc_decode_attn_static_capacity() bytes (16 MiB) that every GPU the library runs on
+ * holds until the process ends.  No counterpart in the reference.  Same arguments and results as fc_decode_attn
+ * minus the workspace; the call allocates nothing and frees nothing.  Shapes whose
+ * fc_decode_attn_workspace_bytes() exceed the capacity are rejected with FC_EUNSUPPORTED.  All calls on one GPU
+ * share the one buffer: calls that overlap on a GPU (different streams, concurrent graphs) race; calls on one
+ * stream are ordered and safe.  Nothing in the buffer has to start at zero, so no clearing is done.
+ */
+int64_t fc_decode_attn_static_capacity(void);
+int fc_decode_attn_static(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer,
+                          const void* q, void* out, int32_t num_q_heads, const int32_t* context_lens,
+                          float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
