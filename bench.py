@@ -2,19 +2,30 @@
 """Benchmark of the KV-cache compression path on one MI355X.
 
 ``python bench.py --gpus 1 --steps K --warmup W`` prints ONE JSON line.  A step is one pass of the
-hot path over one batch of synthetic input that is already resident in HBM.  The default workload
-is configuration 2 (SnapKV press over a Qwen3-8B-shaped paged pool: score -> window fill -> top-k
--> in-place compaction, all 36 layers, batch 8, 4096 tokens per sequence).  ``--workload`` selects
-the other configurations (knorm, ccm, decode, hybrid, hybrid-decode = the 64 decode steps of
-configuration 5; decode-eager = the decode launches without a
-graph, for the profiler; snapkv-lse = cfg2 with the window queries' log-sum-exp given, single pass over K); they are measured the same way.
+hot path over one batch of synthetic input that is already resident in HBM.  Without ``--workload``
+the line's headline (``value``, ``roofline``, ``cpu_baseline``) is configuration 2 (SnapKV press over a
+Qwen3-8B-shaped paged pool: score -> window fill -> top-k -> in-place compaction, all 36 layers, batch 8,
+4096 tokens per sequence), ``decode_tokens_per_s`` is configuration 4 (128 decode steps in one HIP graph),
+and ``configs`` holds the same measurement of every configuration: ms per step, throughput, roofline of the
+dominant kernel, CPU baseline, and the result of the check below.  ``--workload`` measures one
+configuration alone (knorm, snapkv, ccm, decode, hybrid, hybrid-decode = the 64 decode steps of
+configuration 5; decode-eager / hybrid-decode-eager = the decode launches without a graph, the variants
+to run under a profiler; snapkv-lse = cfg2 with the window queries' log-sum-exp given; copy = the
+calibration copy of the traffic counters).
 
-Extra objects on the line:
+Objects on the line:
   roofline      the dominant kernel of the workload: algorithmic bytes per launch divided by its
                 average launch time, measured with HIP events on the launch stream inside the timed
-                region, against the published 8 TB/s HBM peak;
+                region, against the published 8 TB/s HBM peak; ``traffic`` is the HBM byte count of one
+                launch from an earlier rocprofv3 counter run of the same workload (``traffic_recorded``
+                says of which commit and when), not a measurement of this run;
   cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this host on a bounded
-                sample of the same workload and scaled to the full pass.
+                sample of the same workload and scaled to the full pass;
+  checked       one sampled (layer, sequence) column of the step that precedes the timed ones, compared with
+                the oracle (scores / outputs within the parity tolerance, indices and moved bytes exact).
+
+The graph workloads are refused under rocprofv3 (the profiler has crashed while tracing the long graphs);
+use the ``*-eager`` variants there.
 """
 from __future__ import annotations
 
@@ -40,10 +51,23 @@ def _sync_time():
     return time.perf_counter()
 
 
+CPU_THREAD_CAP = 16            # the share of host cores one GPU of the box comes with
+
+
 def _cpu_threads():
-    n = min(os.cpu_count() or 1, 16)
+    n = min(os.cpu_count() or 1, CPU_THREAD_CAP)
     torch.set_num_threads(n)
     return n
+
+
+def _cpu_info(threads):
+    """cores = threads the baseline actually used; the host's own count is stated beside it."""
+    return {"cores": threads, "threads": torch.get_num_threads(), "host_cpu_count": os.cpu_count()}
+
+
+def _under_profiler():
+    """rocprofv3 announces itself through ROCPROF* / ROCP_* variables before the program starts."""
+    return any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
 
 
 class Bracket:
@@ -77,6 +101,44 @@ class Workload:
 
     def __init__(self):
         self.br = Bracket()
+        self.keep = False        # set for the checked step: the step keeps what check_after() needs
+        self.kept = None
+
+    # One sampled (layer, sequence) column of one step (the one before the timed steps) against the oracle:
+    # check_before() snapshots the column's inputs, the step keeps references to its outputs, check_after()
+    # compares and returns a summary or raises.  The line reports "checked".
+    def check_before(self):
+        pass
+
+    def check_after(self):
+        return None
+
+
+def _column_dense(kv_cache, plane, layer, table, n):
+    """Tokens [0, n) of one sequence of one layer as a CPU tensor [1, Hkv, n, D] (HuggingFace layout)."""
+    bs = kv_cache.shape[3]
+    blocks = torch.as_tensor(list(table)[:(n + bs - 1) // bs], device=kv_cache.device, dtype=torch.long)
+    rows = kv_cache[plane, layer, blocks].reshape(-1, kv_cache.shape[4], kv_cache.shape[5])[:n]
+    return rows.permute(1, 0, 2).unsqueeze(0).cpu()
+
+
+def _check_press_column(name, before_k, before_v, after_k, after_v, scores, ref_scores, idx, n_scored):
+    """scores within 1e-3 of the oracle, indices = the oracle's stable selection on these scores, moved rows exact."""
+    from oracle import presses as opress
+    sc, ref = scores[..., :n_scored].cpu(), ref_scores[..., :n_scored]
+    tol = 1e-3 * ref.abs() + 1e-3 * float(ref.abs().mean())
+    if not bool(((sc - ref).abs() <= tol).all()):
+        raise AssertionError(f"{name}: scores of the sampled column differ from the oracle by "
+                             f"{float(((sc - ref).abs() / tol).max()):.2f} x the tolerance")
+    want = opress.topk_lowest_index(scores.cpu(), idx.shape[-1])
+    if not torch.equal(want, idx.cpu().long()):
+        raise AssertionError(f"{name}: kept indices differ from the stable top-k of the scores")
+    n = idx.shape[-1]
+    for tag, b4, aft in (("K", before_k, after_k), ("V", before_v, after_v)):
+        if not torch.equal(opress.gather_tokens(b4, idx.cpu().long().unsqueeze(0)), aft[:, :, :n]):
+            raise AssertionError(f"{name}: compacted {tag} rows differ from the gathered source rows")
+    return {"column": name, "scores_max_err_over_tol": round(float(((sc - ref).abs() / tol).max()), 4),
+            "indices": "exact", "bytes": "exact"}
 
 
 # ---------------------------------------------------------------------------------------------------
@@ -158,6 +220,24 @@ class SnapKVWorkload(Workload):
                                           row_max.data_ptr(), st), "fc_snapkv_fill_window")
         idx = ops.topk_select(scores, self.n_kept)
         ops.compact(kview, vview, kview, vview, idx)
+        if self.keep:
+            self.kept, self.keep = (scores, idx), False
+
+    def check_before(self):
+        self.cl, self.cb = self.L // 2, self.B // 2
+        tab = self.case.block_tables[self.cb]
+        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
+        self.keep = True
+
+    def check_after(self):
+        from oracle import presses as opress
+        scores, idx = self.kept
+        l, b = self.cl, self.cb
+        ref = opress.snapkv_score(self.queries[l, b:b + 1].cpu(), self.snap[0], self.W, self.ksz, True, "sum")[0]
+        tab = self.case.block_tables[b]
+        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]
+        return _check_press_column(f"layer {l}, sequence {b}", self.snap[0], self.snap[1], after[0], after[1],
+                                   scores[l, b], ref, idx[l, b], self.S - self.W)
 
     def cpu_baseline(self, budget_s=12.0):
         """CPU restatement of the same pass, layer by layer until the time budget, scaled linearly."""
@@ -179,7 +259,7 @@ class SnapKVWorkload(Workload):
             if t_total > budget_s:
                 break
         full_pass_s = t_total / layers_done * self.L
-        return {"value": round(self.tokens_per_step / full_pass_s, 1), "unit": self.unit, "cores": threads,
+        return {"value": round(self.tokens_per_step / full_pass_s, 1), "unit": self.unit, **_cpu_info(threads),
                 "kind": "port",
                 "sample": f"{layers_done} of {self.L} layers x all {self.B} sequences, "
                           f"{t_total:.2f} s measured, scaled linearly to the full pass"}
@@ -219,6 +299,23 @@ class KnormWorkload(Workload):
         idx = ops.topk_select(scores, self.n_kept)
         with self.br:
             ops.compact(kview, vview, kview, vview, idx)
+        if self.keep:
+            self.kept, self.keep = (scores, idx), False
+
+    def check_before(self):
+        self.cl = self.L // 2
+        tab = self.case.block_tables[0]
+        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
+        self.keep = True
+
+    def check_after(self):
+        from oracle import presses as opress
+        scores, idx = self.kept
+        l = self.cl
+        tab = self.case.block_tables[0]
+        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]
+        return _check_press_column(f"layer {l}, sequence 0", self.snap[0], self.snap[1], after[0], after[1],
+                                   scores[l, 0], opress.knorm_score(self.snap[0])[0], idx[l, 0], self.S)
 
     def cpu_baseline(self, budget_s=12.0):
         from oracle import pipeline as opipe
@@ -229,7 +326,7 @@ class KnormWorkload(Workload):
         t0 = time.perf_counter()
         opipe.compress_batch(pool, self.case.block_tables, [self.S], comp)
         dt = time.perf_counter() - t0
-        return {"value": round(self.tokens_per_step / dt, 1), "unit": self.unit, "cores": threads, "kind": "port",
+        return {"value": round(self.tokens_per_step / dt, 1), "unit": self.unit, **_cpu_info(threads), "kind": "port",
                 "sample": f"the full pass (all {self.L} layers), {dt:.2f} s"}
 
 
@@ -287,6 +384,35 @@ class CCMWorkload(Workload):
         with self.br:
             self.module.paged_forward(self.case.kv_cache, self.tables, self.lens, self.S, self.it_len)
 
+    def check_before(self):
+        self.cl, self.cb = self.L // 2, self.B // 2
+        tab = self.case.block_tables[self.cb]
+        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
+
+    def check_after(self):
+        """Compressed rows of the sampled column: error norm within 1e-3 of the oracle's norm (both sides
+        accumulate in fp32 and round to the storage dtype after every Linear)."""
+        from oracle import ccm as occm
+        l, b = self.cl, self.cb
+        sd = {}
+        for k, v in self.module.state_dict().items():          # keys are group.layer.index.name
+            g, lay, rest = k.split(".", 2)
+            if int(lay) == l:
+                sd[f"{g}.0.{rest}"] = v.detach().cpu().float()
+        fwd = occm.hybrid_forward if self.hybrid else occm.linear_decouple_forward
+        (rk, rv), = fwd([(self.snap[0], self.snap[1])], self.it_len, sd, self.cf, 1)
+        tab = self.case.block_tables[b]
+        worst = 0.0
+        for p, ref in enumerate((rk, rv)):
+            got = _column_dense(self.case.kv_cache, p, l, tab, self.C).float()
+            ref = ref.float()
+            assert got.shape == ref.shape, (got.shape, ref.shape)
+            rel = float((got - ref).norm() / ref.norm())
+            worst = max(worst, rel)
+            if rel > 1e-3:
+                raise AssertionError(f"cfg MLP: layer {l}, sequence {b}, plane {p}: relative error norm {rel:.2e}")
+        return {"column": f"layer {l}, sequence {b}", "rel_error_norm": float(f"{worst:.3e}")}
+
     def cpu_baseline(self, budget_s=12.0):
         from oracle import ccm as occm
         from oracle import pipeline as opipe
@@ -314,7 +440,7 @@ class CCMWorkload(Workload):
             if t_total > budget_s:
                 break
         full = t_total / done * self.L * (self.B / nb)
-        return {"value": round(self.tokens_per_step / full, 1), "unit": self.unit, "cores": threads, "kind": "port",
+        return {"value": round(self.tokens_per_step / full, 1), "unit": self.unit, **_cpu_info(threads), "kind": "port",
                 "sample": f"{done} of {self.L} layers x {nb} of {self.B} sequences, {t_total:.2f} s measured, "
                           "scaled linearly to the full pass"}
 
@@ -380,6 +506,24 @@ class DecodeWorkload(Workload):
             else:
                 self.dg.replay()
 
+    def check_after(self):
+        """Attention outputs of a few sequences at the first and last step of one layer (every replay appends the
+        same rows, so the pool holds the final state): within 2e-2 absolute of the fp32 oracle."""
+        from oracle import attention as oattn
+        torch.cuda.synchronize()
+        layer, seqs = self.L // 2, [0, self.B // 2, self.B - 1]
+        kc, vc = self.case.kv_cache[0, layer].cpu(), self.case.kv_cache[1, layer].cpu()
+        tab = self.tables[seqs].cpu()
+        worst = 0.0
+        for t in (0, self.T - 1):
+            lens = (self.lens0[seqs] + (t + 1)).cpu()
+            ref = oattn.decode_attention(self.dg.q_steps[t, layer, seqs].cpu(), kc, vc, lens, tab, D ** -0.5)
+            err = float((self.dg.out[t, layer, seqs].cpu().float() - ref.float()).abs().max())
+            worst = max(worst, err)
+            if err > 2e-2:
+                raise AssertionError(f"decode: layer {layer}, step {t}: attention output off by {err:.3e}")
+        return {"column": f"layer {layer}, sequences {seqs}, steps 0 and {self.T - 1}", "max_abs_err": float(f"{worst:.3e}")}
+
     def cpu_baseline(self, budget_s=12.0):
         from oracle import attention as oattn
         threads = _cpu_threads()
@@ -396,7 +540,7 @@ class DecodeWorkload(Workload):
         dt = (time.perf_counter() - t0) / reps
         share = float(lens.sum()) / float(self.lens0.sum())
         step_s = dt / share * self.L
-        return {"value": round(self.B / step_s, 1), "unit": self.unit, "cores": threads, "kind": "port",
+        return {"value": round(self.B / step_s, 1), "unit": self.unit, **_cpu_info(threads), "kind": "port",
                 "sample": f"attention of {nb} of {self.B} sequences, 1 of {self.L} layers, {reps} repetitions, "
                           "scaled by cached tokens and layers to one decode step"}
 
@@ -436,7 +580,7 @@ class CopyWorkload(Workload):
         t0 = time.perf_counter()
         b = a.clone()
         dt = time.perf_counter() - t0
-        return {"value": round(a.shape[0] * a.shape[2] / dt, 1), "unit": self.unit, "cores": threads, "kind": "port",
+        return {"value": round(a.shape[0] * a.shape[2] / dt, 1), "unit": self.unit, **_cpu_info(threads), "kind": "port",
                 "sample": "torch clone of 1 of 4 sequences on the host"}
 
 
@@ -456,6 +600,7 @@ WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkl
 # copy workload below, whose traffic is known (512 MiB read, 512 MiB written):
 #   copy:   FETCH_SIZE 2.623e5 KiB -> scale 1.999;  WRITE_SIZE 5.244e5 KiB -> scale 1.000
 # The commands and raw readings are in profiles/*_hbm_traffic.txt.
+_COUNTER_RUN = {"commit": "3ee0b1a", "date": "2026-11-25"}   # the tree whose kernels the counter runs below measured
 _FETCH_SCALE = 524288 / 2.623e5
 _WRITE_SCALE = 524288 / 5.244e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
@@ -480,20 +625,77 @@ def _measured_traffic(workload_name, algorithmic_bytes_per_launch):
     return int(round((kib[0] * _FETCH_SCALE + kib[1] * _WRITE_SCALE) * 1024 * scale))
 
 
+GRAPH_WORKLOADS = {"decode": "decode-eager", "hybrid-decode": "hybrid-decode-eager"}
+
+
+def measure(workload, seed, dev, steps, warmup, cpu_baseline=True, cpu_budget_s=12.0, check=True):
+    """One workload: warm-up, one checked + timed run of `steps` steps, roofline of the dominant kernel."""
+    w = WORKLOADS[workload](seed, dev)
+    for _ in range(warmup):
+        w.step()
+    checked = None
+    if check:                              # one step of its own, right before the timed ones
+        w.check_before()
+        w.step()
+        checked = w.check_after()          # raises when the sampled column is off: no number without a right result
+    w.br.on = True
+    t0 = _sync_time()
+    for _ in range(steps):
+        w.step()
+    t1 = _sync_time()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    value = w.tokens_per_step / (ms_per_step * 1e-3)
+
+    # the bracket may hold several launches of the dominant kernel: bytes and time are summed over
+    # them, which equals (mean bytes per launch) / (mean launch duration)
+    k_ms = w.br.mean_ms() / w.launches_per_bracket
+    per_launch = w.kernel_bytes // w.launches_per_bracket
+    achieved = w.kernel_bytes / w.launches_per_bracket / (k_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": w.kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": _measured_traffic(w.name, per_launch),
+                "traffic_recorded": _COUNTER_RUN if w.name in _COUNTER_KIB else None,
+                "kernel_ms": round(k_ms, 4), "launches_per_step": w.launches_per_bracket,
+                "algorithmic_bytes_per_launch": per_launch,
+                "pass_gbs": round(w.pass_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+                "pass_frac": round(w.pass_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    if w.kernel_flops:
+        tf = w.kernel_flops / w.launches_per_bracket / (k_ms * 1e-3) / 1e12
+        roofline["mfma_tflops"] = round(tf, 1)
+        roofline["mfma_frac"] = round(tf / MFMA_PEAK_TFLOPS, 4)
+    out = {"metric": w.metric, "value": round(value, 1), "unit": w.unit, "ms_per_step": round(ms_per_step, 4),
+           "steps": steps, "warmup": warmup, "dtype": w.dtype_name, "config": w.config(), "roofline": roofline,
+           "checked": checked is not None, "check": checked}
+    if cpu_baseline:
+        out["cpu_baseline"] = w.cpu_baseline(cpu_budget_s)
+    del w
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="snapkv")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
+                    help="one configuration alone; default: cfg2 as the headline plus every configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
 
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no sharding); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         sys.exit(2)
+    profiled = _under_profiler()
+    if profiled and args.workload in GRAPH_WORKLOADS:
+        # before any GPU call: rocprofv3 has ended in a segmentation fault while tracing the long decode graphs
+        print(f"bench.py: --workload {args.workload} replays a HIP graph of thousands of nodes and is not run under "
+              f"rocprofv3; profile --workload {GRAPH_WORKLOADS[args.workload]} (the same launches without a graph)",
+              file=sys.stderr)
+        sys.exit(3)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
@@ -501,39 +703,29 @@ def main():
     _lib.load()          # fail loudly when the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    cpu, check = not args.no_cpu_baseline, not args.no_check
 
-    w = WORKLOADS[args.workload](args.seed, dev)
-    for _ in range(args.warmup):
-        w.step()
-    w.br.on = True
-    t0 = _sync_time()
-    for _ in range(args.steps):
-        w.step()
-    t1 = _sync_time()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    value = w.tokens_per_step / (ms_per_step * 1e-3)
-
-    # the bracket may hold several launches of the dominant kernel: bytes and time are summed over
-    # them, which equals (mean bytes per launch) / (mean launch duration)
-    k_ms = w.br.mean_ms() / w.launches_per_bracket
-    achieved = w.kernel_bytes / w.launches_per_bracket / (k_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": w.kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _measured_traffic(w.name, w.kernel_bytes // w.launches_per_bracket),
-                "kernel_ms": round(k_ms, 4), "launches_per_step": w.launches_per_bracket,
-                "algorithmic_bytes_per_launch": w.kernel_bytes // w.launches_per_bracket,
-                "pass_gbs": round(w.pass_bytes / (ms_per_step * 1e-3) / 1e9, 1),
-                "pass_frac": round(w.pass_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
-    if w.kernel_flops:
-        tf = w.kernel_flops / w.launches_per_bracket / (k_ms * 1e-3) / 1e12
-        roofline["mfma_tflops"] = round(tf, 1)
-        roofline["mfma_frac"] = round(tf / MFMA_PEAK_TFLOPS, 4)
-
-    out = {"metric": w.metric, "value": round(value, 1), "unit": w.unit, "n_gpus": 1,
-           "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": w.dtype_name,
-           "data": "synthetic", "config": w.config(), "roofline": roofline}
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = w.cpu_baseline()
+    head_name = args.workload or "snapkv"
+    head = measure(head_name, args.seed, dev, args.steps, args.warmup, cpu, 12.0, check)
+    out = {"metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+           "data": "synthetic", "config": head["config"], "roofline": head["roofline"], "checked": head["checked"],
+           "check": head["check"]}
+    if cpu:
+        out["cpu_baseline"] = head["cpu_baseline"]
+    if args.workload is None:
+        # every configuration on the same line; the decode graphs give way to their eager forms under a profiler
+        configs = {"cfg2": head}
+        plan = [("cfg1", "knorm", 10, 3), ("cfg3", "ccm", 10, 3), ("cfg4", "decode", 3, 1),
+                ("cfg5-compress", "hybrid", 10, 3), ("cfg5-decode", "hybrid-decode", 5, 2)]
+        for key, name, steps, warmup in plan:
+            if profiled and name in GRAPH_WORKLOADS:
+                name = GRAPH_WORKLOADS[name]
+            configs[key] = measure(name, args.seed, dev, steps, warmup, cpu, 6.0, check)
+        out["configs"] = configs
+        out["decode_tokens_per_s"] = configs["cfg4"]["value"]
+        out["decode_tokens_per_s_after_compression"] = configs["cfg5-decode"]["value"]
     print(json.dumps(out), flush=True)
 
 

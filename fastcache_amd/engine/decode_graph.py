@@ -37,8 +37,8 @@ class DecodeGraph:
         self.vview = _lib.paged_view(kv_cache[1], block_tables, None, self.max_len)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
 
-    def _enqueue(self) -> None:
-        for t in range(self.steps):
+    def _enqueue(self, steps: Optional[int] = None) -> None:
+        for t in range(self.steps if steps is None else steps):
             ops.store_kv(self.kview, self.vview, self.k_steps[t], self.v_steps[t], self.context_lens)
             ops.advance_lens(self.context_lens, 1)
             for layer in range(self.num_layers):
@@ -53,6 +53,12 @@ class DecodeGraph:
     def capture(self) -> None:
         """Record all steps.  ``context_lens`` is restored afterwards (capture does not execute)."""
         saved = self.context_lens.clone()
+        # One step outside the graph first: whatever a kernel's first launch does on the host (loading its code
+        # object, raising its LDS limit) happens here and not inside the capture.  It appends the rows the
+        # replays will append anyway and its lengths are put back.
+        self._enqueue(1)
+        torch.cuda.synchronize()
+        self.context_lens.copy_(saved)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):

@@ -373,3 +373,21 @@ def test_bench_counter_table_names_real_workloads():
     assert bench._measured_traffic("no such workload", 1) is None
     res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode != 0 and "ONE GPU" in (res.stdout + res.stderr)
+
+
+def test_bench_refuses_graph_workloads_under_the_profiler():
+    """The decode-graph workloads exit before any GPU call when the profiler's environment is present, naming the
+    eager variant to use; the eager variants and the other workloads are not refused on that ground."""
+    import os
+    import pathlib
+    import subprocess
+    import sys
+    root = pathlib.Path(__file__).resolve().parents[1]
+    env = dict(os.environ, ROCPROF_OUTPUT_PATH="/tmp/x")
+    for name, eager in (("decode", "decode-eager"), ("hybrid-decode", "hybrid-decode-eager")):
+        res = subprocess.run([sys.executable, str(root / "bench.py"), "--workload", name], capture_output=True,
+                             text=True, env=env)
+        assert res.returncode == 3 and eager in res.stderr, (res.returncode, res.stderr)
+    res = subprocess.run([sys.executable, str(root / "bench.py"), "--workload", "decode-eager"], capture_output=True,
+                         text=True, env=env)
+    assert res.returncode == 1 and "no GPU" in res.stderr          # passed the fence, stopped at the missing GPU
