@@ -85,7 +85,7 @@ def snapkv_score(queries: torch.Tensor, keys: torch.Tensor, window_size: int, ke
     k_rep = keys.float().repeat_interleave(G, dim=1)                     # repeat_kv
     logits = torch.matmul(queries.float(), k_rep.transpose(2, 3)) * scale  # [B,Hq,W,S]
     if causal_window:
-        mask = torch.full((W, S), float("-inf"))
+        mask = torch.full((W, S), float("-inf"), device=logits.device)
         mask = torch.triu(mask, diagonal=S - W + 1)
         logits = logits + mask
     attn = F.softmax(logits, dim=-1, dtype=torch.float32)
@@ -214,7 +214,7 @@ def near_tie_rows(scores: torch.Tensor, k: int, rel: float = 1e-5) -> torch.Tens
     set is not determined at fp32 scoring accuracy and is left out of index comparisons."""
     s = scores.float()
     if k <= 0 or k >= s.shape[-1]:
-        return torch.zeros(s.shape[:-1], dtype=torch.bool)
+        return torch.zeros(s.shape[:-1], dtype=torch.bool, device=s.device)
     top = torch.topk(s, k + 1, dim=-1).values
     a, b = top[..., k - 1], top[..., k]
     return (a - b).abs() < rel * a.abs()

@@ -32,3 +32,15 @@ def dev():
     import torch
     assert torch.cuda.is_available(), "gpu test selected but no GPU visible"
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Observed worst cases of the MLP parity checks of this run (the tolerance they are held to is calibrated
+    on the CPU; these are the figures of the HIP path)."""
+    mod = sys.modules.get("test_gpu_ccm")
+    obs = getattr(mod, "OBSERVED", None) if mod else None
+    if obs:
+        terminalreporter.write_line(
+            f"MLP parity, {len(obs)} comparisons, {sum(o[0] for o in obs)} elements: worst relative error norm "
+            f"{max(o[1] for o in obs):.3e}, elements beyond 1e-3*max|ref| + 2 ulp: {sum(o[2] for o in obs)}, "
+            f"largest error {max(o[3] for o in obs):.3e} of max|ref|")

@@ -4,8 +4,9 @@ Tolerance.  Both sides accumulate in fp32 and round to the storage dtype after e
 a different summation order, so a hidden activation can round to the neighbouring fp16/bf16 value
 and move the final output by about one unit in the last place of the storage dtype (2^-10 relative
 for fp16, 2^-7 for bf16).  The check is therefore: error norm / reference norm <= 1e-3, and every
-element within 1e-3 * max|ref| + 2 ulp(storage) of the reference, except for at most one element in
-10^3 (a flipped hidden activation times the output weights of its row), which must stay within 1 % of max|ref|.
+element within 1e-3 * max|ref| + 2 ulp(storage) of the reference; the few exceptions allowed in bf16 are what
+a CPU calibration with other fp32 summation orders shows (tests/test_oracle_pinning.py).  The observed figures
+of a run are printed at its end.
 """
 import pytest
 import torch
@@ -25,20 +26,33 @@ def stacked(sd, group, L, dtype, dev):
     return tuple(out)
 
 
-def assert_mlp_close(got, ref, dtype):
+OBSERVED = []   # (elements, relative error norm, elements beyond the bound, max error / max|ref|) of every call; printed at the end of the run
+
+
+def mlp_error_stats(got, ref, dtype):
+    """Relative error norm, number of elements beyond ``1e-3 * max|ref| + 2 ulp(storage) * |ref|``, and the
+    largest error over ``max|ref|``."""
     got, ref = got.float(), ref.float()
     ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
     scale = float(ref.abs().max())
     rel = float((got - ref).norm() / ref.norm())
-    assert rel <= 1e-3, f"relative error norm {rel:.3e}"
     err = (got - ref).abs()
     bound = 1e-3 * scale + 2 * ulp * ref.abs().clamp_min(scale * 2.0 ** -14)
-    # A hidden activation that sits on a rounding boundary of the storage dtype can round the other way
-    # (different summation order); its ulp times an output weight can exceed the bound for that one output
-    # row's 128 outputs.  Such elements must be rare (at most 1 in 10^3) and small (1 % of the largest value).
-    outliers = err > bound
-    assert int(outliers.sum()) <= max(8, err.numel() // 1000), f"{int(outliers.sum())} elements beyond the bound"
-    assert float(err.max()) <= 1e-2 * scale, f"max error {float(err.max()):.3e} vs scale {scale:.3e}"
+    return rel, int((err > bound).sum()), float(err.max()) / scale, err.numel()
+
+
+def assert_mlp_close(got, ref, dtype):
+    """The allowance is calibrated, not assumed: tests/test_oracle_pinning.py::test_mlp_tolerance_calibration
+    evaluates the oracle MLP under other fp32 summation orders.  fp16: no element beyond the bound.  bf16: a
+    hidden activation on a rounding boundary flips to the neighbouring value about 3 times in 10^7 outputs and
+    moves one output by up to 4.2e-3 of max|ref|.  Allowed here: fp16 none; bf16 one element plus two per
+    million (several times the measured rate), none further than 6.5e-3 of max|ref|."""
+    rel, n_out, worst, n = mlp_error_stats(got, ref, dtype)
+    OBSERVED.append((n, rel, n_out, worst))
+    assert rel <= 1e-3, f"relative error norm {rel:.3e}"
+    allowed = 0 if dtype == torch.float16 else 1 + n // 500_000
+    assert n_out <= allowed, f"{n_out} of {n} elements beyond 1e-3 * max|ref| + 2 ulp ({allowed} allowed)"
+    assert worst <= 6.5e-3, f"max error {worst:.3e} of max|ref|"
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

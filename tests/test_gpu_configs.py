@@ -1,8 +1,10 @@
 """The five benchmark configurations at full size on the GPU.
 
 Each test runs the whole pass at the configured shape and checks it (a) against the CPU oracle on
-a sample the oracle finishes in seconds, and (b) through size-independent properties over ALL of
-it: ascending unique in-range indices, gathered rows equal to the source rows they name, untouched
+a sample the oracle finishes in seconds, (b) against the same oracle functions evaluated in fp32 on
+device tensors for EVERY (layer, sequence, head) column (an independent PyTorch reference at full size:
+rocBLAS matrix products and torch reductions, none of this library's kernels), and (c) through
+size-independent properties over all of it: ascending unique in-range indices, gathered rows equal to the source rows they name, untouched
 bytes past the compressed length, two independent code paths (paged in place vs dense out of place)
 agreeing bit for bit, graph replays equal to eager launches, block accounting invariants.
 """
@@ -52,6 +54,22 @@ def check_compaction(pool_after, pool_before, tables, idx, S, n):
         assert torch.equal(after[:, :, :, n:], before[:, :, :, n:])
 
 
+def check_selection_against_scores(idx, ref_scores, n, rel=1e-5):
+    """Kept sets of every row against the stable top-n of the reference scores.  A position may differ between the
+    two sets only if its reference score lies within ``rel`` (relative) of the row's n-th largest score: such
+    positions are not decided at fp32 scoring accuracy.  Returns the number of positions that differ."""
+    rows = ref_scores.reshape(-1, ref_scores.shape[-1])
+    got = torch.zeros_like(rows, dtype=torch.bool).scatter_(1, idx.reshape(rows.shape[0], -1).long(), True)
+    want_idx = opress.topk_lowest_index(rows, n)
+    want = torch.zeros_like(got).scatter_(1, want_idx, True)
+    kth = rows.gather(1, want_idx).min(dim=1, keepdim=True).values
+    diff = got ^ want
+    undecided = (rows - kth).abs() <= rel * kth.abs()
+    assert not bool((diff & ~undecided).any()), "kept sets differ at positions whose scores are not near the threshold"
+    assert bool((got.sum(1) == n).all())
+    return int(diff.sum())
+
+
 def test_config1_knorm_full(dev):
     case = synth.knorm_case(seed=0)                              # CPU draw: bit-identical inputs on both sides
     S, ratio = 1024, 0.5
@@ -91,7 +109,18 @@ def test_config2_snapkv_full(dev):
     # softmax mass: unpooled scores would sum to <= W*G per row; pooling keeps the sum within it
     body = res.scores[..., :S - W]
     assert bool((body >= 0).all()) and float(body.sum(-1).max()) <= W * (Hq // Hkv) * 1.001
-    # oracle on a sample of layers and sequences
+    # every column against the oracle's scoring evaluated in fp32 on the device, layer by layer
+    n_tie = 0
+    for layer in range(L):
+        kd = dense_from_pool(before[0, layer:layer + 1], tables, S)[0]                     # [B, Hkv, S, D]
+        ref = opress.snapkv_score(case.queries[layer], kd, W, ksz, True, "sum")             # [B, Hkv, S] fp32
+        got = res.scores[layer]
+        torch.testing.assert_close(got[..., :S - W], ref[..., :S - W], rtol=1e-3, atol=1e-3 * float(ref[..., :S - W].mean()))
+        ref_full = ref.clone()
+        ref_full[..., S - W:] = got[..., S - W:]
+        n_tie += check_selection_against_scores(res.indices[layer], ref_full, n)
+    assert n_tie <= 1e-4 * L * B * Hkv * n, n_tie        # kept positions that fp32 scoring does not decide
+    # CPU oracle on a sample of layers and sequences
     for layer, b in ((0, 0), (17, 3), (35, 7)):
         k = dense_from_pool(before[0, layer:layer + 1], tables[b:b + 1], S)[0].cpu()
         ref = opress.snapkv_score(case.queries[layer, b:b + 1].cpu(), k, W, ksz, True, "sum")
@@ -135,6 +164,15 @@ def test_config3_ccm_full(dev):
         ref = occm.linear_decouple_forward([(kd[:2].cpu(), vd[:2].cpu())], [img, txt], sd, cf, 1)
         assert_mlp_close(ok[:2].cpu(), ref[0][0], torch.float16)
         assert_mlp_close(ov[:2].cpu(), ref[0][1], torch.float16)
+    # every column of every layer against the oracle's forward evaluated in fp32 on the device
+    sd_dev = {k: v.detach().float() for k, v in mod.state_dict().items()}
+    for layer in range(L):
+        kd = dense_from_pool(before[0, layer:layer + 1], tables, S)[0]
+        vd = dense_from_pool(before[1, layer:layer + 1], tables, S)[0]
+        lsd = {f"{k.split('.')[0]}.0.{k.split('.', 2)[2]}": v for k, v in sd_dev.items() if k.split(".")[1] == str(layer)}
+        (rk, rv), = occm.linear_decouple_forward([(kd, vd)], [img, txt], lsd, cf, 1)
+        assert_mlp_close(dense_from_pool(pool[0, layer:layer + 1], tables, C)[0], rk, torch.float16)
+        assert_mlp_close(dense_from_pool(pool[1, layer:layer + 1], tables, C)[0], rv, torch.float16)
     # bytes past the compressed length are untouched (third block of every table, tail of the second)
     after_tail = dense_from_pool(pool[0], tables, S)[:, :, :, C:]
     assert torch.equal(after_tail, dense_from_pool(before[0], tables, S)[:, :, :, C:])
@@ -186,6 +224,13 @@ def test_config4_decode_full(dev):
         ref = oattn.decode_attention(q[T - 1, layer, sample].cpu(), pool1[0, layer].cpu(), pool1[1, layer].cpu(), len_c,
                                      tab_c, 128 ** -0.5)
         torch.testing.assert_close(out1[T - 1, layer, sample].cpu().float(), ref.float(), atol=2e-2, rtol=0)
+    # every sequence at three steps of three layers against the oracle evaluated in fp32 on the device
+    for t in (0, 63, T - 1):
+        len_t = lens0 + (t + 1)
+        for layer in (0, 17, 31):
+            ref = oattn.decode_attention(q[t, layer], pool1[0, layer], pool1[1, layer], len_t, tables, 128 ** -0.5)
+            err = float((out1[t, layer].float() - ref.float()).abs().max())
+            assert err <= 2e-2, (t, layer, err)
     # and the first step
     len_c0 = torch.tensor([case.seq_lens[b] + 1 for b in sample], dtype=torch.int32)
     ref0 = oattn.decode_attention(q[0, 3, sample].cpu(), pool1[0, 3].cpu(), pool1[1, 3].cpu(), len_c0, tab_c, 128 ** -0.5)
@@ -230,6 +275,16 @@ def test_config5_hybrid_end_to_end(dev):
         assert_mlp_close(got_k, ref[0][0], torch.bfloat16)
         assert_mlp_close(got_v, ref[0][1], torch.bfloat16)
         assert torch.equal(got_k[:, :, 3276:], kd[:, :, 16380:])            # remainder tokens copied through
+    # every column of every layer against the oracle's forward evaluated in fp32 on the device
+    sd_dev = {k: v.detach().float() for k, v in mod.state_dict().items()}
+    for layer in range(L):
+        kd = dense_from_pool(before[0, layer:layer + 1], tt, S)[0]
+        vd = dense_from_pool(before[1, layer:layer + 1], tt, S)[0]
+        lsd = {f"{k.split('.')[0]}.0.{k.split('.', 2)[2]}": v for k, v in sd_dev.items() if k.split(".")[1] == str(layer)}
+        (rk, rv), = occm.hybrid_forward([(kd, vd)], [0, S], lsd, cf, 1)
+        assert_mlp_close(dense_from_pool(runner.kv_cache[0, layer:layer + 1], tt, C)[0], rk, torch.bfloat16)
+        assert_mlp_close(dense_from_pool(runner.kv_cache[1, layer:layer + 1], tt, C)[0], rv, torch.bfloat16)
+        del kd, vd, rk, rv
     # 64 decode steps over the compressed caches: freed blocks are handed out again as sequences grow
     for s in seqs:
         for _ in range(T):
@@ -246,6 +301,13 @@ def test_config5_hybrid_end_to_end(dev):
     out = dg.replay()
     torch.cuda.synchronize()
     assert lens.tolist() == [C + T] * B
+    for t in (0, T - 1):
+        len_t = torch.full((B,), C + t + 1, dtype=torch.int32, device=dev)
+        for layer in (0, 13, 27):
+            ref = oattn.decode_attention(q[t, layer], runner.kv_cache[0, layer], runner.kv_cache[1, layer], len_t,
+                                         tables, 128 ** -0.5)
+            err = float((out[t, layer].float() - ref.float()).abs().max())
+            assert err <= 2e-2, (t, layer, err)
     tab_c = tables[:2].cpu()
     for layer in (0, 27):
         ref = oattn.decode_attention(q[T - 1, layer, :2].cpu(), runner.kv_cache[0, layer].cpu(),

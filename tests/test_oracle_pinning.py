@@ -623,3 +623,100 @@ def test_think_and_simlayer_oracle_by_loops_and_hand():
     total = op.simlayer_lazy_score(k, ql, 0, S - n_last)
     assert abs(total - sum(acc)) <= 1e-12 and total < 1.0
     assert op.simlayer_keep_positions(20, 4, 6, 1).tolist() == [0, 1, 2, 3, 15, 16, 17, 18, 19]
+
+
+# ---- the per-sequence driver ---------------------------------------------------------------------------
+def test_compress_batch_bookkeeping_by_hand():
+    """``pipeline.compress_batch`` on a hand-worked pool: block size 4, two sequences (10 and 5 tokens) on shuffled
+    pages, a compressor that keeps every second token and negates K.  Lengths, released blocks, ratio, written
+    slots and every untouched slot are stated here by hand, not recomputed with the oracle's formulas."""
+    from oracle import pipeline as opipe
+    L, NB, bs, H, D = 2, 9, 4, 2, 3
+    pool = torch.arange(2 * L * NB * bs * H * D, dtype=torch.float32).view(2, L, NB, bs, H, D) + 1.0
+    before = pool.clone()
+    tables, lens = [[7, 1, 4], [3, 8]], [10, 5]
+
+    def every_second(hf, i, n):
+        return [((-k[:, :, ::2]).contiguous(), v[:, :, ::2].contiguous()) for k, v in hf]
+
+    clens, to_free, ratio = opipe.compress_batch(pool, tables, lens, every_second)
+    assert clens == {0: 5, 1: 3}                        # ceil(10/2), ceil(5/2)
+    assert to_free == {0: [4], 1: [8]}                  # 5 tokens need 2 of 3 pages, 3 tokens need 1 of 2
+    assert abs(ratio - 15 / 8) < 1e-12                  # (10 + 5) tokens in, (5 + 3) out, same heads and planes
+    token = lambda seq, s: (tables[seq][s // bs], s % bs)
+    for seq, (n, c) in enumerate(((10, 5), (5, 3))):
+        for l in range(L):
+            for j in range(c):                          # kept token j is source token 2j
+                sb, ss = token(seq, 2 * j)
+                db, ds = token(seq, j)
+                assert torch.equal(pool[0, l, db, ds], -before[0, l, sb, ss])
+                assert torch.equal(pool[1, l, db, ds], before[1, l, sb, ss])
+            for s in range(c, len(tables[seq]) * bs):   # every later slot of the sequence's pages is untouched
+                b_, s_ = token(seq, s)
+                assert torch.equal(pool[:, l, b_, s_], before[:, l, b_, s_])
+    others = [b for b in range(NB) if b not in (7, 1, 4, 3, 8)]
+    assert torch.equal(pool[:, :, others], before[:, :, others])
+
+
+def test_compress_batch_releases_second_page_when_one_suffices():
+    from oracle import pipeline as opipe
+    pool = torch.zeros(2, 1, 4, 4, 1, 2)
+    keep3 = lambda hf, i, n: [(k[:, :, :3].contiguous(), v[:, :, :3].contiguous()) for k, v in hf]
+    clens, to_free, ratio = opipe.compress_batch(pool, [[2, 0]], [5], keep3)
+    assert clens == {0: 3} and to_free == {0: [0]} and abs(ratio - 5 / 3) < 1e-12
+    # nothing to release when the compressed length still needs every page
+    keep5 = lambda hf, i, n: hf
+    clens, to_free, ratio = opipe.compress_batch(pool, [[2, 0]], [5], keep5)
+    assert clens == {0: 5} and to_free == {} and ratio == 1.0
+
+
+# ---- how far two correct fp32-accumulating MLP evaluations can differ -----------------------------------
+def test_mlp_tolerance_calibration():
+    """The MLP parity tolerance of the GPU tests, measured: ``oracle.ccm.mlp3`` against the same three Linears
+    (storage-dtype operands, fp32 accumulation, rounding after every Linear) summed in other orders, in
+    comparisons of 1000 rows as the GPU tests make them.  fp16: no element beyond ``1e-3 * max|ref| + 2 ulp``.
+    bf16: a few per 10^7 (a hidden activation that rounds to the neighbouring bf16 value), each within 5e-3 of
+    max|ref|.  Measured over 15 M elements per case: 5, 5 and 2 outliers for cf 1, 2, 5 in bf16 (worst 4.2e-3),
+    none in fp16 (worst 5.6e-4).  ``assert_mlp_close`` allows 1 + 2 per million in bf16 and none in fp16."""
+    import torch.nn.functional as F
+    from test_gpu_ccm import mlp_error_stats
+
+    def mlp3_order(x, sd, order):
+        dt = x.dtype
+
+        def lin(inp, i):
+            w = sd[f"compress_tk.0.{i}.weight"].to(dt).float()
+            b = sd[f"compress_tk.0.{i}.bias"].to(dt).float()
+            a, K = inp.float(), inp.shape[-1]
+            if order == "halves":
+                y = (a[..., :K // 2] @ w[:, :K // 2].T) + (a[..., K // 2:] @ w[:, K // 2:].T) + b
+            elif order == "reversed":
+                y = a.flip(-1) @ w.flip(-1).T + b
+            elif order == "chunks16":                   # the k-step of the matrix instruction
+                y = b.expand(*a.shape[:-1], w.shape[0]).clone()
+                for k0 in range(0, K, 16):
+                    y = y + a[..., k0:k0 + 16] @ w[:, k0:k0 + 16].T
+            else:                                       # exact sums, one rounding to fp32
+                y = (a.double() @ w.double().T + b.double()).float()
+            return y.to(dt)
+
+        h = F.relu(lin(x, 0))
+        h = F.relu(lin(h, 3))
+        return lin(h, 6)
+
+    for dtype, cf, chunks in ((torch.float16, 2, 6), (torch.float16, 1, 6), (torch.bfloat16, 1, 12), (torch.bfloat16, 5, 6)):
+        sd = occm.reference_init_state_dict("linear_decouple", 1, 128, cf, seed=7)
+        total = outliers = 0
+        worst_rel = worst_err = 0.0
+        for chunk in range(chunks):
+            x = torch.randn(1000, 128 * cf, generator=torch.Generator().manual_seed(chunk)).to(dtype)
+            ref = occm.mlp3(x, sd, "compress_tk", 0)
+            for order in ("halves", "reversed", "chunks16", "fp64"):
+                rel, n_out, worst, n = mlp_error_stats(mlp3_order(x, sd, order), ref, dtype)
+                total, outliers = total + n, outliers + n_out
+                worst_rel, worst_err = max(worst_rel, rel), max(worst_err, worst)
+        assert worst_rel < 2e-4 and worst_err < 5e-3, (dtype, cf, worst_rel, worst_err)
+        if dtype == torch.float16:
+            assert outliers == 0, (cf, outliers)
+        else:
+            assert outliers <= 1 + total // 500_000, (cf, outliers, total)
