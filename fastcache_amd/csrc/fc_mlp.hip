@@ -40,7 +40,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 #define ML_WBYTES (128 * ML_ROWB)   // one 128 x 128 weight block in LDS
 #define ML_TBLTOT 768               // block-table entries cached per workgroup and view, divided among its columns
 #define ML_XS 2048                  // per-wavefront LDS bytes for re-laying token rows: 32 rows x 64 bytes
-#define ML_LDS (4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + ML_WAVES * ML_XS)
+#define ML_LDS (4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + ML_WAVES * ML_XS + ML_WAVES * 4)
 // Nothing is scheduled across this point.  Without it the compiler, short of registers, sinks every
 // prefetch (weight fragments from LDS, token rows from memory) to just before its use and the
 // multiplications wait out the full latency each time.
@@ -97,12 +97,18 @@ __device__ __forceinline__ void ml_wave_sync() {
 // 2 = paged view read through global memory.
 // W1R: all of W1 fits the two LDS chunk buffers (cf <= 2) and is loaded once; otherwise W1 streams
 // through them one chunk per stage, which costs a workgroup barrier per chunk.
-template <int DTYPE, int SRC_T, int DST_T, bool W1R>
+// RAG: every sequence has its own segment: seg_start_v / seg_len_v / dst_start_v [batch] in device memory; c_rows is
+// then the largest row count any sequence can have (it bounds the loops), and a sequence whose segment gives fewer
+// than min_rows rows is left to the copy kernel below.
+template <int DTYPE, int SRC_T, int DST_T, bool W1R, bool RAG>
 __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView src, KvView dst, const char* __restrict__ w1,
                                                             const char* __restrict__ b1, const char* __restrict__ w2,
                                                             const char* __restrict__ b2, const char* __restrict__ w3,
                                                             const char* __restrict__ b3, int cf, int seg_start,
-                                                            int c_rows, int dst_start, int wpc, int ncols, int ncg) {
+                                                            int c_rows, int dst_start, int wpc, int ncols, int ncg,
+                                                            const int* __restrict__ seg_start_v,
+                                                            const int* __restrict__ seg_len_v,
+                                                            const int* __restrict__ dst_start_v, int min_rows) {
   extern __shared__ __align__(16) char lds[];
   char* w1buf = lds;                       // 2 x ML_WBYTES
   char* w2buf = lds + 2 * ML_WBYTES;       // permuted
@@ -110,6 +116,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   float* bias = reinterpret_cast<float*>(lds + 4 * ML_WBYTES);  // [3][128] fp32
   int* tbls = reinterpret_cast<int*>(lds + 4 * ML_WBYTES + 3 * 128 * 4);  // [2 views][columns of the workgroup][tcap]
   char* xsw = lds + 4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + (threadIdx.x >> 6) * ML_XS;
+  int* wave_rows = reinterpret_cast<int*>(lds + 4 * ML_WBYTES + 3 * 128 * 4 + 2 * ML_TBLTOT * 4 + ML_WAVES * ML_XS);
 
   const int l = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -128,8 +135,11 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   const int tcap = ML_TBLTOT / cols_per_wg;
   int* stbl = tbls + (wave / wpc) * tcap;
   int* dtbl = stbl + ML_TBLTOT;
-  const int s_last = seg_start + c_rows * cf - 1, d_last = dst_start + c_rows - 1;
+  // this wavefront's column: first source token, rows, first destination token (the launch's, or the sequence's own)
+  int ss = seg_start, cr = c_rows, ds = dst_start;
   auto fill_tables = [&]() {
+    // a column without rows still loads (clamped) rows of its first cf tokens: its table covers them
+    const int s_last = min(ss + max(cr, 1) * cf, src.max_seq_len) - 1, d_last = ds + cr - 1;
     // also for a wavefront whose column is past the last one (b = 0): its loads are unconditional and need valid addresses
     if (SRC_T == 1)
       for (int i = sub * 64 + lane; i <= (s_last >> src.block_shift); i += 64 * wpc)
@@ -195,8 +205,8 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
   };
 
   const int rows_per_iter = ML_ROWS * wpc;
-  const int n_iter = (c_rows + rows_per_iter - 1) / rows_per_iter;
-  const int q_total = n_iter * cf;      // W1 chunk q = (iteration q / cf, token kc = q % cf) sits in buffer q & 1
+  int n_iter = (c_rows + rows_per_iter - 1) / rows_per_iter;
+  int q_total = n_iter * cf;      // W1 chunk q = (iteration q / cf, token kc = q % cf) sits in buffer q & 1
   const char* sbase = nullptr;   // this lane's piece of token 0 of the column's head, per column group
   char* dbase = nullptr;
 
@@ -210,8 +220,13 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
     // computed from them is never stored.
 #pragma unroll
     for (int rh = 0; rh < 2; ++rh) {
-      const int r = min(row0 + rh * 16 + lq, c_rows - 1);
-      long long off = src_off(seg_start + cf * r + kc);
+      int r = min(row0 + rh * 16 + lq, cr - 1);
+      int tok = ss + cf * r + kc;
+      if constexpr (RAG) {   // a column with no rows, or fewer than the launch's bound, reads some valid token
+        r = max(r, 0);
+        tok = min(ss + cf * r + kc, src.max_seq_len - 1);
+      }
+      long long off = src_off(tok);
       off = off < 0 ? 0 : off;
 #pragma unroll
       for (int c4 = 0; c4 < 4; ++c4) xf[c4 * 2 + rh] = *reinterpret_cast<const uint4*>(sbase + off * 2 + c4 * 64);
@@ -318,7 +333,7 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
       for (int rh = 0; rh < 2; ++rh) {
         const int r = row0 + rh * 16 + lq;
         long long off = -1;
-        if (col_ok && r < c_rows) off = dst_off(dst_start + r);
+        if (col_ok && r < cr) off = dst_off(ds + r);
         rowp[rh] = off >= 0 ? dbase + off * 2 : nullptr;
       }
       // (a half-wave writes one 8-byte half per row, so rows that share a piece position in a bank window keep
@@ -364,12 +379,30 @@ __global__ __launch_bounds__(ML_THREADS, ML_WAVES / 4) void mlp_kernel(KvView sr
     h = col_ok ? col - (col / H) * H : 0;
     sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + lp * 16;
     dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2 + lp * 16;
+    if constexpr (RAG) {
+      // The sequence's own segment.  Numbers from device memory are cut to what the host validated: the views'
+      // max_seq_len (which their block tables cover) and the launch's row bound.
+      ss = min(max(__builtin_amdgcn_readfirstlane(seg_start_v[b]), 0), src.max_seq_len);
+      const int sl = min(max(__builtin_amdgcn_readfirstlane(seg_len_v[b]), 0), src.max_seq_len - ss);
+      ds = min(max(__builtin_amdgcn_readfirstlane(dst_start_v[b]), 0), dst.max_seq_len);
+      cr = sl / cf;
+      if (cr < min_rows || !col_ok) cr = 0;
+      cr = min(min(cr, c_rows), dst.max_seq_len - ds);
+      if (lane == 0) wave_rows[wave] = cr;
+    }
     fill_tables();
     if (!W1R) {
       w1_load(0);
       w1_store(0);
     }
     __syncthreads();   // block tables, biases and the first weights are in LDS
+    if constexpr (RAG) {   // the workgroup walks as many iterations as its longest column needs
+      int most = 0;
+#pragma unroll
+      for (int w = 0; w < ML_WAVES; ++w) most = max(most, wave_rows[w]);
+      n_iter = (most + rows_per_iter - 1) / rows_per_iter;
+      q_total = n_iter * cf;
+    }
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) ml_bias_init(acc[mb], bias, mb * 32, lhalf);
     x_load(xa, 0);
@@ -395,12 +428,44 @@ static int ml_compute_units() {
   return cus[dev];
 }
 
+// What the MLP leaves of a ragged segment: the seg_len % cf remainder tokens, or the whole segment of a sequence
+// too short to compress, copied to their place behind the compressed rows.  One workgroup per (head, sequence,
+// layer); 16 tokens per pass, all loaded before any is stored (destination token <= source token, ascending).
+__global__ __launch_bounds__(256) void mlp_tail_copy_kernel(KvView src, KvView dst, int cf, int min_rows, int c_max,
+                                                            const int* __restrict__ seg_start_v,
+                                                            const int* __restrict__ seg_len_v,
+                                                            const int* __restrict__ dst_start_v, int same_place) {
+  const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
+  const int ss = min(max(seg_start_v[b], 0), src.max_seq_len);
+  const int sl = min(max(seg_len_v[b], 0), src.max_seq_len - ss);
+  const int ds = min(max(dst_start_v[b], 0), dst.max_seq_len);
+  int c = sl / cf;
+  if (c < min_rows) c = 0;
+  c = min(min(c, c_max), dst.max_seq_len - ds);
+  const int s0 = ss + c * cf, d0 = ds + c;
+  const int cnt = min(sl - c * cf, dst.max_seq_len - d0);
+  if (cnt <= 0 || (same_place && s0 == d0)) return;
+  const int sub = threadIdx.x & 15, tr = threadIdx.x >> 4;
+  const char* sb = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * 2 + sub * 16;
+  char* db = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * 2 + sub * 16;
+  for (int i0 = 0; i0 < cnt; i0 += 16) {
+    const int i = i0 + tr;
+    uint4 row = make_uint4(0, 0, 0, 0);
+    long long so = -1, dof = -1;
+    if (i < cnt) {
+      so = fc_token_offset(src, b, s0 + i);
+      dof = fc_token_offset(dst, b, d0 + i);
+    }
+    if (so >= 0) row = *reinterpret_cast<const uint4*>(sb + so * 2);
+    __syncthreads();
+    if (so >= 0 && dof >= 0) *reinterpret_cast<uint4*>(db + dof * 2) = row;
+  }
+}
+
 extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int32_t seg_start, int32_t count,
                               int32_t dst_start, void* stream);
 
-extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int32_t cf,
-                          int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream) {
-  const char* who = "fc_ccm_mlp";
+static int ml_check(const char* who, const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int cf) {
   int rc;
   if ((rc = fc_check_view(src, who)) || (rc = fc_check_view(dst, who))) return rc;
   FC_REQUIRE(src->dtype == dst->dtype && src->num_layers == dst->num_layers && src->batch == dst->batch &&
@@ -409,6 +474,86 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
   FC_REQUIRE(src->dtype == FC_F16 || src->dtype == FC_BF16, FC_EUNSUPPORTED, "%s: fp16/bf16 caches only", who);
   FC_REQUIRE(w && w->w1 && w->b1 && w->w2 && w->b2 && w->w3 && w->b3, FC_EINVAL, "%s: null weights", who);
   FC_REQUIRE(cf >= 1 && cf <= 64, FC_EINVAL, "%s: compression factor %d out of range", who, cf);
+  return FC_OK;
+}
+
+// The MLP launch for c > 0 rows per column: c rows for every sequence from (seg_start, dst_start), or, with the
+// three arrays, every sequence's own segment with at most c rows.
+static int ml_launch(const char* who, const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int cf,
+                     int seg_start, int c, int dst_start, const int32_t* seg_start_v, const int32_t* seg_len_v,
+                     const int32_t* dst_start_v, int min_rows, hipStream_t st) {
+  const bool rag = seg_len_v != nullptr;
+  const int ncols = src->batch * src->num_kv_heads;
+  int wpc = 1;
+  while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && ML_ROWS * wpc * 2 <= c) wpc *= 2;
+  const int cols_per_wg = ML_WAVES / wpc;
+  // One workgroup occupies a compute unit (its LDS), and loading the weights costs it a few microseconds.
+  // When a column group is short work, let each workgroup walk several groups of its layer; pick the number
+  // per workgroup that minimises rounds * (groups * time per group + start-up) in a coarse model.
+  const int ncg = (ncols + cols_per_wg - 1) / cols_per_wg;
+  int gx = ncg;
+  {
+    const int ncu = ml_compute_units();
+    const int n_iter = (c + ML_ROWS * wpc - 1) / (ML_ROWS * wpc);
+    const double t_group = 1.5 * n_iter * (cf + 2), t_start = 4.0;   // microseconds, roughly
+    double best = -1.0;
+    for (int per = 1; cf <= 2 && ncu > 0 && per <= ncg && per <= 64; ++per) {
+      const int g = (ncg + per - 1) / per;
+      const long long rounds = ((long long)g * src->num_layers + ncu - 1) / ncu;
+      const double cost = (double)rounds * (((ncg + g - 1) / g) * t_group + t_start);
+      if (best < 0 || cost < best) {
+        best = cost;
+        gx = g;
+      }
+    }
+  }
+  dim3 grid(gx, src->num_layers);
+  const size_t lds = ML_LDS;
+  KvView s = fc_make_view(src), d = fc_make_view(dst);
+  auto table_mode = [&](const KvView& v, int last_token) {
+    if (!v.block_tables) return 0;
+    return (v.block_shift >= 0 && (last_token >> v.block_shift) < ML_TBLTOT / cols_per_wg) ? 1 : 2;
+  };
+  // ragged segments may end anywhere inside the views
+  const int sm = table_mode(s, rag ? src->max_seq_len - 1 : seg_start + c * cf - 1);
+  const int dm = table_mode(d, rag ? dst->max_seq_len - 1 : dst_start + c - 1);
+  // dense/dense, LDS-cached tables, or the general path through global tables (which also serves dense views)
+  int mode = (sm == 0 && dm == 0) ? 0 : (sm == 1 && dm == 1) ? 1 : (sm == 0 && dm == 1) ? 2 : (sm == 1 && dm == 0) ? 3 : 4;
+  if (rag && mode != 1) mode = 4;
+#define ML_LAUNCH(DT, ST, DTT, WR, RG)                                                                                 \
+  do {                                                                                                             \
+    FC_ALLOW_LDS((mlp_kernel<DT, ST, DTT, WR, RG>), (int)lds);                                                    \
+    hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT, WR, RG>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1, \
+                       (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,             \
+                       (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols, ncg, seg_start_v, seg_len_v,   \
+                       dst_start_v, min_rows);                                                                     \
+  } while (0)
+#define ML_DISPATCH(DT, WR)                                                         \
+  if (rag) {                                                                        \
+    if (mode == 1) ML_LAUNCH(DT, 1, 1, WR, true); else ML_LAUNCH(DT, 2, 2, WR, true); \
+  } else switch (mode) {                                                            \
+    case 0: ML_LAUNCH(DT, 0, 0, WR, false); break;                                  \
+    case 1: ML_LAUNCH(DT, 1, 1, WR, false); break;                                  \
+    case 2: ML_LAUNCH(DT, 0, 1, WR, false); break;                                  \
+    case 3: ML_LAUNCH(DT, 1, 0, WR, false); break;                                  \
+    default: ML_LAUNCH(DT, 2, 2, WR, false); break;                                 \
+  }
+  if (src->dtype == FC_BF16) {
+    if (cf <= 2) { ML_DISPATCH(FC_BF16, true) } else { ML_DISPATCH(FC_BF16, false) }
+  } else {
+    if (cf <= 2) { ML_DISPATCH(FC_F16, true) } else { ML_DISPATCH(FC_F16, false) }
+  }
+#undef ML_DISPATCH
+#undef ML_LAUNCH
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int32_t cf,
+                          int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream) {
+  const char* who = "fc_ccm_mlp";
+  int rc = ml_check(who, src, dst, w, cf);
+  if (rc) return rc;
   FC_REQUIRE(seg_start >= 0 && seg_len >= 0 && dst_start >= 0, FC_EINVAL, "%s: negative range", who);
   FC_REQUIRE((int64_t)seg_start + seg_len <= src->max_seq_len, FC_EINVAL,
              "%s: segment [%d, %d) exceeds the source view's max_seq_len %d", who, seg_start, seg_start + seg_len,
@@ -418,66 +563,35 @@ extern "C" int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc
   FC_REQUIRE((int64_t)dst_start + c + rem <= dst->max_seq_len, FC_EINVAL,
              "%s: output [%d, %d) exceeds the destination view's max_seq_len %d", who, dst_start,
              dst_start + c + rem, dst->max_seq_len);
-  hipStream_t st = (hipStream_t)stream;
-  if (c > 0) {
-    const int ncols = src->batch * src->num_kv_heads;
-    int wpc = 1;
-    while (wpc < ML_WAVES && (int64_t)ncols * wpc / ML_WAVES * src->num_layers < 1024 && ML_ROWS * wpc * 2 <= c) wpc *= 2;
-    const int cols_per_wg = ML_WAVES / wpc;
-    // One workgroup occupies a compute unit (its LDS), and loading the weights costs it a few microseconds.
-    // When a column group is short work, let each workgroup walk several groups of its layer; pick the number
-    // per workgroup that minimises rounds * (groups * time per group + start-up) in a coarse model.
-    const int ncg = (ncols + cols_per_wg - 1) / cols_per_wg;
-    int gx = ncg;
-    {
-      const int ncu = ml_compute_units();
-      const int n_iter = (c + ML_ROWS * wpc - 1) / (ML_ROWS * wpc);
-      const double t_group = 1.5 * n_iter * (cf + 2), t_start = 4.0;   // microseconds, roughly
-      double best = -1.0;
-      for (int per = 1; cf <= 2 && ncu > 0 && per <= ncg && per <= 64; ++per) {
-        const int g = (ncg + per - 1) / per;
-        const long long rounds = ((long long)g * src->num_layers + ncu - 1) / ncu;
-        const double cost = (double)rounds * (((ncg + g - 1) / g) * t_group + t_start);
-        if (best < 0 || cost < best) {
-          best = cost;
-          gx = g;
-        }
-      }
-    }
-    dim3 grid(gx, src->num_layers);
-    const size_t lds = ML_LDS;
-    KvView s = fc_make_view(src), d = fc_make_view(dst);
-    auto table_mode = [&](const KvView& v, int last_token) {
-      if (!v.block_tables) return 0;
-      return (v.block_shift >= 0 && (last_token >> v.block_shift) < ML_TBLTOT / cols_per_wg) ? 1 : 2;
-    };
-    const int sm = table_mode(s, seg_start + c * cf - 1), dm = table_mode(d, dst_start + c - 1);
-    // dense/dense, LDS-cached tables, or the general path through global tables
-    const int mode = (sm == 0 && dm == 0) ? 0 : (sm == 1 && dm == 1) ? 1 : (sm == 0 && dm == 1) ? 2 : (sm == 1 && dm == 0) ? 3 : 4;
-#define ML_LAUNCH(DT, ST, DTT, WR)                                                                                     \
-  do {                                                                                                             \
-    FC_ALLOW_LDS((mlp_kernel<DT, ST, DTT, WR>), (int)lds);                                                    \
-    hipLaunchKernelGGL((mlp_kernel<DT, ST, DTT, WR>), grid, dim3(ML_THREADS), lds, st, s, d, (const char*)w->w1,   \
-                       (const char*)w->b1, (const char*)w->w2, (const char*)w->b2, (const char*)w->w3,             \
-                       (const char*)w->b3, cf, seg_start, c, dst_start, wpc, ncols, ncg);                          \
-  } while (0)
-#define ML_DISPATCH(DT, WR)                      \
-  switch (mode) {                                \
-    case 0: ML_LAUNCH(DT, 0, 0, WR); break;      \
-    case 1: ML_LAUNCH(DT, 1, 1, WR); break;      \
-    case 2: ML_LAUNCH(DT, 0, 1, WR); break;      \
-    case 3: ML_LAUNCH(DT, 1, 0, WR); break;      \
-    default: ML_LAUNCH(DT, 2, 2, WR); break;     \
-  }
-    if (src->dtype == FC_BF16) {
-      if (cf <= 2) { ML_DISPATCH(FC_BF16, true) } else { ML_DISPATCH(FC_BF16, false) }
-    } else {
-      if (cf <= 2) { ML_DISPATCH(FC_F16, true) } else { ML_DISPATCH(FC_F16, false) }
-    }
-#undef ML_DISPATCH
-#undef ML_LAUNCH
-    FC_CHECK_LAUNCH(who);
-  }
+  if (c > 0 && (rc = ml_launch(who, src, dst, w, cf, seg_start, c, dst_start, nullptr, nullptr, nullptr, 0,
+                               (hipStream_t)stream)))
+    return rc;
   if (rem > 0) return fc_copy_tokens(src, dst, seg_start + c * cf, rem, dst_start + c, stream);
+  return FC_OK;
+}
+
+extern "C" int fc_ccm_mlp_ragged(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int32_t cf,
+                                 const int32_t* seg_start, const int32_t* seg_len, const int32_t* dst_start,
+                                 int32_t max_seg_len, int32_t min_rows, void* stream) {
+  const char* who = "fc_ccm_mlp_ragged";
+  int rc = ml_check(who, src, dst, w, cf);
+  if (rc) return rc;
+  FC_REQUIRE(seg_start && seg_len && dst_start, FC_EINVAL, "%s: null segment arrays", who);
+  FC_REQUIRE(max_seg_len >= 0 && max_seg_len <= src->max_seq_len, FC_EINVAL,
+             "%s: max_seg_len %d outside [0, max_seq_len %d]", who, max_seg_len, src->max_seq_len);
+  FC_REQUIRE(min_rows >= 0, FC_EINVAL, "%s: negative min_rows", who);
+  FC_REQUIRE(src->num_kv_heads <= 65535, FC_EUNSUPPORTED, "%s: too many heads", who);
+  if (max_seg_len == 0) return FC_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const int c = max_seg_len / cf;
+  if (c > 0 && c >= min_rows &&
+      (rc = ml_launch(who, src, dst, w, cf, 0, c, 0, seg_start, seg_len, dst_start, min_rows, st)))
+    return rc;
+  // remainders and pass-through segments; nothing to move when a pass-through segment already lies at its place
+  const int same = src->base == dst->base && src->block_tables == dst->block_tables &&
+                   src->stride_layer == dst->stride_layer && src->stride_batch == dst->stride_batch;
+  hipLaunchKernelGGL(mlp_tail_copy_kernel, dim3(src->num_kv_heads, src->batch, src->num_layers), dim3(256), 0, st,
+                     fc_make_view(src), fc_make_view(dst), cf, min_rows, c, seg_start, seg_len, dst_start, same);
+  FC_CHECK_LAUNCH(who);
   return FC_OK;
 }

@@ -6,8 +6,9 @@
 The model forward is not part of this build; a ``PagedKVRunner`` owns the pool and offers the same
 method names, bookkeeping dictionaries and return values, so an engine loop written against the
 reference runner drives it unchanged.  Compressors that expose ``paged_forward`` (every compressor
-of this package) are run in place on the pages for all sequences of equal length at once; any
-other callable goes through extract -> call -> write back, with the copies done by HIP kernels.
+of this package) are run in place on the pages for all sequences of a batch at once, whatever their
+lengths; any other callable goes through extract -> call -> write back, with the copies done by HIP
+kernels.
 """
 from __future__ import annotations
 
@@ -102,17 +103,18 @@ class PagedKVRunner:
         orig = after = 0
         result: Dict[int, int] = {}
         if hasattr(comp, "paged_forward"):
-            groups: Dict[int, List[Sequence]] = {}
-            for s in seqs:
-                groups.setdefault(len(s), []).append(s)
-            for S, group in groups.items():
-                tt, ll = self._table_and_lens([s.block_table for s in group], [S] * len(group))
-                it_len = [image_len, max(1, S - image_len)]
-                C = comp.paged_forward(self.kv_cache, tt, ll, S, it_len)
-                for s in group:
-                    result[s.seq_id] = C
-                orig += 2 * L * H * D * S * len(group)
-                after += 2 * L * H * D * C * len(group)
+            # every sequence of the batch in the same launches, whatever their lengths: the kernels take each
+            # sequence's length (and, for the MLPs, its segments) from device arrays
+            lens = [len(s) for s in seqs]
+            S = max(lens)
+            tt, ll = self._table_and_lens([s.block_table for s in seqs], lens)
+            it_len = [image_len, max(1, S - image_len)]
+            C = comp.paged_forward(self.kv_cache, tt, ll, S, it_len, host_lens=lens)
+            per_seq = list(C) if isinstance(C, (list, tuple)) else [C] * len(seqs)
+            for s, n, c in zip(seqs, lens, per_seq):
+                result[s.seq_id] = c
+                orig += 2 * L * H * D * n
+                after += 2 * L * H * D * c
         else:
             for s in seqs:
                 S = len(s)

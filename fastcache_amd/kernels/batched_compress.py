@@ -112,16 +112,32 @@ class BatchedGEMMCompressor(nn.Module):
     @torch.no_grad()
     def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
                       seq_len: int, it_len: Sequence[int], layers: Optional[Tuple[int, int]] = None,
-                      out: Optional[torch.Tensor] = None) -> int:
+                      out: Optional[torch.Tensor] = None, host_lens: Optional[Sequence[int]] = None):
         """On a paged pool ``[2, L, blocks, block_size, Hkv, D]`` for sequences that all hold ``seq_len``
         tokens: in place, or for the layers ``layers=(l0, l1)`` only, or into ``out [2, L, B, Hkv, C, D]``
-        leaving the pages untouched; returns the compressed length."""
+        leaving the pages untouched; returns the compressed length.  Sequences of different lengths:
+        ``host_lens`` (Python ints; ``seq_len`` is their maximum) -> the list of compressed lengths, from the
+        same number of launches."""
         cf = self.compression_factor
         img = min(int(it_len[0]), seq_len) if it_len[0] > 0 else 0
         l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
         dst = 0
         views = [_lib.paged_view(kv_cache[p][l0:l1], block_tables, seq_lens, seq_len) for p in range(2)]
         dviews = views if out is None else [_lib.dense_view(out[p][l0:l1]) for p in range(2)]
+        if host_lens is not None and len(set(host_lens)) > 1:
+            dev = kv_cache.device
+            mk = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)
+            imgs = [min(int(it_len[0]), n) if it_len[0] > 0 else 0 for n in host_lens]
+            dsts = [0] * len(imgs)
+            for starts, counts, seg in (([0] * len(imgs), imgs, "i"), (imgs, [n - i for n, i in zip(host_lens, imgs)], "t")):
+                if max(counts) == 0:
+                    continue
+                st, ct, dt = mk(starts), mk(counts), mk(dsts)
+                for view, dview, kind in ((views[0], dviews[0], "k"), (views[1], dviews[1], "v")):
+                    ops.ccm_mlp_ragged(view, dview, self._weights(seg + kind, kv_cache.dtype, dev, (l0, l1)), cf, st, ct,
+                                       dt, max(counts), self.min_seq_len)
+                dsts = [d + self._seg_len(n) for d, n in zip(dsts, counts)]
+            return dsts
         for s0, n, seg in ((0, img, "i"), (img, seq_len - img, "t")):
             if n == 0:
                 continue

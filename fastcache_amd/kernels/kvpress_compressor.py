@@ -112,10 +112,14 @@ class KVPressCompressor(nn.Module):
     @torch.no_grad()
     def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
                       seq_len: int, it_len=None, layers: Optional[Tuple[int, int]] = None,
-                      out: Optional[torch.Tensor] = None) -> int:
+                      out: Optional[torch.Tensor] = None, host_lens=None):
         """The same selection and gather on a paged pool ``[2, L, blocks, block_size, Hkv, D]`` for
         sequences that all hold ``seq_len`` tokens: in place, or for the layers ``layers=(l0, l1)`` only, or
-        into ``out [2, L, B, Hkv, C, D]`` leaving the pages untouched; returns the kept length."""
+        into ``out [2, L, B, Hkv, C, D]`` leaving the pages untouched; returns the kept length.  Sequences of
+        different lengths: ``host_lens`` (Python ints; ``seq_len`` is their maximum) -> the list of kept
+        lengths, from the same three launches."""
+        if host_lens is not None and len(set(host_lens)) > 1:
+            return self._paged_forward_ragged(kv_cache, block_tables, seq_lens, seq_len, list(host_lens), layers, out)
         S = seq_len
         n = self.get_compressed_length(S)
         dev = kv_cache.device
@@ -142,6 +146,38 @@ class KVPressCompressor(nn.Module):
         else:
             ops.compact(kview, vview, _lib.dense_view(out[0][l0:l1]), _lib.dense_view(out[1][l0:l1]), idx)
         return n
+
+    def _paged_forward_ragged(self, kv_cache, block_tables, seq_lens, max_len, lens, layers, out):
+        """Every sequence keeps ``get_compressed_length(its own length)`` tokens; the index rows are padded to the
+        longest with -1 and the kernels take the kept counts from a device array.  A sequence that is not
+        shortened keeps all its positions (an identity row)."""
+        dev = kv_cache.device
+        l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
+        L, B = l1 - l0, block_tables.shape[0]
+        kview = _lib.paged_view(kv_cache[0][l0:l1], block_tables, seq_lens, max_len)
+        vview = _lib.paged_view(kv_cache[1][l0:l1], block_tables, seq_lens, max_len)
+        kept = [self.paged_compressed_len(n) for n in lens]
+        width = max(kept)
+        n_kept = torch.tensor(kept, dtype=torch.int32, device=dev)
+        if self.method_name == "knorm" and any(k < n for k, n in zip(kept, lens)):
+            score = ops.knorm_mean_score(kview, dev)                                  # [L, B, S], -inf past each length
+            idx = ops.topk_select(score, width, row_lens=seq_lens, n_kept=n_kept).view(L, B, 1, width)
+        else:
+            rows = torch.full((L, B, width), -1, dtype=torch.int32)
+            for b, (n, k) in enumerate(zip(lens, kept)):
+                if k >= n:
+                    rows[:, b, :n] = torch.arange(n, dtype=torch.int32)
+                elif self.method_name == "random":
+                    for l in range(L):
+                        rows[l, b, :k] = torch.randperm(n)[:k].sort().values.to(torch.int32)
+                else:
+                    rows[:, b, :k] = self._static_indices(n, self.get_compressed_length(n), torch.device("cpu"))
+            idx = rows.view(L, B, 1, width).to(dev)
+        if out is None:
+            ops.compact(kview, vview, kview, vview, idx, n_kept=n_kept)
+        else:
+            ops.compact(kview, vview, _lib.dense_view(out[0][l0:l1]), _lib.dense_view(out[1][l0:l1]), idx, n_kept=n_kept)
+        return kept
 
     @torch.no_grad()
     def forward(self, kv_cache: List[LayerKV], it_len: Optional[List[int]] = None, **kwargs) -> List[LayerKV]:

@@ -219,6 +219,30 @@ def ccm_mlp(src: FcKvView, dst: FcKvView, weights: Tuple[torch.Tensor, ...], cf:
                            current_stream()), "fc_ccm_mlp")
 
 
+def ccm_mlp_ragged(src: FcKvView, dst: FcKvView, weights: Tuple[torch.Tensor, ...], cf: int,
+                   seg_start: torch.Tensor, seg_len: torch.Tensor, dst_start: torch.Tensor, max_seg_len: int,
+                   min_rows: int) -> None:
+    """``ccm_mlp`` with one segment per sequence: int32 device tensors ``[B]``; a sequence whose segment has fewer
+    than ``min_rows * cf`` tokens is copied through; ``max_seg_len`` bounds ``seg_len``."""
+    L, D = src.num_layers, src.head_dim
+    shapes = [(L, D, cf * D), (L, D), (L, D, D), (L, D), (L, D, D), (L, D)]
+    for t, shp, name in zip(weights, shapes, ("w1", "b1", "w2", "b2", "w3", "b3")):
+        _lib.require_gpu(t, name)
+        if tuple(t.shape) != shp or not t.is_contiguous() or _lib.dtype_code(t.dtype) != src.dtype:
+            raise FastcacheError(f"{name} must be contiguous {shp} in the KV dtype, got {tuple(t.shape)} {t.dtype}")
+    dev = weights[0].device
+    arrays = []
+    for t, name in ((seg_start, "seg_start"), (seg_len, "seg_len"), (dst_start, "dst_start")):
+        t = _i32(t, name, dev)
+        if t.numel() != src.batch:
+            raise FastcacheError(f"{name} must hold one entry per sequence ({src.batch}), got {t.numel()}")
+        arrays.append(t)
+    w = FcMlpWeights(*(t.data_ptr() for t in weights))
+    check(fn("fc_ccm_mlp_ragged")(C.byref(src), C.byref(dst), C.byref(w), cf, arrays[0].data_ptr(),
+                                  arrays[1].data_ptr(), arrays[2].data_ptr(), max_seg_len, min_rows,
+                                  current_stream()), "fc_ccm_mlp_ragged")
+
+
 def expected_attention_score(keys: FcKvView, values: FcKvView, mean_query: torch.Tensor,
                              cov_query: Optional[torch.Tensor], n_sink: int = 4, use_vnorm: bool = True,
                              epsilon: float = 0.0, score_stride: Optional[int] = None) -> torch.Tensor:

@@ -9,7 +9,7 @@ of the same pages in place.  Three launches per pass, nothing leaves the device.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -18,9 +18,10 @@ from . import _lib, ops
 
 @dataclass
 class PressResult:
-    indices: torch.Tensor          # int32 [L, B, Hkv (or 1), n_kept] ascending token positions
-    n_kept: int
+    indices: torch.Tensor          # int32 [L, B, Hkv (or 1), n_kept] ascending token positions (-1 past a row's count)
+    n_kept: int                    # kept tokens per sequence (the largest count when the sequences differ)
     scores: Optional[torch.Tensor]  # fp32 [L, B, Hkv, S] (None for index-only presses)
+    kept_per_seq: Optional[List[int]] = None    # set when the sequences have different lengths
 
 
 def n_kept_for(seq_len: int, compression_ratio: float) -> int:
@@ -35,32 +36,49 @@ def _views(kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.T
             _lib.paged_view(kv_cache[1], block_tables, seq_lens, max_seq_len))
 
 
+def _select_and_compact(kview, vview, scores, seq_lens, kept: List[int], compact: bool, heads: int) -> PressResult:
+    """Top-k per (layer, sequence, head) row and in-place compaction; one launch each whether or not the
+    sequences keep the same number of tokens."""
+    width = max(kept)
+    if len(set(kept)) == 1:
+        idx = ops.topk_select(scores, width)
+        if compact and width > 0:
+            ops.compact(kview, vview, kview, vview, idx)
+        return PressResult(idx, width, scores)
+    n_kept = torch.tensor(kept, dtype=torch.int32, device=scores.device)
+    idx = ops.topk_select(scores, width, row_lens=seq_lens, n_kept=n_kept, rows_per_len=heads)
+    if compact and width > 0:
+        ops.compact(kview, vview, kview, vview, idx, n_kept=n_kept)
+    return PressResult(idx, width, scores, list(kept))
+
+
 def knorm_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
-                         seq_len: int, compression_ratio: float, compact: bool = True) -> PressResult:
-    """KnormPress over sequences that all hold ``seq_len`` tokens."""
+                         seq_len: int, compression_ratio: float, compact: bool = True,
+                         host_lens: Optional[Sequence[int]] = None) -> PressResult:
+    """KnormPress over sequences that all hold ``seq_len`` tokens, or, with ``host_lens`` (the lengths as
+    Python ints, ``seq_len`` their maximum), over sequences of different lengths in the same launches: each keeps
+    ``int(its length * (1 - compression_ratio))`` tokens."""
     kview, vview = _views(kv_cache, block_tables, seq_lens, seq_len)
     scores = ops.knorm_score(kview, kv_cache.device)
-    n = n_kept_for(seq_len, compression_ratio)
-    idx = ops.topk_select(scores, n)
-    if compact and n > 0:
-        ops.compact(kview, vview, kview, vview, idx)
-    return PressResult(idx, n, scores)
+    lens = list(host_lens) if host_lens is not None else [seq_len] * block_tables.shape[0]
+    kept = [n_kept_for(n, compression_ratio) for n in lens]
+    return _select_and_compact(kview, vview, scores, seq_lens, kept, compact, kv_cache.shape[4])
 
 
 def snapkv_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
                           seq_len: int, queries: torch.Tensor, compression_ratio: float, window_size: int = 64,
                           kernel_size: int = 5, causal_window: bool = True, reduction: str = "mean",
-                          window_in_budget: bool = True, compact: bool = True) -> PressResult:
-    """SnapKVPress over sequences that all hold ``seq_len`` tokens.  ``queries`` are the rotated
-    window queries ``[L, B, Hq, W, D]``.  With ``window_in_budget`` (kvpress) the observation window
-    counts towards ``n_kept``; otherwise it is kept on top of it."""
+                          window_in_budget: bool = True, compact: bool = True,
+                          host_lens: Optional[Sequence[int]] = None) -> PressResult:
+    """SnapKVPress over sequences that all hold ``seq_len`` tokens, or (``host_lens``) of different lengths in
+    the same launches.  ``queries`` are the rotated window queries ``[L, B, Hq, W, D]`` (the last W positions of
+    every sequence).  With ``window_in_budget`` (kvpress) the observation window counts towards ``n_kept``;
+    otherwise it is kept on top of it."""
     kview, vview = _views(kv_cache, block_tables, seq_lens, seq_len)
     scores = ops.snapkv_score(kview, queries, window_size, kernel_size, causal_window, reduction,
                               seq_lens=seq_lens)
-    n = n_kept_for(seq_len, compression_ratio)
+    lens = list(host_lens) if host_lens is not None else [seq_len] * block_tables.shape[0]
+    kept = [n_kept_for(n, compression_ratio) for n in lens]
     if not window_in_budget:
-        n = min(seq_len, n + window_size)
-    idx = ops.topk_select(scores, n)
-    if compact and n > 0:
-        ops.compact(kview, vview, kview, vview, idx)
-    return PressResult(idx, n, scores)
+        kept = [min(n, k + window_size) for n, k in zip(lens, kept)]
+    return _select_and_compact(kview, vview, scores, seq_lens, kept, compact, kv_cache.shape[4])

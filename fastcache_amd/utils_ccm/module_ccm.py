@@ -112,16 +112,22 @@ class _CCMBase(nn.Module):
     @torch.no_grad()
     def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
                       seq_len: int, it_len: Sequence[int], layers: Optional[Tuple[int, int]] = None,
-                      out: Optional[torch.Tensor] = None) -> int:
+                      out: Optional[torch.Tensor] = None, host_lens: Optional[Sequence[int]] = None):
         """Compress sequences that all hold ``seq_len`` tokens in the pool
         ``kv_cache [2, L, blocks, block_size, Hkv, D]``.  By default in place: the result occupies the
         leading slots of the same block tables (what extract -> forward -> write-back leaves there).
         ``layers=(l0, l1)`` restricts the work to those layers; ``out [2, L, B, Hkv, C, D]`` receives the
-        result instead of the pages (which then stay untouched).  Returns the compressed length."""
+        result instead of the pages (which then stay untouched).  Returns the compressed length.
+
+        Sequences of different lengths go through the same launches: ``host_lens`` gives their lengths as
+        Python ints (``seq_lens`` holds the same numbers on the device, ``seq_len`` is their maximum) and the
+        result is the list of compressed lengths."""
         cf = self.compression_factor
         l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
         views = [_lib.paged_view(kv_cache[p][l0:l1], block_tables, seq_lens, seq_len) for p in range(2)]
         dviews = views if out is None else [_lib.dense_view(out[p][l0:l1]) for p in range(2)]
+        if host_lens is not None and len(set(host_lens)) > 1:
+            return self._paged_forward_ragged(views, dviews, list(host_lens), it_len, (l0, l1), kv_cache)
         dst = 0
         for gk, gv, s0, n in self._paged_segments(seq_len, it_len):
             if n == 0:
@@ -134,6 +140,29 @@ class _CCMBase(nn.Module):
                     w = tuple(t[l0:l1] for t in self._weights(g, kv_cache.dtype, kv_cache.device))
                     ops.ccm_mlp(view, dview, w, cf, s0, n, dst)
             dst += self._segment_len(n)
+        return dst
+
+    def _paged_forward_ragged(self, views, dviews, lens: List[int], it_len, layer_range, kv_cache) -> List[int]:
+        """One launch set for sequences of different lengths: per segment of the class's split rule, the
+        sequences' (start, length, destination) go to the device as three small int32 tensors."""
+        cf, (l0, l1) = self.compression_factor, layer_range
+        dev = kv_cache.device
+        per_seq = [self._paged_segments(n, it_len) for n in lens]
+        dst = [0] * len(lens)
+        for j in range(max(len(p) for p in per_seq)):
+            segs = [p[j] if j < len(p) else (p[-1][0], p[-1][1], 0, 0) for p in per_seq]
+            gk, gv = segs[0][0], segs[0][1]
+            if any((g[0], g[1]) != (gk, gv) for g in segs):
+                raise _lib.FastcacheError("sequences of one batch must take the same split rule")
+            n_max = max(g[3] for g in segs)
+            if n_max == 0:
+                continue
+            mk = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)
+            starts, counts, dsts = mk([g[2] for g in segs]), mk([g[3] for g in segs]), mk(dst)
+            for view, dview, g in ((views[0], dviews[0], gk), (views[1], dviews[1], gv)):
+                w = tuple(t[l0:l1] for t in self._weights(g, kv_cache.dtype, dev))
+                ops.ccm_mlp_ragged(view, dview, w, cf, starts, counts, dsts, n_max, self.min_seq_len)
+            dst = [d + self._segment_len(g[3]) for d, g in zip(dst, segs)]
         return dst
 
     def _forward_split(self, kv_cache: Sequence[LayerKV], it_len: Sequence[int], split: bool) -> List[LayerKV]:

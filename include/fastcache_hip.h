@@ -204,6 +204,19 @@ int fc_ccm_mlp(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weight
                int32_t cf, int32_t seg_start, int32_t seg_len, int32_t dst_start, void* stream);
 
 /*
+ * The same compressor when every sequence has its own segment (a batch of prompts of different lengths compressed in
+ * one pass instead of the reference's per-sequence loop, nanovllm/engine/llava_model_runner.py:745-786):
+ * seg_start[b], seg_len[b], dst_start[b] are int32 arrays of `batch` entries in DEVICE memory.  Per sequence:
+ * c = seg_len[b] / cf rows; with c < min_rows the segment is copied through unchanged (the min_seq_len guard of
+ * compress_layer, module_ccm_v11.py:674-675), otherwise rows j < c go to dst_start[b] + j and the remainder tokens
+ * behind them.  max_seg_len bounds every seg_len[b] (it sizes the launch); values read from the arrays are cut to
+ * the views' max_seq_len on the device.  `dst` may alias `src` when dst_start[b] <= seg_start[b] for every b.
+ */
+int fc_ccm_mlp_ragged(const fc_kv_view* src, const fc_kv_view* dst, const fc_mlp_weights* w, int32_t cf,
+                      const int32_t* seg_start, const int32_t* seg_len, const int32_t* dst_start,
+                      int32_t max_seg_len, int32_t min_rows, void* stream);
+
+/*
  * Expected-attention scores: attention each key can expect from future queries whose distribution is
  * Gaussian with mean mean_query[layer][b][hq][128] and covariance cov_query[layer][b][hq][128][128]
  * (fp32, contiguous; cov_query may be NULL = mean only).  For the keys past the first n_sink of a sequence

@@ -117,3 +117,71 @@ def test_ccm_mlp_dense_out_of_place(dev, dtype):
     # remainder tokens are copied bit-exactly
     n = (S // cf) * cf
     assert torch.equal(out[0, :, :, S // cf:].cpu(), k[0, :, :, n:])
+
+
+@pytest.mark.parametrize("dtype,cf,min_rows", [(torch.float16, 2, 1), (torch.bfloat16, 5, 2), (torch.bfloat16, 3, 1)])
+def test_ccm_mlp_ragged_segments_one_launch(dev, dtype, cf, min_rows):
+    """Ten sequences of ten different lengths (one shorter than the image segment, one whose text segment is too
+    short to compress, several with a remainder) through ONE ragged launch per segment and plane, in place, against
+    the oracle's per-sequence extract -> forward -> write-back."""
+    L, H, img = 2, 3, 40
+    lens = [700, 41, 39, 256, 257, 513, 40 + cf * min_rows - 1, 333, 64, 601]
+    B = len(lens)
+    case = synth.make_paged_case(seed=15, num_layers=L, batch=B, num_kv_heads=H, seq_lens=lens, dtype=dtype)
+    sd = occm.reference_init_state_dict("linear_decouple", L, 128, cf, seed=7)
+    ref_pool = case.kv_cache.clone()
+    ref_lens = []
+    for tab, n in zip(case.block_tables, lens):
+        hf = opaged.extract_kv(ref_pool, tab, n)
+        out = occm.linear_decouple_forward(hf, [img, max(1, n - img)], sd, cf, min_rows)
+        opaged.write_back(ref_pool, out, tab)
+        ref_lens.append(out[0][0].shape[2])
+
+    pool = case.kv_cache.to(dev)
+    tables, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+    S = max(lens)
+    views = [_lib.paged_view(pool[p], tables, lens_d, S) for p in range(2)]
+    mk = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)
+    seg_len = lambda n: n if n // cf < min_rows else n // cf + n % cf
+    imgs = [min(img, n) for n in lens]
+    dst = [0] * B
+    for starts, counts, groups in (([0] * B, imgs, ("compress_ik", "compress_iv")),
+                                   (imgs, [n - i for n, i in zip(lens, imgs)], ("compress_tk", "compress_tv"))):
+        for plane in range(2):
+            ops.ccm_mlp_ragged(views[plane], views[plane], stacked(sd, groups[plane], L, dtype, dev), cf, mk(starts),
+                               mk(counts), mk(dst), max(counts), min_rows)
+        dst = [d + seg_len(n) for d, n in zip(dst, counts)]
+    torch.cuda.synchronize()
+    assert dst == ref_lens
+    got = pool.cpu()
+    for tab, n, c in zip(case.block_tables, lens, ref_lens):
+        g, r = opaged.extract_kv(got, tab, n), opaged.extract_kv(ref_pool, tab, n)
+        for (gk, gv), (rk, rv) in zip(g, r):
+            assert_mlp_close(gk[:, :, :c], rk[:, :, :c], dtype)
+            assert_mlp_close(gv[:, :, :c], rv[:, :, :c], dtype)
+            assert torch.equal(gk[:, :, c:], rk[:, :, c:]) and torch.equal(gv[:, :, c:], rv[:, :, c:])   # stale tail untouched
+    used = {b for t in case.block_tables for b in t}
+    spare = [i for i in range(got.shape[2]) if i not in used]
+    assert torch.equal(got[:, :, spare], case.kv_cache[:, :, spare])
+
+
+def test_ccm_mlp_ragged_clamps_device_side_numbers(dev):
+    """Segment numbers in device memory beyond what the host validated (negative, past the view) are cut on the
+    device: nothing outside the sequences' own pages is written and no page past a table is read."""
+    L, H, cf, dtype = 1, 2, 2, torch.float16
+    lens = [300, 200]
+    case = synth.make_paged_case(seed=3, num_layers=L, batch=2, num_kv_heads=H, seq_lens=lens, dtype=dtype, fill_value=9.0)
+    sd = occm.reference_init_state_dict("linear_decouple", L, 128, cf, seed=7)
+    pool = case.kv_cache.to(dev)
+    tables, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+    view = _lib.paged_view(pool[0], tables, lens_d, 300)
+    mk = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)
+    ops.ccm_mlp_ragged(view, view, stacked(sd, "compress_tk", L, dtype, dev), cf, mk([-5, 2 ** 30]), mk([2 ** 31 - 1, 77]),
+                       mk([0, -3]), 300, 1)
+    torch.cuda.synchronize()
+    got = pool.cpu()
+    used = {b for t in case.block_tables for b in t}
+    spare = [i for i in range(got.shape[2]) if i not in used]
+    assert bool((got[:, :, spare] == 9.0).all())
+    assert torch.equal(got[1], case.kv_cache[1])                 # the V plane was not part of the call
+    assert torch.equal(got[0, :, case.block_tables[1]], case.kv_cache[0, :, case.block_tables[1]])   # start past the view: nothing

@@ -506,3 +506,65 @@ def test_decode_overlap_compression_splices_generated_rows(dev, backend):
     freed = free_compressed_blocks(bm, runner, seqs)
     assert freed == sum(-(-(n + 3) // 256) - (-(-(runner_len) // 256)) for n, runner_len in
                         zip(lens, [s.kv_cache_len for s in seqs]))
+
+
+@pytest.mark.parametrize("backend", ["mlp", "batched", "hybrid", "kvpress-knorm", "kvpress-streaming"])
+def test_runner_ragged_batch_in_one_pass(dev, backend):
+    """Nine running sequences of nine different lengths (the state a lazy compression trigger finds) compressed by
+    ONE paged_forward call, against the reference's per-sequence loop on the CPU."""
+    dtype, L, H, img = torch.bfloat16, 2, 2, 100
+    lens = [700, 257, 256, 255, 101, 1000, 333, 512, 130]
+    case = synth.make_paged_case(seed=77, num_layers=L, batch=len(lens), num_kv_heads=H, seq_lens=lens, dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0)
+    torch.manual_seed(2)
+    kw, image_len = {}, img
+    if backend in ("mlp", "batched"):
+        mlp = KVCacheLinearDecoupleCompressor(llava_cfg(L, H), compression_factor=2).to(dev).to(dtype).eval()
+        sd = {k: v.detach().cpu().float() for k, v in mlp.state_dict().items()}
+        kw["compressor"] = mlp
+        if backend == "batched":
+            bat = BatchedGEMMCompressor(L, H, 128, 2)
+            bat.load_from_original_compressor(mlp)
+            kw["batched_compressor"] = bat
+        oracle_comp = lambda hf, i, n: occm.linear_decouple_forward(hf, [img, max(1, n - img)], sd, 2, 1)
+    elif backend == "hybrid":
+        image_len = 0
+        cfg = SimpleNamespace(architectures=["MiniCPMV"], num_hidden_layers=L, num_key_value_heads=H,
+                              num_attention_heads=H, hidden_size=H * 128)
+        hyb = KVCacheHybridCompressor(cfg, compression_factor=5, min_seq_len=30).to(dev).to(dtype).eval()
+        sd = {k: v.detach().cpu().float() for k, v in hyb.state_dict().items()}
+        kw["compressor"] = hyb
+        oracle_comp = lambda hf, i, n: occm.hybrid_forward(hf, [0, n], sd, 5, 30)      # 101 and 130 tokens pass through
+    else:
+        method = backend.split("-")[1].replace("streaming", "streaming_llm")
+        kw["compressor"] = KVPressCompressor(method, 1.0 - 1.0 / 3)
+        oracle_comp = lambda hf, i, n: [opress.adapter_compress_layer(method, k, v, 1.0 - 1.0 / 3) for k, v in hf]
+    nb = case.kv_cache.shape[2]
+    runner = PagedKVRunner(L, H, 128, num_blocks=nb, dtype=dtype, device=dev, image_token_len=image_len, **kw)
+    bm = BlockManager(nb, 256)
+    seqs = [Sequence(list(range(2000 * i, 2000 * i + n))) for i, n in enumerate(lens)]
+    for s in seqs:
+        bm.allocate(s)
+    _fill_pool_from_case(runner, case, seqs)
+    tables_before = [list(s.block_table) for s in seqs]
+    ref_pool = runner.kv_cache.cpu()
+    ref_lens, ref_free, ref_ratio = opipe.compress_batch(ref_pool, tables_before, lens, oracle_comp)
+
+    comp = runner._active_compressor()
+    calls = []
+    inner = comp.paged_forward
+    comp.paged_forward = lambda *a, **k: (calls.append(1), inner(*a, **k))[1]
+    sec, ratio = runner.compress_kv_cache_batch(seqs)
+    assert len(calls) == 1 and abs(ratio - ref_ratio) < 1e-9
+    got_pool = runner.kv_cache.cpu()
+    for i, (s, tab, n) in enumerate(zip(seqs, tables_before, lens)):
+        C = ref_lens[i]
+        assert runner._compressed_lens[s.seq_id] == C
+        assert runner._blocks_to_free.get(s.seq_id, []) == ref_free.get(i, [])
+        for (gk, gv), (rk, rv) in zip(opaged.extract_kv(got_pool, tab, n), opaged.extract_kv(ref_pool, tab, n)):
+            if backend.startswith("kvpress"):
+                assert torch.equal(gk, rk) and torch.equal(gv, rv)
+            else:
+                assert_mlp_close(gk[:, :, :C], rk[:, :, :C], dtype)
+                assert_mlp_close(gv[:, :, :C], rv[:, :, :C], dtype)
+                assert torch.equal(gk[:, :, C:], rk[:, :, C:]) and torch.equal(gv[:, :, C:], rv[:, :, C:])

@@ -2,7 +2,7 @@
 import pytest
 import torch
 
-from fastcache_amd import _lib, ops, synth
+from fastcache_amd import _lib, ops, paged_press, synth
 from fastcache_amd.presses import SimLayerKVPress, ThinKPress
 from oracle import paged as opaged
 from oracle import presses as opress
@@ -476,3 +476,52 @@ def test_simlayer_press(dev, dtype, n_last, n_recent, n_initial):
     short = kd[:, :, :n_initial + n_recent + n_last]
     ok, _ = lazy.compress(None, None, short, short, None, kw)
     assert ok.data_ptr() == short.data_ptr() and len(lazy.compression_ratios) == 1
+
+
+@pytest.mark.parametrize("press", ["knorm", "snapkv"])
+def test_paged_press_ragged_batch_in_one_launch_set(dev, press):
+    """Eight sequences of eight different lengths scored, selected and compacted by one launch each: every
+    sequence keeps int(its length * (1 - ratio)) tokens, as the reference's per-sequence press does."""
+    dtype, L, Hq, Hkv, W, ksz, ratio = torch.bfloat16, 2, 8, 2, 16, 5, 0.6
+    lens = [700, 130, 257, 256, 64, 1000, 511, 90]       # every budget holds the whole window
+    B = len(lens)
+    case = synth.make_paged_case(seed=41, num_layers=L, batch=B, num_kv_heads=Hkv, seq_lens=lens, dtype=dtype,
+                                 keep_dense=True)
+    q = torch.randn(L, B, Hq, W, 128, generator=torch.Generator().manual_seed(4)).to(dtype)
+    pool = case.kv_cache.to(dev)
+    tables, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+    if press == "knorm":
+        res = paged_press.knorm_compress_paged(pool, tables, lens_d, max(lens), ratio, host_lens=lens)
+    else:
+        res = paged_press.snapkv_compress_paged(pool, tables, lens_d, max(lens), q.to(dev), ratio, W, ksz, True, "sum",
+                                                host_lens=lens)
+    torch.cuda.synchronize()
+    assert res.kept_per_seq == [int(n * (1 - ratio)) for n in lens]
+    got = pool.cpu()
+    for b, n in enumerate(lens):
+        k_keep = res.kept_per_seq[b]
+        for l in range(L):
+            kd, vd = case.dense_k[l][b:b + 1, :, :n], case.dense_v[l][b:b + 1, :, :n]
+            if press == "knorm":
+                ref = opress.knorm_score(kd)
+                scored = n
+            else:
+                ref = opress.snapkv_score(q[l, b:b + 1], kd, W, ksz, True, "sum")
+                scored = n - W
+            sc = res.scores[l, b:b + 1, :, :n].cpu()
+            torch.testing.assert_close(sc[..., :scored], ref[..., :scored], rtol=1e-3, atol=1e-3 * float(ref[..., :scored].abs().mean()))
+            assert bool(torch.isinf(res.scores[l, b, :, n:]).all())
+            idx = res.indices[l, b:b + 1, :, :k_keep].cpu().long()
+            assert bool((res.indices[l, b, :, k_keep:] == -1).all())
+            want = opress.topk_lowest_index(sc, k_keep)                      # the stable selection on the kernel's own scores
+            assert torch.equal(idx, want)
+            tie = opress.near_tie_rows(ref[..., :scored], k_keep - (0 if press == "knorm" else W))
+            ref_full = ref.clone()
+            ref_full[..., scored:] = sc[..., scored:]
+            assert torch.equal(idx[~tie], opress.topk_lowest_index(ref_full, k_keep)[~tie])
+            blocks = case.block_tables[b]
+            for p, dense in enumerate((kd, vd)):
+                rows = torch.cat([got[p, l, blk] for blk in blocks])[:n].permute(1, 0, 2).unsqueeze(0)   # [1, H, n, D]
+                assert torch.equal(rows[:, :, :k_keep], opress.gather_tokens(dense, idx))
+                old = torch.cat([case.kv_cache[p, l, blk] for blk in blocks])[:n].permute(1, 0, 2).unsqueeze(0)
+                assert torch.equal(rows[:, :, k_keep:], old[:, :, k_keep:])
