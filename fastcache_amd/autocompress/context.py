@@ -23,7 +23,8 @@ class GPUArch(Enum):
 
 @dataclass
 class HardwareProfile:
-    """Peak figures used for roofline estimates (context.py:27-107)."""
+    """Peak figures of one GPU (the field list of the reference's profile, context.py:27-107) and the two-roof
+    estimates built on them."""
     gpu_name: str = "Unknown"
     gpu_arch: GPUArch = GPUArch.UNKNOWN
     compute_capability: tuple = (0, 0)
@@ -35,32 +36,35 @@ class HardwareProfile:
     l2_cache_mb: float = 0.0
     sm_count: int = 0
     max_threads_per_sm: int = 0
-    _roofline_intensity: Optional[float] = None
+
+    DEFAULT_RIDGE = 150.0      # FLOP per byte assumed when the peaks are unknown
 
     @property
     def roofline_intensity(self) -> float:
-        """FLOP/byte at which a kernel stops being memory-bound; 150 when the peaks are unknown."""
-        if self._roofline_intensity is not None:
-            return self._roofline_intensity
-        if self.fp16_tflops > 0 and self.memory_bandwidth_gbps > 0:
-            self._roofline_intensity = (self.fp16_tflops * 1e12) / (self.memory_bandwidth_gbps * 1e9)
-            return self._roofline_intensity
-        return 150.0
+        """The ridge of the roofline: FLOP per byte above which fp16 compute, not memory, is the limit."""
+        if self.fp16_tflops <= 0 or self.memory_bandwidth_gbps <= 0:
+            return self.DEFAULT_RIDGE
+        return self.fp16_tflops * 1e3 / self.memory_bandwidth_gbps
+
+    @staticmethod
+    def _decode_work(batch_size: int, seq_len: int, num_heads: int, head_dim: int):
+        """(FLOP, bytes) of one decode step's attention over a 16-bit cache: every cached element is read once
+        for K and once for V and takes part in one multiply-add."""
+        elems = batch_size * seq_len * num_heads * head_dim
+        return 2 * elems, 4 * elems
 
     def is_decode_memory_bound(self, batch_size: int, seq_len: int, num_heads: int = 32, head_dim: int = 128) -> bool:
-        flops = batch_size * seq_len * num_heads * head_dim * 2
-        bytes_read = batch_size * seq_len * num_heads * head_dim * 2 * 2
-        return flops / max(bytes_read, 1) < self.roofline_intensity * 0.5
+        flops, nbytes = self._decode_work(batch_size, seq_len, num_heads, head_dim)
+        return flops < 0.5 * self.roofline_intensity * max(nbytes, 1)
 
     def estimate_decode_latency_ms(self, batch_size: int, seq_len: int, num_heads: int = 32,
                                    head_dim: int = 128) -> float:
-        flops = batch_size * seq_len * num_heads * head_dim * 2
-        bytes_read = batch_size * seq_len * num_heads * head_dim * 2 * 2
-        if flops / max(bytes_read, 1) < self.roofline_intensity:
-            latency_s = bytes_read / (self.memory_bandwidth_gbps * 1e9)
-        else:
-            latency_s = flops / (self.fp16_tflops * 1e12)
-        return latency_s * 1000 + 0.01
+        """The slower of the two roofs plus 10 microseconds of launch overhead."""
+        if self.fp16_tflops <= 0 or self.memory_bandwidth_gbps <= 0:
+            raise ValueError(f"{self.gpu_name}: peak figures unknown")
+        flops, nbytes = self._decode_work(batch_size, seq_len, num_heads, head_dim)
+        seconds = max(nbytes / (self.memory_bandwidth_gbps * 1e9), flops / (self.fp16_tflops * 1e12))
+        return seconds * 1e3 + 0.01
 
 
 @dataclass

@@ -1,4 +1,9 @@
-"""Stream handling for compression beside decoding (reference: nanovllm/autocompress/execution.py:438-500)."""
+"""The two streams of the compress-beside-decode schedule (the role of the reference's ``StreamManager``,
+nanovllm/autocompress/execution.py:438-500).
+
+Both streams have the default priority: the reference asks for a low-priority side stream, which this platform
+does not mix reliably with default-priority work; the order between the streams comes from events either way.
+"""
 from __future__ import annotations
 
 from typing import Optional
@@ -7,44 +12,39 @@ import torch
 
 
 class StreamManager:
-    """The main stream and one side stream for compression.  Both have the default priority: the
-    reference asks for a low-priority side stream, which this platform does not mix reliably with
-    default-priority work; ordering is by events either way."""
+    """Created lazily on first use, so that importing the package never touches the GPU."""
 
     def __init__(self):
-        self._main_stream = None
-        self._compress_stream = None
-        self._initialized = False
+        self._streams: Optional[tuple] = None        # (main, compress)
 
-    def initialize(self):
-        if self._initialized:
-            return
-        if torch.cuda.is_available():
-            self._main_stream = torch.cuda.current_stream()
-            self._compress_stream = torch.cuda.Stream()
-            self._initialized = True
+    def _pair(self) -> tuple:
+        if self._streams is None:
+            if not torch.cuda.is_available():
+                return (None, None)
+            self._streams = (torch.cuda.current_stream(), torch.cuda.Stream())
+        return self._streams
+
+    def initialize(self) -> None:
+        self._pair()
 
     def get_main_stream(self):
-        self.initialize()
-        return self._main_stream
+        return self._pair()[0]
 
     def get_compress_stream(self):
-        self.initialize()
-        return self._compress_stream
+        return self._pair()[1]
 
-    def synchronize_compress_to_main(self):
-        """The main stream waits for everything enqueued on the compression stream so far."""
-        if self._compress_stream is not None:
-            event = torch.cuda.Event()
-            event.record(self._compress_stream)
-            self._main_stream.wait_event(event)
+    def synchronize_compress_to_main(self) -> None:
+        """Everything enqueued on the compression stream so far happens before what the main stream gets next."""
+        main, side = self._pair()
+        if side is not None:
+            main.wait_event(side.record_event())
 
 
-_stream_manager: Optional[StreamManager] = None
+_manager: Optional[StreamManager] = None
 
 
 def get_stream_manager() -> StreamManager:
-    global _stream_manager
-    if _stream_manager is None:
-        _stream_manager = StreamManager()
-    return _stream_manager
+    global _manager
+    if _manager is None:
+        _manager = StreamManager()
+    return _manager

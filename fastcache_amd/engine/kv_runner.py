@@ -41,6 +41,7 @@ class PagedKVRunner:
         self._blocks_to_free: Dict[int, List[int]] = {}
         self._lock = threading.Lock()
         self._compress_stream: Optional[torch.cuda.Stream] = None
+        self._launch_started = False      # set once an enqueue may have begun to rewrite cache rows in place
 
     # -- tables -----------------------------------------------------------------------------------
     def preare_block_tables(self, seqs: Seq[Sequence]) -> torch.Tensor:
@@ -109,6 +110,7 @@ class PagedKVRunner:
             S = max(lens)
             tt, ll = self._table_and_lens([s.block_table for s in seqs], lens)
             it_len = [image_len, max(1, S - image_len)]
+            self._launch_started = True       # from here on a failure may leave rows partly rewritten
             C = comp.paged_forward(self.kv_cache, tt, ll, S, it_len, host_lens=lens)
             per_seq = list(C) if isinstance(C, (list, tuple)) else [C] * len(seqs)
             for s, n, c in zip(seqs, lens, per_seq):
@@ -122,6 +124,7 @@ class PagedKVRunner:
                 it_len = [image_len, max(1, S - image_len)]
                 with torch.no_grad():
                     out = comp(hf, it_len=it_len)
+                self._launch_started = True   # the write-back below is the first thing that touches the pages
                 self._write_compressed_kv_cache_fast(out, s.block_table)
                 result[s.seq_id] = out[0][0].shape[2]
                 orig += sum(k.numel() + v.numel() for k, v in hf)

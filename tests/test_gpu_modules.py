@@ -359,6 +359,18 @@ def test_async_compression_manager_states_and_effective_len(dev):
     bmgr.start_async_compression(seqs[:1], image_len=0)
     bmgr.wait_all_compressions()
     assert bmgr.seq_states[seqs[0].seq_id] == CompressionState.NONE and bmgr.get_effective_kv_len(seqs[0]) == S
+    # a compressor that works in place and fails after it may have launched: the rows are no longer trustworthy,
+    # the sequence is marked FAILED and asking for its length raises instead of handing out a stale number
+    class Halfway:
+        def paged_forward(self, *a, **k):
+            raise RuntimeError("second launch rejected")
+    half = PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0, compressor=Halfway())
+    hmgr = AsyncCompressionManager(half)
+    hmgr.start_async_compression(seqs[:1], image_len=0)
+    hmgr.wait_all_compressions()
+    assert hmgr.seq_states[seqs[0].seq_id] == CompressionState.FAILED
+    with pytest.raises(Exception, match="prefill again"):
+        hmgr.get_effective_kv_len(seqs[0])
     assert AsyncCompressionManager(PagedKVRunner(L, H, 128, 2, dtype, dev)).start_async_compression(seqs) is None
 
 
