@@ -1,5 +1,5 @@
 // Decode-side kernels over the paged cache: append one K/V row per sequence, advance the lengths,
-// and single-query paged attention (split over 256-token chunks, then merged).
+// and single-query paged attention (split over chunks of 256 to 512 tokens, then merged).
 //
 // Attention is HBM-bound (one pass over K and V, ~1 FLOP per byte per query head), so the kernel is
 // organised around keeping loads in flight.  A workgroup owns one (sequence, kv head, 256-token
@@ -17,7 +17,8 @@
 #include "fc_common.h"
 
 #define DA_THREADS 256
-#define DA_CHUNK 256
+#define DA_CHUNK 256               // smallest chunk (tokens per workgroup); it sizes the workspace
+#define DA_CHUNK_MAX 512           // largest: the host picks a multiple of 32 in between from the launch's shape
 #define DA_LOG2E 1.4426950408889634f
 
 template <int DTYPE>
@@ -48,10 +49,10 @@ __device__ __forceinline__ unsigned short da_pack(float f) {
 
 template <int GT>
 struct DaCfg {
-  // ring | logits, then probabilities [GT][256]: fp32, or with eight heads (p * V on the matrix pipe) each
+  // ring | logits, then probabilities [GT][chunk]: fp32, or with eight heads (p * V on the matrix pipe) each
   // probability as two 16-bit halves hi + lo in the cache dtype
   static constexpr bool PV_MFMA = GT >= DA_PV_MFMA_MIN;
-  static constexpr int LDS = DA_RING + GT * DA_CHUNK * 4;
+  static constexpr int lds(int chunk) { return DA_RING + GT * chunk * 4; }
 };
 
 // GT = query heads served per workgroup (a tile of the group, at most 8).
@@ -69,10 +70,11 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
                                                                     const char* __restrict__ q, int Hq,
                                                                     const int* __restrict__ lens, float c,
                                                                     float* __restrict__ part_o,
-                                                                    float* __restrict__ part_ml, int max_splits) {
+                                                                    float* __restrict__ part_ml, int max_splits,
+                                                                    int chunk) {
   extern __shared__ __align__(16) char smem[];
-  float(*sc)[DA_CHUNK] = reinterpret_cast<float(*)[DA_CHUNK]>(smem + DA_RING);
-  unsigned(*p2)[DA_CHUNK] = reinterpret_cast<unsigned(*)[DA_CHUNK]>(smem + DA_RING);   // sc seen as (hi, lo) pairs
+  float* sc = reinterpret_cast<float*>(smem + DA_RING);          // [GT][chunk]
+  unsigned* p2 = reinterpret_cast<unsigned*>(smem + DA_RING);    // the same seen as (hi, lo) pairs
   constexpr bool PV_MFMA = DaCfg<GT>::PV_MFMA;
   float(*red)[GT][FC_HEAD_DIM] = reinterpret_cast<float(*)[GT][FC_HEAD_DIM]>(smem);  // [16] partial outputs, reuses the ring
   static_assert(16 * GT * FC_HEAD_DIM * 4 <= DA_RING, "partial outputs must fit in the ring");
@@ -89,9 +91,9 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
   const int h = blockIdx.y / gtiles, g0 = (blockIdx.y - h * gtiles) * GT;
   int len = __builtin_amdgcn_readfirstlane(lens[b]);
   len = min(len, kc.max_seq_len);
-  const int t0 = split * DA_CHUNK;
+  const int t0 = split * chunk;
   if (t0 >= len) return;
-  const int ntok = min(DA_CHUNK, len - t0);
+  const int ntok = min(chunk, len - t0);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -152,14 +154,26 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
     }
   };
 
-  const int tile_a = wave, tile_b = wave + 4;
-  const bool has_a = tile_a * DA_TILE < ntok, has_b = tile_b * DA_TILE < ntok;   // wave-uniform
-  if (has_a) issue(kc, kbase, tile_a, 0);
-  if (has_b) issue(kc, kbase, tile_b, 1);
+  // This wavefront's tiles are wave, wave + 4, wave + 8, ...: nj of them hold tokens.  Their K tiles and then
+  // their V tiles form one stream of 2 * nj items; item i goes to stage i & 1 and is issued as soon as item
+  // i - 2 has been consumed, so two items (16 KB) are in flight for most of the kernel.
+  const int live_tiles = (ntok + DA_TILE - 1) / DA_TILE;
+  const int nj = wave < live_tiles ? (live_tiles - wave + 3) / 4 : 0;   // wave-uniform
+  auto issue_item = [&](int i) {
+    if (i < nj) issue(kc, kbase, wave + 4 * i, i & 1);
+    else if (i < 2 * nj) issue(vc, vbase, wave + 4 * (i - nj), i & 1);
+  };
+  // item i has landed when at most the loads of item i + 1 (eight per lane) are outstanding
+  auto wait_item = [&](int i) {
+    if (i + 1 < 2 * nj) fc_wait_vm<8>(); else fc_wait_vm<0>();
+  };
+  issue_item(0);
+  issue_item(1);
 
   // ---- phase 1: logits of this wavefront's tiles --------------------------------------------------
   // C[head][key]: the lane owns key lrow of the tile and the heads (i/4)*8 + lhalf*4 + i%4, of which
-  // only heads < 8 exist, that is registers 0..3.
+  // only heads < 8 exist, that is registers 0..3.  Tokens past the sequence end get -inf; tiles past
+  // it are never read (the statistics below stop at ntok).
   const unsigned xs = (unsigned)((lhalf ^ (lrow & 15)) << 4) + lrow * 256;
   auto logits = [&](int tile, int stage) {
     f32x16 acc;
@@ -175,46 +189,38 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int g = lhalf * 4 + i;
-      if (g < GT) sc[g][t] = live ? acc[i] * c : -INFINITY;
+      if (g < GT) sc[g * chunk + t] = live ? acc[i] * c : -INFINITY;
     }
   };
-  auto no_logits = [&](int tile) {
-    for (int i = lane; i < GT * DA_TILE; i += 64) sc[i / DA_TILE][tile * DA_TILE + (i % DA_TILE)] = -INFINITY;
-  };
-  if (has_a) {
-    if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
-    logits(tile_a, 0);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the stage's reads are done before V lands in it
-    issue(vc, vbase, tile_a, 0);
-  } else {
-    no_logits(tile_a);
-  }
-  if (has_b) {
-    fc_wait_vm<8>();   // K tile b has landed, V tile a may still be in flight
-    logits(tile_b, 1);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    issue(vc, vbase, tile_b, 1);
-  } else {
-    no_logits(tile_b);
+  for (int i = 0; i < nj; ++i) {
+    wait_item(i);
+    logits(wave + 4 * i, i & 1);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the stage's reads are done before the next item lands in it
+    issue_item(i + 2);
   }
   fc_lds_barrier();
 
   // ---- phase 2: chunk statistics, one wavefront per query head -------------------------------------
   for (int g = wave; g < GT; g += 4) {
-    float x[4];
+    float x[DA_CHUNK_MAX / 64];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) x[j] = sc[g][lane + 64 * j];
-    const float m = fc_wave_max_uniform(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
+    for (int j = 0; j < DA_CHUNK_MAX / 64; ++j) x[j] = lane + 64 * j < ntok ? sc[g * chunk + lane + 64 * j] : -INFINITY;
+    float mx = x[0];
+#pragma unroll
+    for (int j = 1; j < DA_CHUNK_MAX / 64; ++j) mx = fmaxf(mx, x[j]);
+    const float m = fc_wave_max_uniform(mx);
     float sum = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < DA_CHUNK_MAX / 64; ++j) {
       const float p = __builtin_amdgcn_exp2f(x[j] - m);   // exp2(-inf) = 0 for the padded slots
-      if constexpr (PV_MFMA) {
-        const unsigned short hi = da_pack<DTYPE>(p);
-        const float hf = DTYPE == FC_BF16 ? fc_bf16_to_float(hi) : fc_half_to_float(hi);
-        p2[g][lane + 64 * j] = (unsigned)hi | ((unsigned)da_pack<DTYPE>(p - hf) << 16);
-      } else {
-        sc[g][lane + 64 * j] = p;
+      if (lane + 64 * j < live_tiles * DA_TILE) {         // every slot of a live tile is read by phase 3
+        if constexpr (PV_MFMA) {
+          const unsigned short hi = da_pack<DTYPE>(p);
+          const float hf = DTYPE == FC_BF16 ? fc_bf16_to_float(hi) : fc_half_to_float(hi);
+          p2[g * chunk + lane + 64 * j] = (unsigned)hi | ((unsigned)da_pack<DTYPE>(p - hf) << 16);
+        } else {
+          sc[g * chunk + lane + 64 * j] = p;
+        }
       }
       sum += p;
     }
@@ -246,8 +252,8 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
         const int k0 = s * 16 + lhalf * 8;   // first of this lane's 8 keys of the k-step
         uint4 a = make_uint4(0, 0, 0, 0), a2 = make_uint4(0, 0, 0, 0);
         if (lrow < GT) {
-          const uint4 d0 = *reinterpret_cast<const uint4*>(&p2[lrow][tile * DA_TILE + k0]);
-          const uint4 d1 = *reinterpret_cast<const uint4*>(&p2[lrow][tile * DA_TILE + k0 + 4]);
+          const uint4 d0 = *reinterpret_cast<const uint4*>(&p2[lrow * chunk + tile * DA_TILE + k0]);
+          const uint4 d1 = *reinterpret_cast<const uint4*>(&p2[lrow * chunk + tile * DA_TILE + k0 + 4]);
           // v_perm_b32 bytes: 0-3 second operand, 4-7 first operand
           a = make_uint4(__builtin_amdgcn_perm(d0.y, d0.x, 0x05040100u), __builtin_amdgcn_perm(d0.w, d0.z, 0x05040100u),
                          __builtin_amdgcn_perm(d1.y, d1.x, 0x05040100u), __builtin_amdgcn_perm(d1.w, d1.z, 0x05040100u));
@@ -271,13 +277,11 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
         }
       }
     };
-    if (has_a) {
-      if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
-      pv(tile_a, 0);
-    }
-    if (has_b) {
-      fc_wait_vm<0>();
-      pv(tile_b, 1);
+    for (int i = nj; i < 2 * nj; ++i) {
+      wait_item(i);
+      pv(wave + 4 * (i - nj), i & 1);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      issue_item(i + 2);
     }
     fc_lds_barrier();   // every wavefront is done with its ring before the ring becomes `red`
     // C layout: the lane holds output dimension nb*32 + lrow of the heads lhalf*4 + i (registers 0..3)
@@ -312,19 +316,17 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
         da_unpack8<DTYPE>(vx, vf);
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
-          const float pr = sc[g][tile * DA_TILE + r];
+          const float pr = sc[g * chunk + tile * DA_TILE + r];
 #pragma unroll
           for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e]);
         }
       }
     };
-    if (has_a) {
-      if (has_b) fc_wait_vm<8>(); else fc_wait_vm<0>();
-      pv(tile_a, 0);
-    }
-    if (has_b) {
-      fc_wait_vm<0>();
-      pv(tile_b, 1);
+    for (int i = nj; i < 2 * nj; ++i) {
+      wait_item(i);
+      pv(wave + 4 * (i - nj), i & 1);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      issue_item(i + 2);
     }
     fc_lds_barrier();   // every wavefront is done with its ring before the ring becomes `red`
     // 16 partial outputs (4 wavefronts x 4 row slots) through LDS, summed in a fixed order
@@ -354,7 +356,8 @@ template <int DTYPE>
 __global__ __launch_bounds__(FC_HEAD_DIM) void decode_merge_kernel(const float* __restrict__ part_o,
                                                                    const float* __restrict__ part_ml,
                                                                    const int* __restrict__ lens, int max_seq_len,
-                                                                   int Hq, int max_splits, char* __restrict__ out) {
+                                                                   int Hq, int max_splits, int chunk,
+                                                                   char* __restrict__ out) {
   const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   int len = min(lens[b], max_seq_len);
   unsigned short* o = reinterpret_cast<unsigned short*>(out) + ((long long)b * Hq + hq) * FC_HEAD_DIM + d;
@@ -362,7 +365,7 @@ __global__ __launch_bounds__(FC_HEAD_DIM) void decode_merge_kernel(const float* 
     *o = 0;
     return;
   }
-  const int ns = (len + DA_CHUNK - 1) / DA_CHUNK;
+  const int ns = (len + chunk - 1) / chunk;
   const float* ml = part_ml + ((long long)b * Hq + hq) * max_splits * 2;
   const float* po = part_o + ((long long)b * Hq + hq) * max_splits * FC_HEAD_DIM + d;
   // eight splits per step so that their loads are in flight together
@@ -493,6 +496,18 @@ extern "C" int64_t fc_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_h
   return (int64_t)batch * num_q_heads * (splits > 0 ? splits : 1) * (FC_HEAD_DIM + 2) * (int64_t)sizeof(float);
 }
 
+// compute units of the current device (0 if the query fails), cached per device
+static int da_compute_units() {
+  static int cus[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus[dev] = n;
+  }
+  return cus[dev];
+}
+
 // Checks and launches shared by the entry points; `workspace` is a device address.
 static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer,
                       const void* q, void* out, int32_t num_q_heads, const int32_t* context_lens, float scale,
@@ -512,8 +527,35 @@ static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_vi
   const int64_t need = fc_decode_attn_workspace_bytes(k_cache->batch, num_q_heads, k_cache->max_seq_len);
   FC_REQUIRE(workspace_bytes >= need, FC_EINVAL, "%s: workspace of %lld bytes, %lld needed", who,
              (long long)workspace_bytes, (long long)need);
-  const int splits = (k_cache->max_seq_len + DA_CHUNK - 1) / DA_CHUNK;
   const int B = k_cache->batch, Hkv = k_cache->num_kv_heads, G = num_q_heads / Hkv;
+  // the smallest tile that holds the whole group (padded head rows cost nothing; splitting a group would
+  // read its K and V once per tile); groups of more than 8 heads are served 8 at a time
+  const int gt = G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
+  const int gtiles = (G + gt - 1) / gt;
+  // Tokens per workgroup.  A launch of many rounds of workgroups keeps the smallest chunk (best balance over
+  // ragged lengths).  A launch of a few rounds is all ramp and tail: there the chunk is the multiple of 32
+  // tokens for which the workgroups fill whole rounds of the GPU (two workgroups per compute unit), by a
+  // coarse cost of rounds * (chunk + fixed part).  Only the view's max_seq_len enters, never the lengths on the
+  // device, so the choice is the same at capture and at every replay.
+  int chunk = DA_CHUNK;
+  {
+    const int slots = 2 * da_compute_units();
+    const long long cols = (long long)Hkv * gtiles * B;
+    const long long wgs256 = cols * ((k_cache->max_seq_len + DA_CHUNK - 1) / DA_CHUNK);
+    if (slots > 0 && wgs256 < 4LL * slots) {
+      double best = -1.0;
+      for (int cand = DA_CHUNK; cand <= DA_CHUNK_MAX; cand += DA_TILE) {
+        if (gt == 8 && DaCfg<8>::lds(cand) * 2 >= 160 * 1024) break;   // two workgroups per compute unit must fit its LDS
+        const long long wgs = cols * ((k_cache->max_seq_len + cand - 1) / cand);
+        const double cost = (double)((wgs + slots - 1) / slots) * (cand + 96.0);
+        if (best < 0 || cost < best - 1e-9) {
+          best = cost;
+          chunk = cand;
+        }
+      }
+    }
+  }
+  const int splits = (k_cache->max_seq_len + chunk - 1) / chunk;
   float* part_o = (float*)workspace;
   float* part_ml = part_o + (int64_t)B * num_q_heads * (splits > 0 ? splits : 1) * FC_HEAD_DIM;
   KvView k = fc_make_view(k_cache), v = fc_make_view(v_cache);
@@ -521,10 +563,6 @@ static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_vi
   const float c = scale * DA_LOG2E;
   const bool bf = k_cache->dtype == FC_BF16;
   if (splits > 0) {
-    // the smallest tile that holds the whole group (padded head rows cost nothing; splitting a group would
-    // read its K and V once per tile); groups of more than 8 heads are served 8 at a time
-    const int gt = G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
-    const int gtiles = (G + gt - 1) / gt;
     FC_REQUIRE(Hkv * gtiles <= 65535 && B <= 65535, FC_EUNSUPPORTED, "%s: grid too large", who);
     dim3 grid(splits, Hkv * gtiles, B);
     const auto tile_in_page = [](const fc_kv_view* v, const KvView& d) {
@@ -534,9 +572,9 @@ static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_vi
     const bool fast = tile_in_page(k_cache, k) && tile_in_page(v_cache, v);
 #define DA_LAUNCH(DT, GTV, FA)                                                                                   \
   do {                                                                                                          \
-    FC_ALLOW_LDS((decode_attn_kernel<DT, GTV, FA>), DaCfg<GTV>::LDS);                                         \
-    hipLaunchKernelGGL((decode_attn_kernel<DT, GTV, FA>), grid, dim3(DA_THREADS), DaCfg<GTV>::LDS, st, k, v,    \
-                       layer, (const char*)q, num_q_heads, context_lens, c, part_o, part_ml, splits);           \
+    FC_ALLOW_LDS((decode_attn_kernel<DT, GTV, FA>), DaCfg<GTV>::lds(DA_CHUNK_MAX));                             \
+    hipLaunchKernelGGL((decode_attn_kernel<DT, GTV, FA>), grid, dim3(DA_THREADS), DaCfg<GTV>::lds(chunk), st, k, \
+                       v, layer, (const char*)q, num_q_heads, context_lens, c, part_o, part_ml, splits, chunk); \
   } while (0)
 #define DA_DISPATCH2(DT, FA)                        \
   switch (gt) {                                     \
@@ -556,10 +594,10 @@ static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_vi
   dim3 mgrid(num_q_heads, B);
   if (bf)
     hipLaunchKernelGGL((decode_merge_kernel<FC_BF16>), mgrid, dim3(FC_HEAD_DIM), 0, st, part_o, part_ml, context_lens,
-                       k_cache->max_seq_len, num_q_heads, splits, (char*)out);
+                       k_cache->max_seq_len, num_q_heads, splits, chunk, (char*)out);
   else
     hipLaunchKernelGGL((decode_merge_kernel<FC_F16>), mgrid, dim3(FC_HEAD_DIM), 0, st, part_o, part_ml, context_lens,
-                       k_cache->max_seq_len, num_q_heads, splits, (char*)out);
+                       k_cache->max_seq_len, num_q_heads, splits, chunk, (char*)out);
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }
