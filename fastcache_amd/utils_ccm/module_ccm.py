@@ -29,6 +29,48 @@ def _mlp_list(n_layer: int, head_dim: int, cf: int) -> nn.ModuleList:
     return nn.ModuleList([_mlp(head_dim, cf) for _ in range(n_layer)])
 
 
+class CompressibleCache:
+    """What ``KVCacheHybridCompressor.forward`` returns for a cache object (the reference's
+    ``CompressibleCache``, utils_ccm/module_ccm_v11.py:93-127): per-layer ``key_cache`` / ``value_cache`` lists
+    plus the number of tokens the model has SEEN, which after a compression is larger than the rows the cache
+    holds and is what ``get_seq_length`` reports (positions go on from there).  A plain object with the list
+    attributes and methods the reference's class has; it does not derive from a ``transformers`` cache class,
+    whose storage differs between library versions."""
+
+    def __init__(self):
+        self.key_cache: List[torch.Tensor] = []
+        self.value_cache: List[torch.Tensor] = []
+        self._seen_tokens = -1            # < 0: never set, report the rows held
+
+    @property
+    def seen_tokens(self) -> int:
+        return self._seen_tokens
+
+    def set_seen_tokens(self, seen_tokens: int) -> None:
+        self._seen_tokens = int(seen_tokens)
+
+    def get_actual_seq_length(self, layer_idx: int = 0) -> int:
+        if layer_idx >= len(self.key_cache) or self.key_cache[layer_idx].numel() == 0:
+            return 0
+        return self.key_cache[layer_idx].shape[-2]
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        return self._seen_tokens if self._seen_tokens >= 0 else self.get_actual_seq_length(layer_idx)
+
+    def __len__(self) -> int:
+        return len(self.key_cache)
+
+    def __getitem__(self, layer_idx: int) -> LayerKV:
+        return self.key_cache[layer_idx], self.value_cache[layer_idx]
+
+    def clone(self) -> "CompressibleCache":
+        other = CompressibleCache()
+        other.key_cache = [k.clone().detach() for k in self.key_cache]
+        other.value_cache = [v.clone().detach() for v in self.value_cache]
+        other._seen_tokens = self._seen_tokens
+        return other
+
+
 class _CCMBase(nn.Module):
     """Shared machinery: stacked weight cache and the segment compressor."""
 
@@ -233,10 +275,11 @@ class KVCacheHybridCompressor(_CCMBase):
 
     @torch.no_grad()
     def forward(self, kv_cache, it_len=[1, 1], strategy_com="retain", forward_mode="val"):
-        """List input -> list output; an object with ``key_cache`` / ``value_cache`` lists (an HF cache)
-        gets those lists replaced and is returned.  ``it_len[0]`` must be 0: with an image segment long
-        enough to be compressed the reference subscripts ``None`` (module_ccm_v11.py:877-878,
-        1033-1035) and raises ``TypeError``; so does this class."""
+        """List input -> list output.  An object with ``key_cache`` / ``value_cache`` lists (an HF cache) is left
+        as it is and a new ``CompressibleCache`` comes back, holding the compressed layers and, as its seen-token
+        count, the input's ``get_seq_length()`` (module_ccm_v11.py:932-999).  ``it_len[0]`` must be 0: with an
+        image segment long enough to be compressed the reference subscripts ``None`` (:877-878, 1033-1035) and
+        raises ``TypeError``; so does this class."""
         if forward_mode == "train":
             raise NotImplementedError("inference-only build: forward_mode='train' is not supported")
         as_cache = hasattr(kv_cache, "key_cache") and hasattr(kv_cache, "value_cache")
@@ -249,9 +292,12 @@ class KVCacheHybridCompressor(_CCMBase):
         out = self._forward_split(layers, [0, 0], split=False) if it_len[0] == 0 else \
             self._forward_passthrough_image(layers, int(it_len[0]))
         if as_cache:
-            kv_cache.key_cache = [k for k, _ in out]
-            kv_cache.value_cache = [v for _, v in out]
-            return kv_cache
+            fresh = CompressibleCache()
+            fresh.key_cache = [k for k, _ in out]
+            fresh.value_cache = [v for _, v in out]
+            seen = kv_cache.get_seq_length() if hasattr(kv_cache, "get_seq_length") else layers[0][0].shape[2]
+            fresh.set_seen_tokens(seen)
+            return fresh
         return out
 
     def _paged_segments(self, seq_len: int, it_len: Sequence[int]):

@@ -12,8 +12,16 @@
  *     descriptor structs themselves (fc_kv_view, fc_mlp_weights), which are
  *     read on the host during the call and may be freed after it returns;
  *   - the call only ENQUEUES work on `stream` (a hipStream_t passed as void*;
- *     NULL = the default stream): no allocation, no synchronisation, no global
- *     state, so it may be recorded into a HIP graph;
+ *     NULL = the default stream): no allocation and no synchronisation, so it
+ *     may be recorded into a HIP graph.  What the library keeps between calls
+ *     is small and per process: the calling thread's last error text; for each
+ *     kernel that needs more than 64 KB of dynamic LDS, one bit per device
+ *     saying that its limit has been raised (hipFuncSetAttribute on the first
+ *     launch on a device; unsynchronised, setting it twice is harmless); the
+ *     compute-unit count of each device; and, for fc_decode_attn_static only,
+ *     the device address of its built-in buffer.  The first launch of a kernel
+ *     on a device therefore does host-side work: make it outside a graph
+ *     capture;
  *   - return value: FC_OK (0) or a negative FC_E* code; nothing is enqueued
  *     when an error is returned; fc_last_error() gives a message for the
  *     calling thread;

@@ -78,6 +78,20 @@ def test_hybrid_and_minicpm_modules(dev):
     out_p = h(to_dev(kv, dev), it_len=[7, S - 7])
     assert torch.equal(out_p[0][0][:, :, :7].cpu(), kv[0][0][:, :, :7])
     assert_mlp_close(out_p[0][1].cpu(), ref_p[0][1], dtype)
+    # a cache object in: a NEW CompressibleCache out, the input untouched, the seen-token count carried over
+    from fastcache_amd.utils_ccm import CompressibleCache
+    src = CompressibleCache()
+    src.key_cache, src.value_cache = [k.to(dev) for k, _ in kv], [v.to(dev) for _, v in kv]
+    src.set_seen_tokens(S + 11)                     # the model has seen more tokens than the cache holds rows
+    got = h(src, it_len=[0, S])
+    assert isinstance(got, CompressibleCache) and got is not src
+    assert src.key_cache[0].shape[2] == S and src.get_seq_length() == S + 11
+    assert got.get_seq_length() == S + 11 and got.get_actual_seq_length() == ref[0][0].shape[2] == len(got[0][0][0][0])
+    for layer in range(L):
+        assert torch.equal(got.key_cache[layer], out[layer][0]) and torch.equal(got.value_cache[layer], out[layer][1])
+    twin = got.clone()
+    assert twin.get_seq_length() == S + 11 and torch.equal(twin.key_cache[1], got.key_cache[1]) \
+        and twin.key_cache[1].data_ptr() != got.key_cache[1].data_ptr()
     # short sequences come back unchanged (min_seq_len guard)
     short = rand_kv(L, B, H, 6, dtype, seed=2)
     out_s = h(to_dev(short, dev), it_len=[0, 6])
