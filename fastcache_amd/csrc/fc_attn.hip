@@ -18,7 +18,7 @@
 
 #define DA_THREADS 256
 #define DA_CHUNK 256               // smallest chunk (tokens per workgroup); it sizes the workspace
-#define DA_CHUNK_MAX 512           // largest: the host picks a multiple of 32 in between from the launch's shape
+#define DA_CHUNK_MAX 1024          // largest: the host picks a multiple of 32 in between from the launch's shape
 #define DA_LOG2E 1.4426950408889634f
 
 template <int DTYPE>
@@ -532,26 +532,26 @@ static int da_enqueue(const char* who, const fc_kv_view* k_cache, const fc_kv_vi
   // read its K and V once per tile); groups of more than 8 heads are served 8 at a time
   const int gt = G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
   const int gtiles = (G + gt - 1) / gt;
-  // Tokens per workgroup.  A launch of many rounds of workgroups keeps the smallest chunk (best balance over
-  // ragged lengths).  A launch of a few rounds is all ramp and tail: there the chunk is the multiple of 32
-  // tokens for which the workgroups fill whole rounds of the GPU (two workgroups per compute unit), by a
-  // coarse cost of rounds * (chunk + fixed part).  Only the view's max_seq_len enters, never the lengths on the
+  // Tokens per workgroup: the multiple of 32 between 256 and 1024 that minimises rounds * (chunk + fixed part),
+  // rounds = workgroups / (two per compute unit), rounded up.  Longer chunks spend less of a workgroup's life on
+  // its ramp (first tiles in flight, nothing to compute yet) and its tail (statistics, partial results, no loads
+  // in flight); a launch of few workgroups wants the chunk that fills whole rounds.  Measured: cfg4 (2880
+  // columns, up to 2304 tokens) 0.327 ms per layer with 256, 0.297 with 512, 0.294 with 768; cfg5's decode (64
+  // columns, 3584 tokens) 33.3 us with 256, 30.4 with 448.  Two workgroups must still fit a compute unit's LDS, which
+  // caps the chunk for groups of 8 query heads.  Only the view's max_seq_len enters, never the lengths on the
   // device, so the choice is the same at capture and at every replay.
   int chunk = DA_CHUNK;
   {
     const int slots = 2 * da_compute_units();
     const long long cols = (long long)Hkv * gtiles * B;
-    const long long wgs256 = cols * ((k_cache->max_seq_len + DA_CHUNK - 1) / DA_CHUNK);
-    if (slots > 0 && wgs256 < 4LL * slots) {
-      double best = -1.0;
-      for (int cand = DA_CHUNK; cand <= DA_CHUNK_MAX; cand += DA_TILE) {
-        if (gt == 8 && DaCfg<8>::lds(cand) * 2 >= 160 * 1024) break;   // two workgroups per compute unit must fit its LDS
-        const long long wgs = cols * ((k_cache->max_seq_len + cand - 1) / cand);
-        const double cost = (double)((wgs + slots - 1) / slots) * (cand + 96.0);
-        if (best < 0 || cost < best - 1e-9) {
-          best = cost;
-          chunk = cand;
-        }
+    double best = -1.0;
+    for (int cand = DA_CHUNK; slots > 0 && cand <= DA_CHUNK_MAX; cand += DA_TILE) {
+      if ((DA_RING + gt * cand * 4) * 2 > 158 * 1024) break;
+      const long long wgs = cols * ((k_cache->max_seq_len + cand - 1) / cand);
+      const double cost = (double)((wgs + slots - 1) / slots) * (cand + 96.0);
+      if (best < 0 || cost < best - 1e-9) {
+        best = cost;
+        chunk = cand;
       }
     }
   }
