@@ -41,16 +41,23 @@ def mlp_error_stats(got, ref, dtype):
     return rel, int((err > bound).sum()), float(err.max()) / scale, err.numel()
 
 
+def mlp_outliers_allowed(n, dtype):
+    """fp16: none.  bf16: a flipped hidden activation moves a few of its row's 128 outputs past the bound at once, so
+    outliers come in clusters of 1-3; four for the odd cluster plus one per million outputs, about three times the
+    rate the CPU calibration measures (3 in 10^7)."""
+    return 0 if dtype == torch.float16 else 4 + n // 1_000_000
+
+
 def assert_mlp_close(got, ref, dtype):
     """The allowance is calibrated, not assumed: tests/test_oracle_pinning.py::test_mlp_tolerance_calibration
     evaluates the oracle MLP under other fp32 summation orders.  fp16: no element beyond the bound.  bf16: a
     hidden activation on a rounding boundary flips to the neighbouring value about 3 times in 10^7 outputs and
-    moves one output by up to 4.2e-3 of max|ref|.  Allowed here: fp16 none; bf16 one element plus two per
-    million (several times the measured rate), none further than 6.5e-3 of max|ref|."""
+    moves one or two outputs of its row by up to 4.2e-3 of max|ref|.  Allowed here: ``mlp_outliers_allowed``,
+    none further than 6.5e-3 of max|ref|."""
     rel, n_out, worst, n = mlp_error_stats(got, ref, dtype)
     OBSERVED.append((n, rel, n_out, worst))
     assert rel <= 1e-3, f"relative error norm {rel:.3e}"
-    allowed = 0 if dtype == torch.float16 else 1 + n // 500_000
+    allowed = mlp_outliers_allowed(n, dtype)
     assert n_out <= allowed, f"{n_out} of {n} elements beyond 1e-3 * max|ref| + 2 ulp ({allowed} allowed)"
     assert worst <= 6.5e-3, f"max error {worst:.3e} of max|ref|"
 

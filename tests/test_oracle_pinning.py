@@ -677,9 +677,11 @@ def test_mlp_tolerance_calibration():
     comparisons of 1000 rows as the GPU tests make them.  fp16: no element beyond ``1e-3 * max|ref| + 2 ulp``.
     bf16: a few per 10^7 (a hidden activation that rounds to the neighbouring bf16 value), each within 5e-3 of
     max|ref|.  Measured over 15 M elements per case: 5, 5 and 2 outliers for cf 1, 2, 5 in bf16 (worst 4.2e-3),
-    none in fp16 (worst 5.6e-4).  ``assert_mlp_close`` allows 1 + 2 per million in bf16 and none in fp16."""
+    none in fp16 (worst 5.6e-4); a flip moves one or two outputs of its row, so they come in small clusters (450
+    comparisons of 64 000 outputs: 441 with none, up to 9 with one, up to 2 with two).  ``assert_mlp_close`` allows
+    4 + 1 per million in bf16 and none in fp16."""
     import torch.nn.functional as F
-    from test_gpu_ccm import mlp_error_stats
+    from test_gpu_ccm import mlp_error_stats, mlp_outliers_allowed
 
     def mlp3_order(x, sd, order):
         dt = x.dtype
@@ -719,4 +721,4 @@ def test_mlp_tolerance_calibration():
         if dtype == torch.float16:
             assert outliers == 0, (cf, outliers)
         else:
-            assert outliers <= 1 + total // 500_000, (cf, outliers, total)
+            assert outliers <= mlp_outliers_allowed(total, dtype), (cf, outliers, total)
