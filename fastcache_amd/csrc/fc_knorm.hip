@@ -4,44 +4,11 @@
 // A token-head row is 128 elements = 512 B (fp32) or 256 B (fp16/bf16): it is read by 32 or 16
 // lanes with one 16-byte load each, squared and reduced across those lanes in fp32.  The tile's
 // scores are staged in LDS so that each head's TS scores leave as one contiguous segment.
-#include "fc_common.h"
+#include "fc_norm.h"
 
 #define KN_TS 16   // tokens per workgroup tile: small enough that short caches still give thousands of workgroups
 #define KN_THREADS 256
 #define KN_U 4     // rows per lane and pass
-
-// sum of squares of the 16 bytes a lane holds of its row
-template <int DTYPE>
-__device__ __forceinline__ float row_sumsq_part(const uint4& x) {
-  if (DTYPE == FC_F32) {
-    const float a = __uint_as_float(x.x), b = __uint_as_float(x.y), c = __uint_as_float(x.z), d = __uint_as_float(x.w);
-    return a * a + b * b + c * c + d * d;
-  } else {
-    unsigned w[4] = {x.x, x.y, x.z, x.w};
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float lo, hi;
-      if (DTYPE == FC_BF16) {
-        lo = fc_bf16_to_float((unsigned short)(w[i] & 0xffff));
-        hi = fc_bf16_to_float((unsigned short)(w[i] >> 16));
-      } else {
-        lo = fc_half_to_float((unsigned short)(w[i] & 0xffff));
-        hi = fc_half_to_float((unsigned short)(w[i] >> 16));
-      }
-      acc += lo * lo;
-      acc += hi * hi;
-    }
-    return acc;
-  }
-}
-
-template <int DTYPE>
-__device__ __forceinline__ float round_to_storage(float x) {
-  if (DTYPE == FC_BF16) return fc_bf16_to_float(fc_float_to_bf16(x));
-  if (DTYPE == FC_F16) return fc_half_to_float(fc_float_to_half(x));
-  return x;
-}
 
 // MEAN == false: scores[l][b][h][s] = -norm.   MEAN == true: out[l][b][s] = mean_h norm, with the
 // per-head norm and the mean each rounded to the storage dtype (torch's keys.norm().mean(1)).

@@ -7,19 +7,11 @@
 // needed.  A final ordered pass keeps every key > T plus the first `need` keys == T in index
 // order, using wavefront ballots for the running ranks, so the output is ascending and
 // deterministic.  Rows too long for LDS are re-read from global memory (L2-resident).
-#include "fc_common.h"
+#include "fc_select.h"
 
-#define TK_BINS 256
 #define TK_LDS_MAX_KEYS 15360        // 60 KiB of keys: several workgroups of 256 threads per CU
 #define TK_LONG_ROW 8192             // rows longer than this take 1024 threads
 #define TK_LDS_MAX_KEYS_LONG 36864   // 144 KiB of keys: one workgroup of 1024 threads per CU
-
-__device__ __forceinline__ unsigned tk_key(float f) {
-  unsigned u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;  // NaN ranks above +inf
-  if ((u & 0x7fffffffu) == 0u) u = 0u;                      // -0 == +0
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
 
 template <bool LDS_KEYS, int TK_THREADS>
 __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restrict__ scores,
@@ -28,15 +20,11 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
                                                           int rows_per_len, int row_lens_mod, int k,
                                                           const int* __restrict__ n_kept,
                                                           int* __restrict__ indices, int index_stride) {
-  constexpr int TK_WAVES = TK_THREADS / FC_WAVE;
   extern __shared__ __align__(16) unsigned lds_keys[];
-  __shared__ unsigned hist[TK_BINS];
-  __shared__ unsigned wave_tot[TK_BINS / FC_WAVE];
-  __shared__ unsigned sel_bin, sel_remaining;
-  __shared__ unsigned w_eq[TK_WAVES], w_gt[TK_WAVES];
+  __shared__ TkShared<TK_THREADS> sh;
 
   const int r = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x;
   const int li = (row_lens || n_kept) ? (r / rows_per_len) % row_lens_mod : 0;
   int n = row_lens ? row_lens[li] : len;
   if (n > len) n = len;
@@ -75,101 +63,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float* __restric
   }
   auto key_at = [&](int i) -> unsigned { return LDS_KEYS ? lds_keys[i] : tk_key(row[i]); };
 
-  unsigned prefix = 0, mask = 0, remaining = (unsigned)kk;
-  for (int shift = 24; shift >= 0; shift -= 8) {
-    if (tid < TK_BINS) hist[tid] = 0;
-    __syncthreads();
-    for (int i0 = 0; i0 < n; i0 += TK_THREADS) {
-      const int i = i0 + tid;
-      const unsigned u = i < n ? key_at(i) : 0u;
-      bool todo = i < n && (u & mask) == prefix;
-      const unsigned bin = (u >> shift) & 255u;
-      // Scores of one row share their leading bits, so most lanes of a wavefront hit the same bin in the
-      // first passes and their atomics would serialise: the two most common bins are counted with a
-      // ballot and one atomic each, what is left goes through per-lane atomics.
-#pragma unroll
-      for (int rep = 0; rep < 2; ++rep) {
-        const unsigned long long act = __ballot(todo);
-        if (act == 0ull) break;
-        const int leader = __ffsll((long long)act) - 1;
-        const unsigned lb = __shfl(bin, leader, 64);
-        const unsigned long long same = __ballot(todo && bin == lb);
-        if (lane == leader) atomicAdd(&hist[lb], (unsigned)__popcll(same));
-        todo = todo && bin != lb;
-      }
-      if (todo) atomicAdd(&hist[bin], 1u);
-    }
-    __syncthreads();
-    // suffix sums over bins: thread t < 256 owns bin 255 - t
-    unsigned h = 0, incl = 0;
-    if (tid < TK_BINS) {
-      h = hist[TK_BINS - 1 - tid];
-      incl = h;
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        unsigned up = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += up;
-      }
-      if (lane == 63) wave_tot[wave] = incl;
-    }
-    __syncthreads();
-    if (tid < TK_BINS) {
-      unsigned base = 0;
-      for (int w = 0; w < wave; ++w) base += wave_tot[w];
-      incl += base;
-      const unsigned excl = incl - h;  // elements in strictly larger bins
-      if (excl < remaining && remaining <= incl) {
-        sel_bin = (unsigned)(TK_BINS - 1 - tid);
-        sel_remaining = remaining - excl;
-      }
-    }
-    __syncthreads();
-    prefix |= sel_bin << shift;
-    mask |= 255u << shift;
-    remaining = sel_remaining;
-    __syncthreads();
-  }
-  const unsigned T = prefix;
-  const unsigned need = remaining;  // how many keys == T to keep (>= 1)
-
-  // each wave owns a contiguous segment, walked 64 keys at a time
-  const int seg = (((n + TK_WAVES - 1) / TK_WAVES) + 63) & ~63;
-  const int beg = wave * seg;
-  const int end = min(n, beg + seg);
-  unsigned eq_cnt = 0, gt_cnt = 0;
-  for (int i0 = beg; i0 < end; i0 += 64) {
-    int i = i0 + lane;
-    unsigned u = (i < end) ? key_at(i) : 0u;
-    bool live = i < end;
-    eq_cnt += __popcll(__ballot(live && u == T));
-    gt_cnt += __popcll(__ballot(live && u > T));
-  }
-  if (lane == 0) { w_eq[wave] = eq_cnt; w_gt[wave] = gt_cnt; }
-  __syncthreads();
-  unsigned eq_seen = 0, out_pos = 0;
-  {
-    unsigned eq_run = 0;
-    for (int w = 0; w < wave; ++w) {
-      unsigned take = need > eq_run ? min(need - eq_run, w_eq[w]) : 0u;
-      out_pos += w_gt[w] + take;
-      eq_run += w_eq[w];
-    }
-    eq_seen = eq_run;
-  }
-  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  for (int i0 = beg; i0 < end; i0 += 64) {
-    int i = i0 + lane;
-    bool live = i < end;
-    unsigned u = live ? key_at(i) : 0u;
-    bool is_eq = live && u == T;
-    unsigned long long eqb = __ballot(is_eq);
-    unsigned my_rank = eq_seen + __popcll(eqb & lt_mask);
-    bool sel = live && (u > T || (is_eq && my_rank < need));
-    unsigned long long sb = __ballot(sel);
-    if (sel) out[out_pos + __popcll(sb & lt_mask)] = i;
-    eq_seen += __popcll(eqb);
-    out_pos += __popcll(sb);
-  }
+  tk_select_row<TK_THREADS>(sh, key_at, n, kk, [&](int pos, int i) { out[pos] = i; });
 }
 
 extern "C" int fc_topk_select(const float* scores, int32_t score_stride, int32_t rows, int32_t len,

@@ -195,6 +195,27 @@ def compact(src_k: FcKvView, src_v: FcKvView, dst_k: FcKvView, dst_v: FcKvView, 
           "fc_compact")
 
 
+KNORM_PRESS_MAX_SEQ = 8192      # longest sequence the one-launch Knorm press takes
+
+
+def knorm_press(keys: FcKvView, values: FcKvView, k: int, device, n_kept: Optional[torch.Tensor] = None,
+                ragged: bool = False):
+    """Knorm scores, top-``k`` (or ``n_kept[b]``) per (layer, sequence, kv head) row and in-place compaction of
+    both planes in one launch; returns ``(scores [L, B, Hkv, max_seq_len] fp32, indices [L, B, Hkv, k] int32)`` equal
+    to ``knorm_score`` + ``topk_select`` + ``compact``.  With ``n_kept`` or ``ragged`` (sequences that may hold fewer
+    than ``k`` tokens) index entries past a row's kept count are -1."""
+    L, B, H, S = keys.num_layers, keys.batch, keys.num_kv_heads, keys.max_seq_len
+    scores = torch.empty((L, B, H, S), dtype=torch.float32, device=device)
+    n_kept = _i32(n_kept, "n_kept", device)
+    if n_kept is not None or ragged:
+        idx = torch.full((L, B, H, k), -1, dtype=torch.int32, device=device)
+    else:
+        idx = torch.empty((L, B, H, k), dtype=torch.int32, device=device)
+    check(fn("fc_knorm_press")(C.byref(keys), C.byref(values), scores.data_ptr(), S, k, ptr(n_kept), idx.data_ptr(), k,
+                               current_stream()), "fc_knorm_press")
+    return scores, idx
+
+
 def copy_tokens(src: FcKvView, dst: FcKvView, seg_start: int, count: int, dst_start: int) -> None:
     check(fn("fc_copy_tokens")(C.byref(src), C.byref(dst), seg_start, count, dst_start, current_stream()),
           "fc_copy_tokens")

@@ -59,9 +59,18 @@ def knorm_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, seq
     Python ints, ``seq_len`` their maximum), over sequences of different lengths in the same launches: each keeps
     ``int(its length * (1 - compression_ratio))`` tokens."""
     kview, vview = _views(kv_cache, block_tables, seq_lens, seq_len)
-    scores = ops.knorm_score(kview, kv_cache.device)
     lens = list(host_lens) if host_lens is not None else [seq_len] * block_tables.shape[0]
     kept = [n_kept_for(n, compression_ratio) for n in lens]
+    width = max(kept)
+    if compact and 0 < width and seq_len <= ops.KNORM_PRESS_MAX_SEQ:
+        # one launch: every (layer, sequence, head) column is scored, selected and compacted by one workgroup
+        if len(set(kept)) == 1:
+            scores, idx = ops.knorm_press(kview, vview, width, kv_cache.device)
+            return PressResult(idx, width, scores)
+        n_kept = torch.tensor(kept, dtype=torch.int32, device=kv_cache.device)
+        scores, idx = ops.knorm_press(kview, vview, width, kv_cache.device, n_kept=n_kept)
+        return PressResult(idx, width, scores, list(kept))
+    scores = ops.knorm_score(kview, kv_cache.device)
     return _select_and_compact(kview, vview, scores, seq_lens, kept, compact, kv_cache.shape[4])
 
 

@@ -175,6 +175,19 @@ int fc_topk_select(const float* scores, int32_t score_stride, int32_t rows, int3
                    int32_t* indices, int32_t index_stride, void* stream);
 
 /*
+ * Knorm press in one launch: fc_knorm_score, fc_topk_select (rows of one sequence keep n_kept[b] of their
+ * seq_lens[b] scores, or `k` when n_kept is NULL) and fc_compact of `keys` and `values` onto themselves, for every
+ * (layer, b, kv head) column, with the same scores, indices (entries past a row's kept count are left as they are)
+ * and cache bytes as those three calls.  Sequences of up to 8192 tokens; longer views are refused with
+ * FC_EUNSUPPORTED and take the three calls.
+ * Replaces, for KnormPress, the per-sequence loop extract -> press -> write back of
+ * LlavaModelRunner.compress_kv_cache_batch (nanovllm/engine/llava_model_runner.py:745-786) with
+ * kvpress KnormPress.score + ScorerPress.compress (third-party) inside.
+ */
+int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, float* scores, int32_t score_stride, int32_t k,
+                   const int32_t* n_kept, int32_t* indices, int32_t index_stride, void* stream);
+
+/*
  * Gather + compaction.  For each (layer, b, kv head): dst token j <- src token
  * indices[(l*batch + b)*heads_in_index + (h % heads_in_index)][j] for j < n_kept[b] (or k).
  * `dst` may alias `src` (same pool, same tables): indices must then be ascending, and the

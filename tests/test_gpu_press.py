@@ -72,6 +72,77 @@ def test_knorm_press_paged_inplace(dev, dtype, shape):
         assert torch.equal(pool.cpu().view(torch.uint8), ref_pool.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lens,block_size,keep", [
+    ([700, 512, 1], 256, [350, 256, 0]),          # ragged, a sequence that keeps nothing
+    ([1024], 256, [512]),                         # the shape of the first configuration, one sequence
+    ([300, 300], 64, [300, 299]),                 # keep everything / all but one
+    ([2500, 130, 2049], 128, [1, 129, 700]),      # several pages, a single kept row
+    ([193, 77], 48, [100, 33]),                   # pages whose size is not a power of two
+])
+def test_knorm_press_one_launch_equals_three(dev, dtype, lens, block_size, keep):
+    """fc_knorm_press against fc_knorm_score + fc_topk_select + fc_compact on the same pool: scores, indices and
+    every byte of both planes identical (ties included: both run the same selection)."""
+    case = synth.make_paged_case(seed=11, num_layers=2, batch=len(lens), num_kv_heads=3, seq_lens=lens, dtype=dtype,
+                                 outlier_channels=4, block_size=block_size)
+    # equal rows inside a column: ties that the selection has to break by position
+    pool_a = case.kv_cache.to(dev)
+    t0 = case.block_tables[0]
+    pool_a[0, :, t0[0], 5] = pool_a[0, :, t0[0], 2]
+    pool_a[0, :, t0[0], 9] = pool_a[0, :, t0[0], 2]
+    pool_b = pool_a.clone()
+    tables, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+    S, width = max(lens), max(keep)
+    n_kept = torch.tensor(keep, dtype=torch.int32, device=dev)
+
+    ka, va = (_lib.paged_view(pool_a[p], tables, lens_d, S) for p in range(2))
+    scores_a = ops.knorm_score(ka, dev)
+    idx_a = ops.topk_select(scores_a, width, row_lens=lens_d, n_kept=n_kept, rows_per_len=3)
+    ops.compact(ka, va, ka, va, idx_a, n_kept=n_kept)
+
+    kb, vb = (_lib.paged_view(pool_b[p], tables, lens_d, S) for p in range(2))
+    scores_b, idx_b = ops.knorm_press(kb, vb, width, dev, n_kept=n_kept)
+    torch.cuda.synchronize()
+    assert torch.equal(scores_a.view(torch.int32), scores_b.view(torch.int32))
+    assert torch.equal(idx_a, idx_b)
+    assert torch.equal(pool_a.view(torch.uint8), pool_b.view(torch.uint8))
+    # and something did move
+    assert not torch.equal(pool_b.view(torch.uint8), case.kv_cache.to(dev).view(torch.uint8)) or width == 0
+
+
+def test_knorm_press_one_launch_limits_and_clamps(dev):
+    """Sequences beyond 8192 tokens are refused by name; a kept count in device memory larger than the sequence or
+    the index row is clamped; a dense view works like a paged one."""
+    L, B, H, S = 1, 2, 2, 96
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn((L, B, H, S, 128), generator=g).to(dev)
+    v = torch.randn((L, B, H, S, 128), generator=g).to(dev)
+    k2, v2 = k.clone(), v.clone()
+    n_kept = torch.tensor([10_000, 40], dtype=torch.int32, device=dev)      # first one far too large
+    lens_d = torch.tensor([S, 50], dtype=torch.int32, device=dev)
+    def views(kt, vt):
+        out = (_lib.dense_view(kt), _lib.dense_view(vt))
+        for view in out:
+            view.seq_lens = lens_d.data_ptr()
+        return out
+    ka, va = views(k, v)
+    sa = ops.knorm_score(ka, dev)
+    ia = ops.topk_select(sa, 64, row_lens=lens_d, n_kept=n_kept, rows_per_len=H)
+    ops.compact(ka, va, ka, va, ia, n_kept=n_kept)
+    kb, vb = views(k2, v2)
+    sb, ib = ops.knorm_press(kb, vb, 64, dev, n_kept=n_kept)
+    torch.cuda.synchronize()
+    assert torch.equal(sa.view(torch.int32), sb.view(torch.int32)) and torch.equal(ia, ib)
+    assert torch.equal(k, k2) and torch.equal(v, v2)
+    row = ib[0, 0, 0]                                                        # 10 000 asked for: clamped to the 64 of the row
+    assert (row >= 0).all() and (row < S).all() and (row[1:] > row[:-1]).all()
+    row = ib[0, 1, 1]
+    assert (row[:40] >= 0).all() and (row[:40] < 50).all() and (row[40:] == -1).all()
+    big = torch.zeros((1, 1, 1, 8200, 128), device=dev)
+    with pytest.raises(_lib.FastcacheError, match="8192"):
+        ops.knorm_press(_lib.dense_view(big), _lib.dense_view(big.clone()), 10, dev)
+
+
 def _oracle_snapkv_scores(case, W, ksz, causal, reduction):
     """[L, B, Hkv, S] fp32 scores from the dense K of every sequence (all sequences share S)."""
     out = []
