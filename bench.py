@@ -148,6 +148,7 @@ class SnapKVWorkload(Workload):
     name = "cfg2-snapkv-qwen3-8b"
     dtype_name = "bf16"
     kernel_name = "snapkv_kernel"
+    separate_selection = False     # True: fc_topk_select and fc_compact as two launches (sequences beyond 8192 tokens)
 
     def __init__(self, seed, device, given_lse=False):
         super().__init__()
@@ -218,8 +219,11 @@ class SnapKVWorkload(Workload):
         # the window fill needs every row maximum of the layer, so it is its own (small) launch
         check(fn("fc_snapkv_fill_window")(scores.data_ptr(), S, L, B, Hkv, self.lens.data_ptr(), S, self.W,
                                           row_max.data_ptr(), st), "fc_snapkv_fill_window")
-        idx = ops.topk_select(scores, self.n_kept)
-        ops.compact(kview, vview, kview, vview, idx)
+        if self.separate_selection:
+            idx = ops.topk_select(scores, self.n_kept)
+            ops.compact(kview, vview, kview, vview, idx)
+        else:                                    # what paged_press.snapkv_compress_paged issues
+            idx = ops.select_compact(kview, vview, scores, self.n_kept)
         if self.keep:
             self.kept, self.keep = (scores, idx), False
 
@@ -602,10 +606,18 @@ class CopyWorkload(Workload):
                 "sample": "torch clone of 1 of 4 sequences on the host"}
 
 
+def _separate(w):
+    w.separate_selection = True
+    w.name += "-separate-selection"
+    return w
+
+
 WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkload, "knorm-3": KnormThreeLaunchWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
              "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True),
              # cfg2 with the window queries' log-sum-exp handed in (not the BASELINE metric: the reference has no such input)
              "snapkv-lse": lambda seed, dev: SnapKVWorkload(seed, dev, given_lse=True),
+             # cfg2 with selection and compaction as two launches
+             "snapkv-sep": lambda seed, dev: _separate(SnapKVWorkload(seed, dev)),
              # the decode launches without a graph, 4 steps per bracket: rocprofv3 cannot walk the 128-step graph
              "decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True),
              # the 64 decode steps that follow the compression in configuration 5, in one graph

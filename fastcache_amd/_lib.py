@@ -69,6 +69,7 @@ SIGNATURES = {
     "fc_topk_select": (C.c_int, [_VP, _I, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _VP]),
     "fc_compact": (C.c_int, [_V, _V, _V, _V, _VP, _I, _I, _I, _VP, _VP]),
     "fc_knorm_press": (C.c_int, [_V, _V, _VP, _I, _I, _VP, _VP, _I, _VP]),
+    "fc_select_compact": (C.c_int, [_V, _V, _VP, _I, _I, _VP, _VP, _I, _VP]),
     "fc_ccm_mlp": (C.c_int, [_V, _V, C.POINTER(FcMlpWeights), _I, _I, _I, _I, _VP]),
     "fc_ccm_mlp_ragged": (C.c_int, [_V, _V, C.POINTER(FcMlpWeights), _I, _VP, _VP, _VP, _I, _I, _VP]),
     "fc_linear_act": (C.c_int, [_VP, C.c_int64, _VP, _VP, _VP, C.c_int64, C.c_int64, _I, _I, _I, _I, _VP]),

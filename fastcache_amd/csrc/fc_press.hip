@@ -15,6 +15,47 @@
 #define KP_U 4          // key rows per lane in flight while scoring
 #define KP_WIDE_FROM 512   // sequences from this length on get 1024 threads per column, shorter ones 256
 
+// What both kernels of this file end with: the kk best of the column's S scores in LDS (0 < kk <= S, clamped by the
+// caller), their positions to the index row and to LDS, and the kept K and V rows moved to the front of the column.
+template <int EB, int THREADS>
+__device__ __forceinline__ void kp_select_and_move(const KvView& kv, const KvView& vv, const int* ktbl, bool k_lds,
+                                                   const int* vtbl, bool v_lds, const float* sc, int* sel,
+                                                   TkShared<THREADS>& sh, int l, int b, int h, int S, int kk,
+                                                   int* __restrict__ idx_row) {
+  const int tid = threadIdx.x, sub = tid % (FC_HEAD_DIM * EB / 16);
+  if (kk == S) {   // everything stays where it is
+    for (int i = tid; i < S; i += THREADS) idx_row[i] = i;
+    return;
+  }
+  tk_select_row<THREADS>(sh, [&](int i) { return tk_key(sc[i]); }, S, kk, [&](int pos, int i) {
+    idx_row[pos] = i;
+    sel[pos] = i;
+  });
+  __syncthreads();
+  // compaction in place: row j <- row sel[j], K then V
+  char* kbase = kv.base + ((long long)l * kv.stride_layer + (long long)h * kv.stride_head) * EB + sub * 16;
+  cp_walk<EB, 1, THREADS>(kv, kv, ktbl, k_lds, ktbl, k_lds, b, S, kk, kbase, kbase, kv.base + sub * 16, 0,
+                          [&](int j) { return sel[j]; });
+  char* vbase = vv.base + ((long long)l * vv.stride_layer + (long long)h * vv.stride_head) * EB + sub * 16;
+  cp_walk<EB, 1, THREADS>(vv, vv, vtbl, v_lds, vtbl, v_lds, b, S, kk, vbase, vbase, vv.base + sub * 16, 0,
+                          [&](int j) { return sel[j]; });
+}
+
+// the sequence's block-table rows of both views into LDS (when they fit); the caller synchronises
+template <int THREADS>
+__device__ __forceinline__ void kp_tables(const KvView& kv, const KvView& vv, int* ktbl, int* vtbl, int b, int S,
+                                          bool& k_lds, bool& v_lds) {
+  const int tid = threadIdx.x;
+  const int nblk_k = kv.block_shift >= 0 ? ((S - 1) >> kv.block_shift) + 1 : 0;
+  const int nblk_v = vv.block_shift >= 0 ? ((S - 1) >> vv.block_shift) + 1 : 0;
+  k_lds = kv.block_tables && kv.block_shift >= 0 && nblk_k <= CP_TBL;
+  v_lds = vv.block_tables && vv.block_shift >= 0 && nblk_v <= CP_TBL;
+  if (k_lds)
+    for (int i = tid; i < nblk_k; i += THREADS) ktbl[i] = kv.block_tables[(long long)b * kv.table_stride + i];
+  if (v_lds)
+    for (int i = tid; i < nblk_v; i += THREADS) vtbl[i] = vv.block_tables[(long long)b * vv.table_stride + i];
+}
+
 template <int DTYPE, int THREADS>
 __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView vv, float* __restrict__ scores,
                                                               int score_stride, int k, const int* __restrict__ n_kept,
@@ -38,14 +79,8 @@ __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView 
   for (int s = S + tid; s < score_stride; s += THREADS) out_row[s] = -INFINITY;
   if (S <= 0) return;
 
-  const int nblk_k = kv.block_shift >= 0 ? ((S - 1) >> kv.block_shift) + 1 : 0;
-  const int nblk_v = vv.block_shift >= 0 ? ((S - 1) >> vv.block_shift) + 1 : 0;
-  const bool k_lds = kv.block_tables && kv.block_shift >= 0 && nblk_k <= CP_TBL;
-  const bool v_lds = vv.block_tables && vv.block_shift >= 0 && nblk_v <= CP_TBL;
-  if (k_lds)
-    for (int i = tid; i < nblk_k; i += THREADS) ktbl[i] = kv.block_tables[(long long)b * kv.table_stride + i];
-  if (v_lds)
-    for (int i = tid; i < nblk_v; i += THREADS) vtbl[i] = vv.block_tables[(long long)b * vv.table_stride + i];
+  bool k_lds, v_lds;
+  kp_tables<THREADS>(kv, vv, ktbl, vtbl, b, S, k_lds, v_lds);
   __syncthreads();
 
   // ---- norms: KP_U rows per lane and pass, all loads issued before the first is reduced --------------------
@@ -76,27 +111,45 @@ __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView 
   int kk = n_kept ? n_kept[b] : k;
   kk = min(min(kk, S), index_stride);
   if (kk <= 0) return;
-  if (kk == S) {   // everything stays where it is
-    for (int i = tid; i < S; i += THREADS) idx_row[i] = i;
-    return;
-  }
-  tk_select_row<THREADS>(sh, [&](int i) { return tk_key(sc[i]); }, S, kk, [&](int pos, int i) {
-    idx_row[pos] = i;
-    sel[pos] = i;
-  });
-  __syncthreads();
-
-  // ---- compaction in place: row j <- row sel[j], K then V -----------------------------------------------------
-  cp_walk<EB, 1, THREADS>(kv, kv, ktbl, k_lds, ktbl, k_lds, b, S, kk, kbase, kbase, kv.base + sub * 16, 0,
-                          [&](int j) { return sel[j]; });
-  char* vbase = vv.base + ((long long)l * vv.stride_layer + (long long)h * vv.stride_head) * EB + sub * 16;
-  cp_walk<EB, 1, THREADS>(vv, vv, vtbl, v_lds, vtbl, v_lds, b, S, kk, vbase, vbase, vv.base + sub * 16, 0,
-                          [&](int j) { return sel[j]; });
+  kp_select_and_move<EB, THREADS>(kv, vv, ktbl, k_lds, vtbl, v_lds, sc, sel, sh, l, b, h, S, kk, idx_row);
 }
 
-extern "C" int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, float* scores, int32_t score_stride,
-                              int32_t k, const int32_t* n_kept, int32_t* indices, int32_t index_stride, void* stream) {
-  const char* who = "fc_knorm_press";
+// Selection and compaction of a column from scores that another kernel wrote (any press whose scores are per
+// (layer, sequence, kv head, token)): fc_topk_select and fc_compact of a cache onto itself in one launch.
+template <int EB, int THREADS>
+__global__ __launch_bounds__(THREADS) void select_compact_kernel(KvView kv, KvView vv, const float* __restrict__ scores,
+                                                                 int score_stride, int k,
+                                                                 const int* __restrict__ n_kept,
+                                                                 int* __restrict__ indices, int index_stride, int smax) {
+  extern __shared__ __align__(16) float sc[];  // [smax] scores of the column, then the kept positions
+  int* sel = reinterpret_cast<int*>(sc + smax);
+  __shared__ int ktbl[CP_TBL], vtbl[CP_TBL];
+  __shared__ TkShared<THREADS> sh;
+  const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int S = min(fc_seq_len(kv, b), smax);
+  int kk = n_kept ? n_kept[b] : k;
+  kk = min(min(kk, S), index_stride);
+  if (kk <= 0) return;
+  const long long row_id = ((long long)l * kv.batch + b) * kv.num_kv_heads + h;
+  const float* row = scores + row_id * score_stride;
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const float4* row4 = reinterpret_cast<const float4*>(row);
+    float4* sc4 = reinterpret_cast<float4*>(sc);
+    for (int i = tid; i < (S >> 2); i += THREADS) sc4[i] = row4[i];
+    for (int i = (S & ~3) + tid; i < S; i += THREADS) sc[i] = row[i];
+  } else {
+    for (int i = tid; i < S; i += THREADS) sc[i] = row[i];
+  }
+  bool k_lds, v_lds;
+  kp_tables<THREADS>(kv, vv, ktbl, vtbl, b, S, k_lds, v_lds);
+  __syncthreads();
+  kp_select_and_move<EB, THREADS>(kv, vv, ktbl, k_lds, vtbl, v_lds, sc, sel, sh, l, b, h, S, kk,
+                                  indices + row_id * index_stride);
+}
+
+static int kp_check(const char* who, const fc_kv_view* keys, const fc_kv_view* values, const void* scores,
+                    int32_t score_stride, int32_t k, const int32_t* n_kept, const void* indices, int32_t index_stride) {
   int rc;
   if ((rc = fc_check_view(keys, who)) || (rc = fc_check_view(values, who))) return rc;
   FC_REQUIRE(keys->dtype == values->dtype && keys->num_layers == values->num_layers && keys->batch == values->batch &&
@@ -110,9 +163,17 @@ extern "C" int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, 
   FC_REQUIRE(n_kept != nullptr || (k >= 0 && k <= index_stride), FC_EINVAL, "%s: k=%d vs index_stride=%d", who, k,
              index_stride);
   FC_REQUIRE(keys->max_seq_len <= KP_MAX_S, FC_EUNSUPPORTED,
-             "%s: sequences of up to %d tokens (got %d); longer ones take fc_knorm_score, fc_topk_select and fc_compact",
-             who, KP_MAX_S, keys->max_seq_len);
+             "%s: sequences of up to %d tokens (got %d); longer ones take fc_topk_select and fc_compact", who, KP_MAX_S,
+             keys->max_seq_len);
   FC_REQUIRE(keys->batch <= 65535 && keys->num_layers <= 65535, FC_EUNSUPPORTED, "%s: grid too large", who);
+  return FC_OK;
+}
+
+extern "C" int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, float* scores, int32_t score_stride,
+                              int32_t k, const int32_t* n_kept, int32_t* indices, int32_t index_stride, void* stream) {
+  const char* who = "fc_knorm_press";
+  int rc = kp_check(who, keys, values, scores, score_stride, k, n_kept, indices, index_stride);
+  if (rc) return rc;
   if (keys->max_seq_len == 0 || score_stride == 0) return FC_OK;
   KvView kv = fc_make_view(keys), vv = fc_make_view(values);
   const int smax = keys->max_seq_len;
@@ -135,6 +196,34 @@ extern "C" int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, 
     default: KP_DISPATCH(FC_BF16); break;
   }
 #undef KP_DISPATCH
+#undef KP_LAUNCH
+  FC_CHECK_LAUNCH(who);
+  return FC_OK;
+}
+
+extern "C" int fc_select_compact(const fc_kv_view* keys, const fc_kv_view* values, const float* scores,
+                                 int32_t score_stride, int32_t k, const int32_t* n_kept, int32_t* indices,
+                                 int32_t index_stride, void* stream) {
+  const char* who = "fc_select_compact";
+  int rc = kp_check(who, keys, values, scores, score_stride, k, n_kept, indices, index_stride);
+  if (rc) return rc;
+  if (keys->max_seq_len == 0 || (!n_kept && k == 0)) return FC_OK;
+  KvView kv = fc_make_view(keys), vv = fc_make_view(values);
+  const int smax = keys->max_seq_len;
+  const size_t lds = ((size_t)smax + (size_t)index_stride) * 4;
+  dim3 grid(keys->num_kv_heads, keys->batch, keys->num_layers);
+  hipStream_t st = (hipStream_t)stream;
+#define KP_LAUNCH(E, TH)                                                                                          \
+  do {                                                                                                           \
+    FC_ALLOW_LDS((select_compact_kernel<E, TH>), KP_MAX_S * 8);                                                   \
+    hipLaunchKernelGGL((select_compact_kernel<E, TH>), grid, dim3(TH), lds, st, kv, vv, scores, score_stride, k, \
+                       n_kept, indices, index_stride, smax);                                                     \
+  } while (0)
+  if (keys->dtype == FC_F32) {
+    if (smax >= KP_WIDE_FROM) KP_LAUNCH(4, 1024); else KP_LAUNCH(4, 256);
+  } else {
+    if (smax >= KP_WIDE_FROM) KP_LAUNCH(2, 1024); else KP_LAUNCH(2, 256);
+  }
 #undef KP_LAUNCH
   FC_CHECK_LAUNCH(who);
   return FC_OK;

@@ -216,6 +216,26 @@ def knorm_press(keys: FcKvView, values: FcKvView, k: int, device, n_kept: Option
     return scores, idx
 
 
+def select_compact(keys: FcKvView, values: FcKvView, scores: torch.Tensor, k: int,
+                   n_kept: Optional[torch.Tensor] = None, ragged: bool = False) -> torch.Tensor:
+    """``topk_select`` over each sequence's own length and ``compact`` of both planes onto themselves in one launch;
+    ``scores`` fp32 ``[L, B, Hkv, stride]`` contiguous.  Returns the indices ``[L, B, Hkv, k]`` (-1 past a row's kept
+    count with ``n_kept`` or ``ragged``)."""
+    _lib.require_gpu(scores, "scores")
+    L, B, H = keys.num_layers, keys.batch, keys.num_kv_heads
+    if scores.dtype != torch.float32 or scores.dim() != 4 or tuple(scores.shape[:3]) != (L, B, H) or \
+            not scores.is_contiguous():
+        raise FastcacheError("scores must be a contiguous fp32 [L, B, Hkv, stride] tensor matching the views")
+    n_kept = _i32(n_kept, "n_kept", scores.device)
+    if n_kept is not None or ragged:
+        idx = torch.full((L, B, H, k), -1, dtype=torch.int32, device=scores.device)
+    else:
+        idx = torch.empty((L, B, H, k), dtype=torch.int32, device=scores.device)
+    check(fn("fc_select_compact")(C.byref(keys), C.byref(values), scores.data_ptr(), scores.shape[3], k, ptr(n_kept),
+                                  idx.data_ptr(), k, current_stream()), "fc_select_compact")
+    return idx
+
+
 def copy_tokens(src: FcKvView, dst: FcKvView, seg_start: int, count: int, dst_start: int) -> None:
     check(fn("fc_copy_tokens")(C.byref(src), C.byref(dst), seg_start, count, dst_start, current_stream()),
           "fc_copy_tokens")

@@ -40,6 +40,13 @@ def _select_and_compact(kview, vview, scores, seq_lens, kept: List[int], compact
     """Top-k per (layer, sequence, head) row and in-place compaction; one launch each whether or not the
     sequences keep the same number of tokens."""
     width = max(kept)
+    one_launch = (compact and width > 0 and kview.max_seq_len <= ops.KNORM_PRESS_MAX_SEQ and scores.dim() == 4 and
+                  scores.shape[2] == kview.num_kv_heads and scores.is_contiguous())
+    if one_launch:       # selection and compaction of a column by one workgroup
+        if len(set(kept)) == 1:
+            return PressResult(ops.select_compact(kview, vview, scores, width), width, scores)
+        n_kept = torch.tensor(kept, dtype=torch.int32, device=scores.device)
+        return PressResult(ops.select_compact(kview, vview, scores, width, n_kept=n_kept), width, scores, list(kept))
     if len(set(kept)) == 1:
         idx = ops.topk_select(scores, width)
         if compact and width > 0:

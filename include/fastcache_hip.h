@@ -188,6 +188,18 @@ int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, float* scor
                    const int32_t* n_kept, int32_t* indices, int32_t index_stride, void* stream);
 
 /*
+ * Selection and in-place compaction in one launch, from scores that a scoring entry point wrote: for every
+ * (layer, b, kv head) row of scores[.., score_stride], fc_topk_select over the row's first seq_lens[b] entries
+ * (keeping n_kept[b], or `k` when n_kept is NULL) and fc_compact of `keys` and `values` onto themselves with the row's
+ * own indices, with the same indices (entries past a row's kept count are left as they are) and cache bytes as those
+ * two calls.  Sequences of up to 8192 tokens; longer views are refused with FC_EUNSUPPORTED and take the two calls.
+ * Replaces scores.topk + gather of kvpress ScorerPress.compress (third-party) together with
+ * LlavaModelRunner._write_compressed_kv_cache_fast (nanovllm/engine/llava_model_runner.py:874-912).
+ */
+int fc_select_compact(const fc_kv_view* keys, const fc_kv_view* values, const float* scores, int32_t score_stride,
+                      int32_t k, const int32_t* n_kept, int32_t* indices, int32_t index_stride, void* stream);
+
+/*
  * Gather + compaction.  For each (layer, b, kv head): dst token j <- src token
  * indices[(l*batch + b)*heads_in_index + (h % heads_in_index)][j] for j < n_kept[b] (or k).
  * `dst` may alias `src` (same pool, same tables): indices must then be ascending, and the

@@ -110,6 +110,47 @@ def test_knorm_press_one_launch_equals_three(dev, dtype, lens, block_size, keep)
     assert not torch.equal(pool_b.view(torch.uint8), case.kv_cache.to(dev).view(torch.uint8)) or width == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("lens,block_size,keep", [
+    ([700, 512, 3], 256, [350, 256, 0]),
+    ([4096], 256, [1024]),
+    ([300, 300], 64, [300, 299]),
+    ([2500, 130, 2049], 128, [1, 129, 700]),
+    ([193, 77], 48, [100, 33]),
+])
+def test_select_compact_one_launch_equals_two(dev, dtype, lens, block_size, keep):
+    """fc_select_compact against fc_topk_select + fc_compact on the same pool and the same scores (random, with
+    repeated values and -inf past each sequence's end): indices and every byte of both planes identical."""
+    H = 3
+    case = synth.make_paged_case(seed=12, num_layers=2, batch=len(lens), num_kv_heads=H, seq_lens=lens, dtype=dtype,
+                                 block_size=block_size)
+    pool_a = case.kv_cache.to(dev)
+    pool_b = pool_a.clone()
+    tables, lens_d = case.table_tensor(dev), case.lens_tensor(dev)
+    S, width = max(lens), max(keep)
+    g = torch.Generator().manual_seed(3)
+    scores = torch.randn((2, len(lens), H, S), generator=g)
+    scores[..., ::7] = 0.25                                   # many equal scores: the tie-break decides
+    for b, n in enumerate(lens):
+        scores[:, b, :, n:] = float("-inf")
+    scores = scores.to(dev)
+    n_kept = torch.tensor(keep, dtype=torch.int32, device=dev)
+    ka, va = (_lib.paged_view(pool_a[p], tables, lens_d, S) for p in range(2))
+    idx_a = ops.topk_select(scores, width, row_lens=lens_d, n_kept=n_kept, rows_per_len=H)
+    ops.compact(ka, va, ka, va, idx_a, n_kept=n_kept)
+    kb, vb = (_lib.paged_view(pool_b[p], tables, lens_d, S) for p in range(2))
+    idx_b = ops.select_compact(kb, vb, scores, width, n_kept=n_kept)
+    torch.cuda.synchronize()
+    assert torch.equal(idx_a, idx_b)
+    assert torch.equal(pool_a.view(torch.uint8), pool_b.view(torch.uint8))
+    if len(set(keep)) == 1 and len(set(lens)) == 1:           # the form without per-sequence counts
+        pool_c = case.kv_cache.to(dev)
+        kc, vc = (_lib.paged_view(pool_c[p], tables, lens_d, S) for p in range(2))
+        idx_c = ops.select_compact(kc, vc, scores, width)
+        assert torch.equal(idx_c, ops.topk_select(scores, width))
+        assert torch.equal(pool_c.view(torch.uint8), pool_a.view(torch.uint8))
+
+
 def test_knorm_press_one_launch_limits_and_clamps(dev):
     """Sequences beyond 8192 tokens are refused by name; a kept count in device memory larger than the sequence or
     the index row is clamped; a dense view works like a paged one."""
