@@ -148,7 +148,9 @@ class SnapKVWorkload(Workload):
     name = "cfg2-snapkv-qwen3-8b"
     dtype_name = "bf16"
     kernel_name = "snapkv_kernel"
-    separate_selection = False     # True: fc_topk_select and fc_compact as two launches (sequences beyond 8192 tokens)
+    one_launch = True              # scoring, selection and compaction of a column by one workgroup (fc_snapkv_press);
+                                   # False: fc_snapkv_score, then fc_select_compact (shapes the press does not take)
+    separate_selection = False     # with one_launch False: fc_topk_select and fc_compact as two launches
 
     def __init__(self, seed, device, given_lse=False):
         super().__init__()
@@ -172,8 +174,10 @@ class SnapKVWorkload(Workload):
         k_bytes = self.L * self.B * self.Hkv * self.S * D * e
         gather_bytes = 4 * self.L * self.B * self.Hkv * self.n_kept * D * e
         score_bytes = self.L * self.B * self.Hkv * self.S * 4
-        # dominant kernel = SnapKV scoring: Q window and K read once, fp32 scores written once
-        self.kernel_bytes = q_bytes + k_bytes + score_bytes
+        # SnapKV scoring: Q window and K read once, fp32 scores written once; the one-launch press also moves the
+        # kept K and V rows (read + written) in the same launch
+        self.score_bytes_total = q_bytes + k_bytes + score_bytes
+        self.kernel_bytes = self.score_bytes_total + gather_bytes
         self.kernel_flops = 2 * self.B * self.L * self.Hq * self.W * self.S * D
         self.pass_bytes = q_bytes + k_bytes + gather_bytes
         self.lse = None
@@ -207,6 +211,13 @@ class SnapKVWorkload(Workload):
         scores = torch.empty((L, B, Hkv, S), dtype=torch.float32, device=self.device)
         row_max = torch.empty((L, B, Hkv), dtype=torch.float32, device=self.device)
         st = current_stream()
+        if self.one_launch:                       # what paged_press.snapkv_compress_paged issues for this shape
+            with self.br:
+                scores, idx = ops.snapkv_press(kview, vview, self.queries, self.W, self.ksz, self.n_kept, True, "sum",
+                                               seq_lens=self.lens, lse=self.lse)
+            if self.keep:
+                self.kept, self.keep = (scores, idx), False
+            return
         with self.br:
             if self.lse is None:
                 check(fn("fc_snapkv_score")(C.byref(kview), self.queries.data_ptr(), self.Hq, self.W, self.ksz, 1,
@@ -606,9 +617,12 @@ class CopyWorkload(Workload):
                 "sample": "torch clone of 1 of 4 sequences on the host"}
 
 
-def _separate(w):
-    w.separate_selection = True
-    w.name += "-separate-selection"
+def _separate(w, three):
+    """cfg2 as two launches (scoring; selection + compaction) or three (scoring; selection; compaction)."""
+    w.one_launch = False
+    w.separate_selection = three
+    w.kernel_bytes = w.score_bytes_total
+    w.name += "-three-launches" if three else "-two-launches"
     return w
 
 
@@ -616,8 +630,10 @@ WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkl
              "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True),
              # cfg2 with the window queries' log-sum-exp handed in (not the BASELINE metric: the reference has no such input)
              "snapkv-lse": lambda seed, dev: SnapKVWorkload(seed, dev, given_lse=True),
-             # cfg2 with selection and compaction as two launches
-             "snapkv-sep": lambda seed, dev: _separate(SnapKVWorkload(seed, dev)),
+             # cfg2 with the selection and compaction as launches of their own
+             "snapkv-two": lambda seed, dev: _separate(SnapKVWorkload(seed, dev), False),
+             "snapkv-three": lambda seed, dev: _separate(SnapKVWorkload(seed, dev), True),
+             "snapkv-lse-two": lambda seed, dev: _separate(SnapKVWorkload(seed, dev, given_lse=True), False),
              # the decode launches without a graph, 4 steps per bracket: rocprofv3 cannot walk the 128-step graph
              "decode-eager": lambda seed, dev: DecodeWorkload(seed, dev, graph_steps=4, eager=True),
              # the 64 decode steps that follow the compression in configuration 5, in one graph
@@ -640,8 +656,8 @@ _WRITE_SCALE = 524288 / 5.244e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
     "cfg1-knorm-llama-7b": (5.246e5, 5.304e5),
     "cfg1-knorm-llama-7b-three-launches": (2.641e5, 5.263e5),
-    "cfg2-snapkv-qwen3-8b": (2.390e6, 3.636e4),
-    "cfg2-snapkv-qwen3-8b+given-lse": (1.273e6, 3.636e4),           # one sweep: K is read once
+    "cfg2-snapkv-qwen3-8b-two-launches": (2.390e6, 3.636e4),
+    "cfg2-snapkv-qwen3-8b+given-lse-two-launches": (1.273e6, 3.636e4),           # one sweep: K is read once
     "cfg3-ccm-linear-decouple-llava-1.5-7b": (1.861e6, 1.845e6),      # mean over the 4 launches of a step
     "cfg5-ccm-hybrid-minicpm-v-2.6": (3.919e6, 1.468e6),
     # The decode launches were counted without the graph, 4 steps per bracket (the profiler is not run on the long

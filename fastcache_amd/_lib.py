@@ -63,6 +63,7 @@ SIGNATURES = {
     "fc_knorm_mean_score": (C.c_int, [_V, _VP, _I, _VP]),
     "fc_snapkv_score": (C.c_int, [_V, _VP, _I, _I, _I, _I, _F, _F, _VP, _I, _VP, _VP]),
     "fc_snapkv_score_lse": (C.c_int, [_V, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP, _I, _VP, _VP]),
+    "fc_snapkv_press": (C.c_int, [_V, _V, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP, _I, _VP, _I, _VP, _VP, _I, _VP]),
     "fc_snapkv_split_workspace_bytes": (C.c_int64, [_I, _I, _I, _I, _I, _I, _I]),
     "fc_snapkv_score_split": (C.c_int, [_V, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP, _I, _VP, _I, _VP, C.c_int64, _VP]),
     "fc_snapkv_fill_window": (C.c_int, [_VP, _I, _I, _I, _I, _VP, _I, _I, _VP, _VP]),

@@ -30,8 +30,7 @@
 //
 // Table entries of a live sequence must be allocated blocks: a negative entry inside the sequence
 // reads block 0 instead of faulting.
-#include "fc_common.h"
-
+#include "fc_press.h"
 
 #define SK_KT 64           // keys per tile
 #define SK_TILEB (SK_KT * 256)  // LDS bytes per key tile (rows unpadded, 16-byte chunks XOR-swizzled)
@@ -53,11 +52,29 @@ struct SkCfg {
 // MODE 1: sweep 1 over the piece's tiles only; (largest scaled logit, sum of exp2) per query go to `part`;
 // MODE 2: sweep 2 over the piece's tiles with the log-sum-exp given; the per-key sums go to `raw` unpooled
 //         (a small kernel takes the moving average afterwards, across the pieces' borders).
-template <int DTYPE, int NW, bool FAST, int MODE>
+// PRESS (MODE 0, at least four wavefronts): the workgroup goes on to select the column's kept positions (the
+// window always among them) and to move the kept K and V rows to the front of the column, see the end of the kernel.
+struct SkPress {
+  KvView vv;            // the value plane, same geometry as the keys
+  int k;                // kept positions per row when n_kept is null
+  const int* n_kept;    // [batch] in device memory, or null
+  int* indices;         // [layers][batch][kv heads][index_stride]
+  int index_stride;
+};
+
+// LDS the press tail carves out of the key tiles and the per-key sum area behind them: the score row, the kept
+// positions, the value view's block-table row and the selection's counters
+template <int NW>
+constexpr int sk_press_room() { return SkCfg<NW>::ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4; }
+__host__ __device__ constexpr int sk_press_need(int max_seq_len, int index_stride) {
+  return 4 * max_seq_len + 4 * index_stride + 4 * SK_TBL + 2048;
+}
+
+template <int DTYPE, int NW, bool FAST, int MODE, bool PRESS = false>
 __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     KvView kv, const char* __restrict__ q, int Hq, int W, int ksz, int causal, float c, float out_mul,
     float* __restrict__ scores, int score_stride, float* __restrict__ row_max, const float* __restrict__ lse,
-    int nsplit, float* __restrict__ part, float* __restrict__ raw) {
+    int nsplit, float* __restrict__ part, float* __restrict__ raw, SkPress press) {
   constexpr int THREADS = NW * 64;
   constexpr int ST = SkCfg<NW>::ST;
   constexpr int LPW = 16 / NW;   // 1 KB wave-loads (4 key rows) per wavefront and tile
@@ -88,6 +105,12 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     if (MODE != 0) return;   // the pooling kernel writes such rows
     for (int s = tid; s < score_stride; s += THREADS) out_row[s] = s < S ? 0.f : -INFINITY;
     if (row_max && tid == 0) row_max[((long long)l * kv.batch + b) * Hkv + h] = -INFINITY;
+    if constexpr (PRESS) {   // every position is a window position: the first kept-count of them stay where they are
+      int kk = press.n_kept ? press.n_kept[b] : press.k;
+      kk = min(min(kk, S), press.index_stride);
+      int* idx_row = press.indices + (((long long)l * kv.batch + b) * Hkv + h) * (long long)press.index_stride;
+      for (int i = tid; i < kk; i += THREADS) idx_row[i] = i;
+    }
     return;
   }
   const int SW = S - W;                       // scored keys
@@ -492,6 +515,32 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       row_max[((long long)l * kv.batch + b) * Hkv + h] = mx;
     }
   }
+  // ---- press: select and compact this column --------------------------------------------------------------
+  // The window positions rank above every scored key (the caller fills them with the layer's largest score afterwards;
+  // here they are +inf), so with more kept positions than window positions the selection equals the one over the
+  // filled row.  The score row is read back from memory (this workgroup wrote it; its stores are waited for) into the
+  // LDS that held the key tiles.
+  if constexpr (PRESS) {
+    static_assert(MODE == 0 && NW >= 4, "the press tail needs a whole column and at least 256 threads");
+    int kk = press.n_kept ? press.n_kept[b] : press.k;
+    kk = min(min(kk, S), press.index_stride);
+    if (kk <= W) return;   // not a selection this tail can make; the host does not ask for it
+    fc_wait_vm<0>();
+    __syncthreads();
+    float* sc = reinterpret_cast<float*>(smem);
+    int* sel = reinterpret_cast<int*>(smem) + S;
+    int* vtbl = sel + press.index_stride;
+    TkShared<THREADS>& sh = *reinterpret_cast<TkShared<THREADS>*>(vtbl + SK_TBL);
+    for (int s = tid; s < S; s += THREADS) sc[s] = s < SW ? out_row[s] : INFINITY;
+    const KvView& vv = press.vv;
+    const int nblk_v = vv.block_shift >= 0 ? ((S - 1) >> vv.block_shift) + 1 : 0;
+    const bool v_lds = vv.block_tables && vv.block_shift >= 0 && nblk_v <= SK_TBL;
+    if (v_lds)
+      for (int i = tid; i < nblk_v; i += THREADS) vtbl[i] = vv.block_tables[(long long)b * vv.table_stride + i];
+    __syncthreads();
+    int* idx_row = press.indices + (((long long)l * kv.batch + b) * Hkv + h) * (long long)press.index_stride;
+    kp_select_and_move<2, THREADS>(kv, vv, tbl, tbl_lds, vtbl, v_lds, sc, sel, sh, l, b, h, S, kk, idx_row);
+  }
 }
 
 // Split columns: the pieces' (max, sum) per window query -> natural-log sum of exponentials.
@@ -605,7 +654,10 @@ __global__ __launch_bounds__(1024) void snapkv_fill_kernel(float* __restrict__ s
 
 static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void* queries, int32_t num_q_heads,
                              int32_t window, int32_t kernel_size, int32_t causal_window, float scale, float out_scale,
-                             float* scores, int32_t score_stride, float* row_max, const float* lse, void* stream) {
+                             float* scores, int32_t score_stride, float* row_max, const float* lse, void* stream,
+                             const fc_kv_view* press_values = nullptr, int32_t press_k = 0,
+                             const int32_t* press_n_kept = nullptr, int32_t* press_indices = nullptr,
+                             int32_t press_index_stride = 0) {
   int rc = fc_check_view(keys, who);
   if (rc) return rc;
   FC_REQUIRE(queries && scores, FC_EINVAL, "%s: null pointer", who);
@@ -631,12 +683,58 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
   const float c = scale * 1.4426950408889634f;
   const float out_mul = out_scale / (float)kernel_size;
   const char* q = (const char*)queries;
+  // a key tile lies inside one page (whose table row fits the LDS copy), or the view is dense
+  const bool fast = keys->stride_token >= 0 && keys->stride_token < (1 << 24) &&   // a tile's byte offsets fit 32 bits
+                    (!keys->block_tables ||
+                     (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL));
+  if (press_values) {   // scoring, selection and compaction of every column by its workgroup
+    const fc_kv_view* values = press_values;
+    if ((rc = fc_check_view(values, who))) return rc;
+    FC_REQUIRE(keys->dtype == values->dtype && keys->num_layers == values->num_layers &&
+                   keys->batch == values->batch && keys->num_kv_heads == values->num_kv_heads &&
+                   keys->max_seq_len == values->max_seq_len,
+               FC_EINVAL, "%s: key and value views disagree on dtype/layers/batch/heads/length", who);
+    FC_REQUIRE(press_indices, FC_EINVAL, "%s: null indices", who);
+    FC_REQUIRE(press_index_stride >= 0 && press_index_stride <= keys->max_seq_len, FC_EINVAL,
+               "%s: index_stride %d exceeds max_seq_len %d", who, press_index_stride, keys->max_seq_len);
+    FC_REQUIRE(press_n_kept != nullptr || (press_k > window && press_k <= press_index_stride), FC_EINVAL,
+               "%s: k=%d must exceed the window (%d) and fit index_stride=%d", who, press_k, window,
+               press_index_stride);
+    const int nw = waves <= 4 ? 4 : (waves <= 8 ? 8 : 16);
+    const int room = nw == 4 ? sk_press_room<4>() : (nw == 8 ? sk_press_room<8>() : sk_press_room<16>());
+    FC_REQUIRE(fast && sk_press_need(keys->max_seq_len, press_index_stride) <= room, FC_EUNSUPPORTED,
+               "%s: the one-launch press takes dense views or pages of 64*2^n tokens and 4*(max_seq_len + "
+               "index_stride) + 6144 <= %d bytes (got max_seq_len %d, index_stride %d); use fc_snapkv_score and "
+               "fc_select_compact", who, room, keys->max_seq_len, press_index_stride);
+    SkPress press;
+    press.vv = fc_make_view(values);
+    press.k = press_k;
+    press.n_kept = press_n_kept;
+    press.indices = press_indices;
+    press.index_stride = press_index_stride;
+#define SK_PRESS(DT, NWV)                                                                                        \
+  do {                                                                                                         \
+    FC_ALLOW_LDS((snapkv_kernel<DT, NWV, true, 0, true>), SkCfg<NWV>::LDS);                                     \
+    hipLaunchKernelGGL((snapkv_kernel<DT, NWV, true, 0, true>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, \
+                       q, num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,   \
+                       row_max, lse, 1, (float*)nullptr, (float*)nullptr, press);                              \
+  } while (0)
+#define SK_PRESS_NW(DT)                 \
+  if (nw == 4) SK_PRESS(DT, 4);         \
+  else if (nw == 8) SK_PRESS(DT, 8);    \
+  else SK_PRESS(DT, 16)
+    if (keys->dtype == FC_BF16) { SK_PRESS_NW(FC_BF16); } else { SK_PRESS_NW(FC_F16); }
+#undef SK_PRESS_NW
+#undef SK_PRESS
+    FC_CHECK_LAUNCH(who);
+    return FC_OK;
+  }
 #define SK_LAUNCH(DT, NWV, FA)                                                                                  \
   do {                                                                                                       \
     FC_ALLOW_LDS((snapkv_kernel<DT, NWV, FA, 0>), SkCfg<NWV>::LDS);                                           \
     hipLaunchKernelGGL((snapkv_kernel<DT, NWV, FA, 0>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,    \
                        num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,    \
-                       row_max, lse, 1, (float*)nullptr, (float*)nullptr);                                   \
+                       row_max, lse, 1, (float*)nullptr, (float*)nullptr, SkPress{});                        \
   } while (0)
 #define SK_DISPATCH2(DT, FA)                 \
   if (waves <= 1) SK_LAUNCH(DT, 1, FA);      \
@@ -646,10 +744,6 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
   else SK_LAUNCH(DT, 16, FA)
 #define SK_DISPATCH(DT) \
   if (fast) { SK_DISPATCH2(DT, true); } else { SK_DISPATCH2(DT, false); }
-  // a key tile lies inside one page (whose table row fits the LDS copy), or the view is dense
-  const bool fast = keys->stride_token >= 0 && keys->stride_token < (1 << 24) &&   // a tile's byte offsets fit 32 bits
-                    (!keys->block_tables ||
-                     (kv.block_shift >= 6 && ((keys->max_seq_len - 1) >> kv.block_shift) < SK_TBL));
   if (keys->dtype == FC_BF16) { SK_DISPATCH(FC_BF16); } else { SK_DISPATCH(FC_F16); }
 #undef SK_DISPATCH2
 #undef SK_DISPATCH
@@ -673,6 +767,17 @@ extern "C" int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, 
   FC_REQUIRE(lse, FC_EINVAL, "%s: null log-sum-exp pointer", who);
   return snapkv_score_impl(who, keys, queries, num_q_heads, window, kernel_size, causal_window, scale, out_scale,
                            scores, score_stride, row_max, lse, stream);
+}
+
+extern "C" int fc_snapkv_press(const fc_kv_view* keys, const fc_kv_view* values, const void* queries, const float* lse,
+                               int32_t num_q_heads, int32_t window, int32_t kernel_size, int32_t causal_window,
+                               float scale, float out_scale, float* scores, int32_t score_stride, float* row_max,
+                               int32_t k, const int32_t* n_kept, int32_t* indices, int32_t index_stride,
+                               void* stream) {
+  const char* who = "fc_snapkv_press";
+  FC_REQUIRE(values, FC_EINVAL, "%s: null value view", who);
+  return snapkv_score_impl(who, keys, queries, num_q_heads, window, kernel_size, causal_window, scale, out_scale,
+                           scores, score_stride, row_max, lse, stream, values, k, n_kept, indices, index_stride);
 }
 
 // ---- split columns ------------------------------------------------------------------------------------
@@ -737,7 +842,7 @@ extern "C" int fc_snapkv_score_split(const fc_kv_view* keys, const void* queries
     FC_ALLOW_LDS((snapkv_kernel<DT, NWV, true, MD>), SkCfg<NWV>::LDS);                                            \
     hipLaunchKernelGGL((snapkv_kernel<DT, NWV, true, MD>), grid, dim3(NWV * 64), SkCfg<NWV>::LDS, st, kv, q,     \
                        num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,        \
-                       row_max, lse_use, nsplit, part, raw);                                                     \
+                       row_max, lse_use, nsplit, part, raw, SkPress{});                                          \
   } while (0)
 #define SK_SPLIT_NW(DT, MD)                     \
   if (waves <= 1) SK_SPLIT(DT, 1, MD);          \

@@ -140,6 +140,74 @@ def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size
     return out
 
 
+def snapkv_press_fits(keys: FcKvView, num_q_heads: int, window: int, index_stride: int) -> bool:
+    """Whether :func:`snapkv_press` takes this shape (otherwise: ``snapkv_score`` + ``select_compact``): 3 to 16 blocks
+    of 32 window queries per kv head, pages of 64*2^n tokens or a dense view, and
+    the score row plus the kept positions inside the LDS of the key tiles."""
+    if num_q_heads % keys.num_kv_heads:
+        return False
+    blocks = (num_q_heads // keys.num_kv_heads) * ((window + 31) // 32)
+    if blocks < 3 or blocks > 16:
+        return False
+    waves = 4 if blocks <= 4 else (8 if blocks <= 8 else 16)
+    tiles = 4 if waves >= 8 else 3
+    room = tiles * 64 * 256 + (4 * waves + 4) * 64 * 4
+    paged_ok = (not keys.block_tables) or (keys.block_size >= 64 and keys.block_size & (keys.block_size - 1) == 0
+                                           and (keys.max_seq_len - 1) // keys.block_size < 1024)
+    return bool(paged_ok and 4 * (keys.max_seq_len + index_stride) + 6144 <= room and
+                0 <= keys.stride_token < (1 << 24))
+
+
+def snapkv_press(keys: FcKvView, values: FcKvView, queries: torch.Tensor, window: int, kernel_size: int, k: int,
+                 causal_window: bool = True, reduction: str = "mean", scale: Optional[float] = None,
+                 seq_lens: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                 n_kept: Optional[torch.Tensor] = None, ragged: bool = False):
+    """SnapKV scores, selection (the window always kept; ``k`` or ``n_kept[b]`` positions per row, window included,
+    more than the window) and in-place compaction of both planes, each (layer, sequence, kv head) column by one
+    workgroup in one launch; then the window fill of the scores.  Returns ``(scores, indices)`` equal to
+    ``snapkv_score`` + ``select_compact``.  Shapes must satisfy :func:`snapkv_press_fits`."""
+    if queries.dim() == 4:
+        queries = queries.unsqueeze(0)
+        if lse is not None and lse.dim() == 3:
+            lse = lse.unsqueeze(0)
+    if not queries.is_contiguous():
+        queries = queries.contiguous()
+    _lib.require_gpu(queries, "queries")
+    L, B, Hq, W, D = queries.shape
+    H = keys.num_kv_heads
+    if (L, B) != (keys.num_layers, keys.batch) or W != window or D != keys.head_dim:
+        raise FastcacheError(f"queries {tuple(queries.shape)} do not match the key view "
+                             f"(L={keys.num_layers}, B={keys.batch}, W={window}, D={keys.head_dim})")
+    if _lib.dtype_code(queries.dtype) != keys.dtype:
+        raise FastcacheError("queries and keys must share a dtype")
+    if reduction not in ("mean", "sum"):
+        raise ValueError("reduction must be 'mean' or 'sum'")
+    out_scale = 1.0 / (W * (Hq // H)) if reduction == "mean" else 1.0
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    dev = queries.device
+    stride = keys.max_seq_len
+    scores = torch.empty((L, B, H, stride), dtype=torch.float32, device=dev)
+    row_max = torch.empty((L, B, H), dtype=torch.float32, device=dev)
+    n_kept = _i32(n_kept, "n_kept", dev)
+    if n_kept is not None or ragged:
+        idx = torch.full((L, B, H, k), -1, dtype=torch.int32, device=dev)
+    else:
+        idx = torch.empty((L, B, H, k), dtype=torch.int32, device=dev)
+    if lse is not None:
+        _lib.require_gpu(lse, "lse")
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (L, B, Hq, W):
+            raise FastcacheError(f"lse must be fp32 [L={L}, B={B}, Hq={Hq}, W={W}], got {lse.dtype} {tuple(lse.shape)}")
+        lse = lse.contiguous()
+    st = current_stream()
+    check(fn("fc_snapkv_press")(C.byref(keys), C.byref(values), queries.data_ptr(), ptr(lse), Hq, window, kernel_size,
+                                int(causal_window), scale, out_scale, scores.data_ptr(), stride, row_max.data_ptr(), k,
+                                ptr(n_kept), idx.data_ptr(), k, st), "fc_snapkv_press")
+    check(fn("fc_snapkv_fill_window")(scores.data_ptr(), stride, L, B, H, ptr(seq_lens), keys.max_seq_len, window,
+                                      row_max.data_ptr(), st), "fc_snapkv_fill_window")
+    return scores, idx
+
+
 # ---------------------------------------------------------------------------------------------
 # selection and compaction
 # ---------------------------------------------------------------------------------------------

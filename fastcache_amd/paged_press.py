@@ -91,10 +91,21 @@ def snapkv_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, se
     every sequence).  With ``window_in_budget`` (kvpress) the observation window counts towards ``n_kept``;
     otherwise it is kept on top of it."""
     kview, vview = _views(kv_cache, block_tables, seq_lens, seq_len)
-    scores = ops.snapkv_score(kview, queries, window_size, kernel_size, causal_window, reduction,
-                              seq_lens=seq_lens)
     lens = list(host_lens) if host_lens is not None else [seq_len] * block_tables.shape[0]
     kept = [n_kept_for(n, compression_ratio) for n in lens]
     if not window_in_budget:
         kept = [min(n, k + window_size) for n, k in zip(lens, kept)]
+    width = max(kept)
+    # the workgroup that scored a column also selects and compacts it when every row keeps more than the window
+    # (sequences no longer than the window keep their first positions either way)
+    if (compact and all(k > window_size or n <= window_size for n, k in zip(lens, kept)) and width > window_size and
+            ops.snapkv_press_fits(kview, queries.shape[-3], window_size, width) and
+            ops.snapkv_splits(kview, queries.shape[-3], window_size) == 1):   # few columns: key ranges pay more
+        same = len(set(kept)) == 1 and len(set(lens)) == 1
+        n_kept = None if same else torch.tensor(kept, dtype=torch.int32, device=kv_cache.device)
+        scores, idx = ops.snapkv_press(kview, vview, queries, window_size, kernel_size, width, causal_window,
+                                       reduction, seq_lens=seq_lens, n_kept=n_kept)
+        return PressResult(idx, width, scores, None if same else list(kept))
+    scores = ops.snapkv_score(kview, queries, window_size, kernel_size, causal_window, reduction,
+                              seq_lens=seq_lens)
     return _select_and_compact(kview, vview, scores, seq_lens, kept, compact, kv_cache.shape[4])

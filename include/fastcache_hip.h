@@ -133,6 +133,25 @@ int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float
                         float out_scale, float* scores, int32_t score_stride, float* row_max, void* stream);
 
 /*
+ * SnapKV press in one launch: fc_snapkv_score (or fc_snapkv_score_lse when `lse` is not NULL) and, by the same
+ * workgroup that scored a (layer, b, kv head) column, the selection of the column's kept positions and the compaction
+ * of `keys` and `values` onto themselves.  Kept counts (k, or n_kept[b] in device memory) include the window and must
+ * exceed it: the window positions rank first, as they do after fc_snapkv_fill_window, so the indices and cache bytes
+ * are those of fc_snapkv_score + fc_snapkv_fill_window + fc_topk_select + fc_compact.  `scores` receives the scored
+ * positions and `row_max` (required) the per-row maxima; the caller runs fc_snapkv_fill_window afterwards if it wants
+ * the window entries of `scores` filled.  Rows of sequences no longer than the window keep their first positions.
+ * Takes dense views or pages of 64*2^n tokens and sequences short enough for the score row and the kept positions to
+ * fit the LDS of the key tiles: 4 * (max_seq_len + index_stride) + 6144 bytes within 54272 (up to four 32-row query
+ * blocks per kv head) or 74752 (more), e.g. 13 000 tokens of which a quarter is kept; refused with FC_EUNSUPPORTED
+ * otherwise.  A row whose kept count does not exceed the window (n_kept comes from device memory) is left untouched.  Replaces, for SnapKVPress, the per-sequence loop of
+ * LlavaModelRunner.compress_kv_cache_batch (nanovllm/engine/llava_model_runner.py:745-786).
+ */
+int fc_snapkv_press(const fc_kv_view* keys, const fc_kv_view* values, const void* queries, const float* lse,
+                    int32_t num_q_heads, int32_t window, int32_t kernel_size, int32_t causal_window, float scale,
+                    float out_scale, float* scores, int32_t score_stride, float* row_max, int32_t k,
+                    const int32_t* n_kept, int32_t* indices, int32_t index_stride, void* stream);
+
+/*
  * The same scores with every (layer, sequence, kv head) column cut into `nsplit` key ranges, one workgroup each:
  * statistics of the pieces, their merge, per-key sums of the pieces, then the moving average across the pieces'
  * borders.  For launches with too few columns to fill the GPU (one long prompt of a model with few kv heads:

@@ -151,6 +151,65 @@ def test_select_compact_one_launch_equals_two(dev, dtype, lens, block_size, keep
         assert torch.equal(pool_c.view(torch.uint8), pool_a.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lens,Hq,H,W,ksz,keep,given_lse", [
+    ([1000, 1000], 8, 2, 64, 7, [250, 250], False),         # 8 query blocks per kv head, equal lengths
+    ([700, 512, 20, 300], 8, 2, 32, 5, [175, 128, 5, 75], False),    # ragged, one sequence shorter than the window
+    ([2048], 28, 4, 64, 7, [512], False),                   # 14 blocks: 16 wavefronts
+    ([900, 333], 4, 1, 32, 1, [225, 83], True),             # 4 blocks, log-sum-exp given, no pooling
+    ([4096], 8, 2, 64, 7, [1024], False),                   # the second configuration's column
+])
+def test_snapkv_press_one_launch_equals_separate(dev, dtype, lens, Hq, H, W, ksz, keep, given_lse):
+    """fc_snapkv_press against fc_snapkv_score + fc_snapkv_fill_window + fc_topk_select + fc_compact: the same
+    kernel code scores, so scores (window fill included), indices and every cache byte must be identical."""
+    L = 2
+    case = synth.make_paged_case(seed=21, num_layers=L, batch=len(lens), num_kv_heads=H, seq_lens=lens, dtype=dtype,
+                                 num_q_heads=Hq, window=W)
+    pool_a = case.kv_cache.to(dev)
+    pool_b = pool_a.clone()
+    tables, lens_d, q = case.table_tensor(dev), case.lens_tensor(dev), case.queries.to(dev)
+    S, width = max(lens), max(keep)
+    n_kept = torch.tensor(keep, dtype=torch.int32, device=dev)
+    ka, va = (_lib.paged_view(pool_a[p], tables, lens_d, S) for p in range(2))
+    lse = None
+    if given_lse:
+        lse = torch.empty((L, len(lens), Hq, W), dtype=torch.float32, device=dev)
+        for l in range(L):
+            for b, n in enumerate(lens):
+                kd = opaged.extract_kv(case.kv_cache[:, l:l + 1], case.block_tables[b], n)[0][0][0].float()   # [H, n, D]
+                logits = torch.matmul(case.queries[l, b].float(), kd.repeat_interleave(Hq // H, 0).transpose(1, 2))
+                mask = torch.triu(torch.full((W, n), float("-inf")), diagonal=n - W + 1) if n >= W else torch.zeros(W, n)
+                lse[l, b] = torch.logsumexp(logits * 128 ** -0.5 + mask, dim=-1).to(dev)
+    assert ops.snapkv_press_fits(ka, Hq, W, width)
+    scores_a = ops.snapkv_score(ka, q, W, ksz, True, "sum", seq_lens=lens_d, lse=lse, splits=1)
+    idx_a = ops.topk_select(scores_a, width, row_lens=lens_d, n_kept=n_kept, rows_per_len=H)
+    ops.compact(ka, va, ka, va, idx_a, n_kept=n_kept)
+    kb, vb = (_lib.paged_view(pool_b[p], tables, lens_d, S) for p in range(2))
+    scores_b, idx_b = ops.snapkv_press(kb, vb, q, W, ksz, width, True, "sum", seq_lens=lens_d, lse=lse, n_kept=n_kept)
+    torch.cuda.synchronize()
+    assert torch.equal(scores_a.view(torch.int32), scores_b.view(torch.int32))
+    assert torch.equal(idx_a, idx_b)
+    assert torch.equal(pool_a.view(torch.uint8), pool_b.view(torch.uint8))
+    assert not torch.equal(pool_b.view(torch.uint8), case.kv_cache.to(dev).view(torch.uint8))
+
+
+def test_snapkv_press_refuses_what_it_cannot_take(dev):
+    case = synth.make_paged_case(seed=2, num_layers=1, batch=1, num_kv_heads=1, seq_lens=[512], dtype=torch.bfloat16,
+                                 num_q_heads=4, window=64)
+    pool = case.kv_cache.to(dev)
+    tables, lens_d, q = case.table_tensor(dev), case.lens_tensor(dev), case.queries.to(dev)
+    kv, vv = (_lib.paged_view(pool[p], tables, lens_d, 512) for p in range(2))
+    with pytest.raises(_lib.FastcacheError, match="exceed the window"):
+        ops.snapkv_press(kv, vv, q, 64, 7, 64)                 # a kept count that does not exceed the window
+    long = synth.make_paged_case(seed=2, num_layers=1, batch=1, num_kv_heads=1, seq_lens=[20000], dtype=torch.bfloat16,
+                                 num_q_heads=4, window=64)
+    pool = long.kv_cache.to(dev)
+    kv, vv = (_lib.paged_view(pool[p], long.table_tensor(dev), long.lens_tensor(dev), 20000) for p in range(2))
+    assert not ops.snapkv_press_fits(kv, 4, 64, 5000)
+    with pytest.raises(_lib.FastcacheError, match="fc_select_compact"):
+        ops.snapkv_press(kv, vv, long.queries.to(dev), 64, 7, 5000)
+
+
 def test_knorm_press_one_launch_limits_and_clamps(dev):
     """Sequences beyond 8192 tokens are refused by name; a kept count in device memory larger than the sequence or
     the index row is clamped; a dense view works like a paged one."""
