@@ -650,12 +650,14 @@ _COUNTER_RUN = {"commit": "76bf753", "date": "2026-11-25"}   # the tree whose ke
 # (cfg5's MLP launch keeps the first round's reading: this round's counter run of that workload ended in a host-side
 #  crash of the profiled process inside the profiler's dispatch hook, while torch was still building the inputs)
 _COUNTER_RUN_OF = {"cfg5-ccm-hybrid-minicpm-v-2.6": {"commit": "3ee0b1a", "date": "2026-11-25"},
-                   "cfg1-knorm-llama-7b": {"commit": "f22b65d", "date": "2026-11-25"}}
+                   "cfg1-knorm-llama-7b": {"commit": "f22b65d", "date": "2026-11-25"},
+                   "cfg2-snapkv-qwen3-8b": {"commit": "f63ab2e", "date": "2026-11-25"}}
 _FETCH_SCALE = 524288 / 2.623e5
 _WRITE_SCALE = 524288 / 5.244e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
     "cfg1-knorm-llama-7b": (5.246e5, 5.304e5),
     "cfg1-knorm-llama-7b-three-launches": (2.641e5, 5.263e5),
+    "cfg2-snapkv-qwen3-8b": (2.994e6, 1.225e6),                       # the one-launch press: kept rows moved as well
     "cfg2-snapkv-qwen3-8b-two-launches": (2.390e6, 3.636e4),
     "cfg2-snapkv-qwen3-8b+given-lse-two-launches": (1.273e6, 3.636e4),           # one sweep: K is read once
     "cfg3-ccm-linear-decouple-llava-1.5-7b": (1.861e6, 1.845e6),      # mean over the 4 launches of a step
