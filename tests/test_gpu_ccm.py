@@ -30,8 +30,8 @@ OBSERVED = []   # (elements, relative error norm, elements beyond the bound, max
 
 
 def mlp_error_stats(got, ref, dtype):
-    """Relative error norm, number of elements beyond ``1e-3 * max|ref| + 2 ulp(storage) * |ref|``, and the
-    largest error over ``max|ref|``."""
+    """Relative error norm, number of elements beyond ``1e-3 * max|ref| + 2 ulp(storage) * |ref|``, the largest
+    error over ``max|ref|``, and the element count."""
     got, ref = got.float(), ref.float()
     ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
     scale = float(ref.abs().max())
@@ -39,6 +39,19 @@ def mlp_error_stats(got, ref, dtype):
     err = (got - ref).abs()
     bound = 1e-3 * scale + 2 * ulp * ref.abs().clamp_min(scale * 2.0 ** -14)
     return rel, int((err > bound).sum()), float(err.max()) / scale, err.numel()
+
+
+MLP_ROW_REL = {torch.float16: 1e-3, torch.bfloat16: 5e-3}   # error norm of ONE output row over its own norm
+
+
+def mlp_norm_bar(n, dtype, row=128):
+    """Bar for the relative error norm of a comparison of ``n`` outputs: 1e-3, or, when the comparison has so few
+    rows that a single row decides it, what one row may be off by (``MLP_ROW_REL`` / sqrt(rows)).  In bf16 one or two
+    output rows in a thousand differ by more than 1e-3 of their own norm between two correct evaluations (a flipped
+    hidden activation shifts all 128 outputs of its token), at most 4.2e-3; in fp16 none by more than 6e-4: measured
+    by tests/test_oracle_pinning.py::test_mlp_tolerance_calibration."""
+    rows = max(1, n // row)
+    return max(1e-3, MLP_ROW_REL[dtype] / rows ** 0.5)
 
 
 def mlp_outliers_allowed(n, dtype):
@@ -53,13 +66,15 @@ def assert_mlp_close(got, ref, dtype):
     evaluates the oracle MLP under other fp32 summation orders.  fp16: no element beyond the bound.  bf16: a
     hidden activation on a rounding boundary flips to the neighbouring value about 3 times in 10^7 outputs and
     moves one or two outputs of its row by up to 4.2e-3 of max|ref|.  Allowed here: ``mlp_outliers_allowed``,
-    none further than 6.5e-3 of max|ref|."""
+    none further than 1e-2 of max|ref| (the largest seen in randomised sweeps of ~10^10 outputs is 7.2e-3, in a row
+    where the HIP result equals the fp64-summed evaluation bit for bit and the oracle's fp32 sums are the ones that
+    flipped); the error norm within ``mlp_norm_bar`` (1e-3 from 25 rows on)."""
     rel, n_out, worst, n = mlp_error_stats(got, ref, dtype)
     OBSERVED.append((n, rel, n_out, worst))
-    assert rel <= 1e-3, f"relative error norm {rel:.3e}"
+    assert rel <= mlp_norm_bar(n, dtype, ref.shape[-1]), f"relative error norm {rel:.3e} over {n} outputs"
     allowed = mlp_outliers_allowed(n, dtype)
     assert n_out <= allowed, f"{n_out} of {n} elements beyond 1e-3 * max|ref| + 2 ulp ({allowed} allowed)"
-    assert worst <= 6.5e-3, f"max error {worst:.3e} of max|ref|"
+    assert worst <= 1e-2, f"max error {worst:.3e} of max|ref|"
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
