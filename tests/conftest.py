@@ -42,5 +42,5 @@ def pytest_terminal_summary(terminalreporter):
     if obs:
         terminalreporter.write_line(
             f"MLP parity, {len(obs)} comparisons, {sum(o[0] for o in obs)} elements: worst relative error norm "
-            f"{max(o[1] for o in obs):.3e}, elements beyond 1e-3*max|ref| + 2 ulp: {sum(o[2] for o in obs)}, "
+            f"{max(o[1] for o in obs):.3e}, rows with an element beyond 1e-3*max|ref| + 2 ulp: {sum(o[2] for o in obs)}, "
             f"largest error {max(o[3] for o in obs):.3e} of max|ref|")

@@ -30,15 +30,19 @@ OBSERVED = []   # (elements, relative error norm, elements beyond the bound, max
 
 
 def mlp_error_stats(got, ref, dtype):
-    """Relative error norm, number of elements beyond ``1e-3 * max|ref| + 2 ulp(storage) * |ref|``, the largest
-    error over ``max|ref|``, and the element count."""
+    """Relative error norm, number of output rows (last axis: the 128 outputs of one token) that hold an element
+    beyond ``1e-3 * max|ref| + 2 ulp(storage) * |ref|``, the largest error over ``max|ref|``, and the element count.
+    Rows are counted, not elements: one flipped hidden activation shifts every output of its row and puts one to five
+    of them past the bound."""
     got, ref = got.float(), ref.float()
     ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
     scale = float(ref.abs().max())
     rel = float((got - ref).norm() / ref.norm())
     err = (got - ref).abs()
     bound = 1e-3 * scale + 2 * ulp * ref.abs().clamp_min(scale * 2.0 ** -14)
-    return rel, int((err > bound).sum()), float(err.max()) / scale, err.numel()
+    out = err > bound
+    rows_out = out.any(dim=-1) if out.dim() > 1 else out
+    return rel, int(rows_out.sum()), float(err.max()) / scale, err.numel()
 
 
 MLP_ROW_REL = {torch.float16: 1e-3, torch.bfloat16: 5e-3}   # error norm of ONE output row over its own norm
@@ -54,26 +58,25 @@ def mlp_norm_bar(n, dtype, row=128):
     return max(1e-3, MLP_ROW_REL[dtype] / rows ** 0.5)
 
 
-def mlp_outliers_allowed(n, dtype):
-    """fp16: none.  bf16: a flipped hidden activation moves a few of its row's 128 outputs past the bound at once, so
-    outliers come in clusters of 1-3; four for the odd cluster plus one per million outputs, about three times the
-    rate the CPU calibration measures (3 in 10^7)."""
-    return 0 if dtype == torch.float16 else 4 + n // 1_000_000
+def mlp_outliers_allowed(n, dtype, row=128):
+    """Output rows that may hold an element beyond the bound.  fp16: none.  bf16: two, plus one per 4000 rows of the
+    comparison: about six times the rate the CPU calibration measures (one row in 26 000)."""
+    return 0 if dtype == torch.float16 else 2 + (n // row) // 4000
 
 
 def assert_mlp_close(got, ref, dtype):
     """The allowance is calibrated, not assumed: tests/test_oracle_pinning.py::test_mlp_tolerance_calibration
     evaluates the oracle MLP under other fp32 summation orders.  fp16: no element beyond the bound.  bf16: a
-    hidden activation on a rounding boundary flips to the neighbouring value about 3 times in 10^7 outputs and
-    moves one or two outputs of its row by up to 4.2e-3 of max|ref|.  Allowed here: ``mlp_outliers_allowed``,
-    none further than 1e-2 of max|ref| (the largest seen in randomised sweeps of ~10^10 outputs is 7.2e-3, in a row
+    hidden activation on a rounding boundary flips to the neighbouring value in about one row of 26 000 and
+    moves one to five outputs of that row by up to 4.2e-3 of max|ref|.  Allowed here: ``mlp_outliers_allowed``
+    such rows, no element further than 1e-2 of max|ref| (the largest seen in randomised sweeps of ~10^10 outputs is 7.2e-3, in a row
     where the HIP result equals the fp64-summed evaluation bit for bit and the oracle's fp32 sums are the ones that
     flipped); the error norm within ``mlp_norm_bar`` (1e-3 from 25 rows on)."""
     rel, n_out, worst, n = mlp_error_stats(got, ref, dtype)
     OBSERVED.append((n, rel, n_out, worst))
     assert rel <= mlp_norm_bar(n, dtype, ref.shape[-1]), f"relative error norm {rel:.3e} over {n} outputs"
-    allowed = mlp_outliers_allowed(n, dtype)
-    assert n_out <= allowed, f"{n_out} of {n} elements beyond 1e-3 * max|ref| + 2 ulp ({allowed} allowed)"
+    allowed = mlp_outliers_allowed(n, dtype, ref.shape[-1])
+    assert n_out <= allowed, f"{n_out} rows of {n} outputs hold an element beyond 1e-3 * max|ref| + 2 ulp ({allowed} allowed)"
     assert worst <= 1e-2, f"max error {worst:.3e} of max|ref|"
 
 
