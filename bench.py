@@ -113,6 +113,13 @@ class Workload:
     def check_after(self):
         return None
 
+    def check_collect(self):
+        """What measure() calls right after the checked step: returns a callable that gives check_after()'s result.
+        Here the check is evaluated at once; a workload whose check takes seconds of host work copies what the check
+        needs and evaluates it when called, i.e. after the timed steps, so that the GPU does not idle before them."""
+        result = self.check_after()
+        return lambda: result
+
 
 def _column_dense(kv_cache, plane, layer, table, n):
     """Tokens [0, n) of one sequence of one layer as a CPU tensor [1, Hkv, n, D] (HuggingFace layout)."""
@@ -244,15 +251,20 @@ class SnapKVWorkload(Workload):
         self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
         self.keep = True
 
-    def check_after(self):
-        from oracle import presses as opress
+    def check_collect(self):
         scores, idx = self.kept
         l, b = self.cl, self.cb
-        ref = opress.snapkv_score(self.queries[l, b:b + 1].cpu(), self.snap[0], self.W, self.ksz, True, "sum")[0]
         tab = self.case.block_tables[b]
-        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]
-        return _check_press_column(f"layer {l}, sequence {b}", self.snap[0], self.snap[1], after[0], after[1],
-                                   scores[l, b], ref, idx[l, b], self.S - self.W)
+        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]    # before any later step
+        sc, ix, q = scores[l, b].cpu(), idx[l, b].cpu(), self.queries[l, b:b + 1].cpu()
+        self.kept = None
+
+        def evaluate():
+            from oracle import presses as opress
+            ref = opress.snapkv_score(q, self.snap[0], self.W, self.ksz, True, "sum")[0]
+            return _check_press_column(f"layer {l}, sequence {b}", self.snap[0], self.snap[1], after[0], after[1],
+                                       sc, ref, ix, self.S - self.W)
+        return evaluate
 
     def cpu_baseline(self, budget_s=12.0):
         """CPU restatement of the same pass, layer by layer until the time budget, scaled linearly."""
@@ -319,14 +331,19 @@ class KnormWorkload(Workload):
         self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
         self.keep = True
 
-    def check_after(self):
-        from oracle import presses as opress
+    def check_collect(self):
         scores, idx = self.kept
         l = self.cl
         tab = self.case.block_tables[0]
-        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]
-        return _check_press_column(f"layer {l}, sequence 0", self.snap[0], self.snap[1], after[0], after[1],
-                                   scores[l, 0], opress.knorm_score(self.snap[0])[0], idx[l, 0], self.S)
+        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]    # before any later step
+        sc, ix = scores[l, 0].cpu(), idx[l, 0].cpu()
+        self.kept = None
+
+        def evaluate():
+            from oracle import presses as opress
+            return _check_press_column(f"layer {l}, sequence 0", self.snap[0], self.snap[1], after[0], after[1],
+                                       sc, opress.knorm_score(self.snap[0])[0], ix, self.S)
+        return evaluate
 
     def cpu_baseline(self, budget_s=12.0):
         from oracle import pipeline as opipe
@@ -684,17 +701,18 @@ GRAPH_WORKLOADS = {"decode": "decode-eager", "hybrid-decode": "hybrid-decode-eag
 def measure(workload, seed, dev, steps, warmup, cpu_baseline=True, cpu_budget_s=12.0, check=True, min_warm_s=0.0):
     """One workload: one checked step, warm-up, a timed run of exactly `steps` steps right behind it, roofline of
     the dominant kernel, then a longer run for the sustained rate.
-    The checked step comes first because its host side (the CPU oracle) leaves the GPU idle for seconds, and after
-    any idle gap, even 50 ms, the next ~25 passes of the SnapKV workload run at a lower shader clock (2.4 ms falling
-    to 1.9 ms): the warm-up is there to absorb that, so nothing may separate it from the timed steps.
+    The checked step comes first and its comparison with the CPU oracle last: that comparison leaves the GPU idle for
+    seconds, and after any idle gap, even 5 ms, the next ~25 passes of the SnapKV workload run at a lower shader
+    clock (2.4 ms falling to 1.9 ms), so nothing may separate the warm-up from the timed steps and as little as
+    possible the workload's set-up from the warm-up.
     `min_warm_s` keeps warming up until that much time has passed (used for the configurations whose warm-up count
     is this file's own choice, not the caller's)."""
     w = WORKLOADS[workload](seed, dev)
-    checked = None
+    checked = pending = None
     if check:                              # one step of its own, on the fresh pool
         w.check_before()
         w.step()
-        checked = w.check_after()          # raises when the sampled column is off: no number without a right result
+        pending = w.check_collect()        # evaluated below, after the timed steps, where it costs seconds of host work
     t_warm = _sync_time()
     done = 0
     while done < warmup or _sync_time() - t_warm < min_warm_s:
@@ -708,6 +726,8 @@ def measure(workload, seed, dev, steps, warmup, cpu_baseline=True, cpu_budget_s=
     t1 = _sync_time()
     ms_per_step = (t1 - t0) * 1e3 / steps
     value = w.tokens_per_step / (ms_per_step * 1e-3)
+    if pending is not None:
+        checked = pending()                # raises when the sampled column is off: no number without a right result
     # the rate once the clocks have settled: the same step for another ~0.3 s, not part of `value`
     sustained = None
     w.br.on = False
