@@ -664,7 +664,7 @@ WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkl
 #   copy:   FETCH_SIZE 2.623e5 KiB -> scale 1.999;  WRITE_SIZE 5.244e5 KiB -> scale 1.000
 # The commands and raw readings are in profiles/*_hbm_traffic.txt.
 _COUNTER_RUN = {"commit": "76bf753", "date": "2026-11-25"}   # the tree whose kernels the counter runs below measured
-# (cfg5's MLP launch keeps the first round's reading: this round's counter run of that workload ended in a host-side
+# (cfg5's MLP launch keeps an earlier reading, commit 3ee0b1a: the later counter run of that workload ended in a host-side
 #  crash of the profiled process inside the profiler's dispatch hook, while torch was still building the inputs)
 _COUNTER_RUN_OF = {"cfg5-ccm-hybrid-minicpm-v-2.6": {"commit": "3ee0b1a", "date": "2026-11-25"},
                    "cfg1-knorm-llama-7b": {"commit": "f22b65d", "date": "2026-11-25"},
