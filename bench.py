@@ -157,7 +157,7 @@ class SnapKVWorkload(Workload):
     kernel_name = "snapkv_kernel"
     one_launch = True              # scoring, selection and compaction of a column by one workgroup (fc_snapkv_press);
                                    # False: fc_snapkv_score, then fc_select_compact (shapes the press does not take)
-    separate_selection = False     # with one_launch False: fc_topk_select and fc_compact as two launches
+    separate_selection = False     # with one_launch False: fc_topk_select and fc_compact as launches of their own
 
     def __init__(self, seed, device, given_lse=False):
         super().__init__()
@@ -359,7 +359,7 @@ class KnormWorkload(Workload):
 
 
 class KnormThreeLaunchWorkload(KnormWorkload):
-    """The same pass as three launches (norms, top-k, compaction), the form sequences beyond 8192 tokens take."""
+    """The same pass as three launches (norms, top-k, compaction), the form that columns too long for LDS take."""
     name = "cfg1-knorm-llama-7b-three-launches"
     kernel_name = "compact_kernel"
 

@@ -10,7 +10,7 @@
 #include "fc_norm.h"
 #include "fc_press.h"
 
-#define KP_MAX_S 8192   // longest sequence: its scores and kept positions stay in LDS (64 KB)
+#define KP_MAX_LDS (144 * 1024)   // the column's scores and kept positions stay in LDS: 4 * (max_seq_len + index_stride) bytes
 #define KP_U 4          // key rows per lane in flight while scoring
 #define KP_WIDE_FROM 512   // sequences from this length on get 1024 threads per column, shorter ones 256
 
@@ -120,9 +120,10 @@ static int kp_check(const char* who, const fc_kv_view* keys, const fc_kv_view* v
              "%s: index_stride %d exceeds max_seq_len %d", who, index_stride, keys->max_seq_len);
   FC_REQUIRE(n_kept != nullptr || (k >= 0 && k <= index_stride), FC_EINVAL, "%s: k=%d vs index_stride=%d", who, k,
              index_stride);
-  FC_REQUIRE(keys->max_seq_len <= KP_MAX_S, FC_EUNSUPPORTED,
-             "%s: sequences of up to %d tokens (got %d); longer ones take fc_topk_select and fc_compact", who, KP_MAX_S,
-             keys->max_seq_len);
+  FC_REQUIRE(4LL * ((long long)keys->max_seq_len + index_stride) <= KP_MAX_LDS, FC_EUNSUPPORTED,
+             "%s: 4 * (max_seq_len + index_stride) = 4 * (%d + %d) bytes exceed the %d of LDS a column may take; such "
+             "shapes take the separate launches (fc_topk_select, fc_compact)", who, keys->max_seq_len, index_stride,
+             KP_MAX_LDS);
   FC_REQUIRE(keys->batch <= 65535 && keys->num_layers <= 65535, FC_EUNSUPPORTED, "%s: grid too large", who);
   return FC_OK;
 }
@@ -142,7 +143,7 @@ extern "C" int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, 
   // 1024 threads measured 11 % faster than 256 on 1024-token fp32 columns; short columns cannot feed that many.
 #define KP_LAUNCH(DT, TH)                                                                                        \
   do {                                                                                                           \
-    FC_ALLOW_LDS((knorm_press_kernel<DT, TH>), KP_MAX_S * 8);                                                     \
+    FC_ALLOW_LDS((knorm_press_kernel<DT, TH>), KP_MAX_LDS);                                                       \
     hipLaunchKernelGGL((knorm_press_kernel<DT, TH>), grid, dim3(TH), lds, st, kv, vv, scores, score_stride, k,   \
                        n_kept, indices, index_stride, smax);                                                     \
   } while (0)
@@ -173,7 +174,7 @@ extern "C" int fc_select_compact(const fc_kv_view* keys, const fc_kv_view* value
   hipStream_t st = (hipStream_t)stream;
 #define KP_LAUNCH(E, TH)                                                                                          \
   do {                                                                                                           \
-    FC_ALLOW_LDS((select_compact_kernel<E, TH>), KP_MAX_S * 8);                                                   \
+    FC_ALLOW_LDS((select_compact_kernel<E, TH>), KP_MAX_LDS);                                                     \
     hipLaunchKernelGGL((select_compact_kernel<E, TH>), grid, dim3(TH), lds, st, kv, vv, scores, score_stride, k, \
                        n_kept, indices, index_stride, smax);                                                     \
   } while (0)

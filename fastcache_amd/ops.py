@@ -263,7 +263,10 @@ def compact(src_k: FcKvView, src_v: FcKvView, dst_k: FcKvView, dst_v: FcKvView, 
           "fc_compact")
 
 
-KNORM_PRESS_MAX_SEQ = 8192      # longest sequence the one-launch Knorm press takes
+def press_column_fits(max_seq_len: int, k: int) -> bool:
+    """Whether :func:`knorm_press` / :func:`select_compact` take sequences of ``max_seq_len`` tokens keeping ``k``: a
+    column's scores and kept positions stay in LDS, ``4 * (max_seq_len + k)`` bytes of at most 144 KB."""
+    return 4 * (max_seq_len + k) <= 144 * 1024
 
 
 def knorm_press(keys: FcKvView, values: FcKvView, k: int, device, n_kept: Optional[torch.Tensor] = None,

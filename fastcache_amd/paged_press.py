@@ -40,7 +40,7 @@ def _select_and_compact(kview, vview, scores, seq_lens, kept: List[int], compact
     """Top-k per (layer, sequence, head) row and in-place compaction; one launch each whether or not the
     sequences keep the same number of tokens."""
     width = max(kept)
-    one_launch = (compact and width > 0 and kview.max_seq_len <= ops.KNORM_PRESS_MAX_SEQ and scores.dim() == 4 and
+    one_launch = (compact and width > 0 and ops.press_column_fits(kview.max_seq_len, width) and scores.dim() == 4 and
                   scores.shape[2] == kview.num_kv_heads and scores.is_contiguous())
     if one_launch:       # selection and compaction of a column by one workgroup
         if len(set(kept)) == 1:
@@ -69,7 +69,7 @@ def knorm_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, seq
     lens = list(host_lens) if host_lens is not None else [seq_len] * block_tables.shape[0]
     kept = [n_kept_for(n, compression_ratio) for n in lens]
     width = max(kept)
-    if compact and 0 < width and seq_len <= ops.KNORM_PRESS_MAX_SEQ:
+    if compact and 0 < width and ops.press_column_fits(seq_len, width):
         # one launch: every (layer, sequence, head) column is scored, selected and compacted by one workgroup
         if len(set(kept)) == 1:
             scores, idx = ops.knorm_press(kview, vview, width, kv_cache.device)

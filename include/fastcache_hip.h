@@ -197,8 +197,8 @@ int fc_topk_select(const float* scores, int32_t score_stride, int32_t rows, int3
  * Knorm press in one launch: fc_knorm_score, fc_topk_select (rows of one sequence keep n_kept[b] of their
  * seq_lens[b] scores, or `k` when n_kept is NULL) and fc_compact of `keys` and `values` onto themselves, for every
  * (layer, b, kv head) column, with the same scores, indices (entries past a row's kept count are left as they are)
- * and cache bytes as those three calls.  Sequences of up to 8192 tokens; longer views are refused with
- * FC_EUNSUPPORTED and take the three calls.
+ * and cache bytes as those three calls.  A column's scores and kept positions stay in LDS: views with
+ * 4 * (max_seq_len + index_stride) > 147456 bytes are refused with FC_EUNSUPPORTED and take the three calls.
  * Replaces, for KnormPress, the per-sequence loop extract -> press -> write back of
  * LlavaModelRunner.compress_kv_cache_batch (nanovllm/engine/llava_model_runner.py:745-786) with
  * kvpress KnormPress.score + ScorerPress.compress (third-party) inside.
@@ -211,7 +211,8 @@ int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, float* scor
  * (layer, b, kv head) row of scores[.., score_stride], fc_topk_select over the row's first seq_lens[b] entries
  * (keeping n_kept[b], or `k` when n_kept is NULL) and fc_compact of `keys` and `values` onto themselves with the row's
  * own indices, with the same indices (entries past a row's kept count are left as they are) and cache bytes as those
- * two calls.  Sequences of up to 8192 tokens; longer views are refused with FC_EUNSUPPORTED and take the two calls.
+ * two calls.  Views with 4 * (max_seq_len + index_stride) > 147456 bytes (the column's scores and kept positions stay
+ * in LDS) are refused with FC_EUNSUPPORTED and take the two calls.
  * Replaces scores.topk + gather of kvpress ScorerPress.compress (third-party) together with
  * LlavaModelRunner._write_compressed_kv_cache_fast (nanovllm/engine/llava_model_runner.py:874-912).
  */

@@ -79,6 +79,7 @@ def test_knorm_press_paged_inplace(dev, dtype, shape):
     ([300, 300], 64, [300, 299]),                 # keep everything / all but one
     ([2500, 130, 2049], 128, [1, 129, 700]),      # several pages, a single kept row
     ([193, 77], 48, [100, 33]),                   # pages whose size is not a power of two
+    ([20000, 9000], 256, [5000, 2250]),           # long sequences: 100 KB of LDS per column
 ])
 def test_knorm_press_one_launch_equals_three(dev, dtype, lens, block_size, keep):
     """fc_knorm_press against fc_knorm_score + fc_topk_select + fc_compact on the same pool: scores, indices and
@@ -117,6 +118,7 @@ def test_knorm_press_one_launch_equals_three(dev, dtype, lens, block_size, keep)
     ([300, 300], 64, [300, 299]),
     ([2500, 130, 2049], 128, [1, 129, 700]),
     ([193, 77], 48, [100, 33]),
+    ([30000, 12345], 256, [4000, 1700]),
 ])
 def test_select_compact_one_launch_equals_two(dev, dtype, lens, block_size, keep):
     """fc_select_compact against fc_topk_select + fc_compact on the same pool and the same scores (random, with
@@ -238,8 +240,9 @@ def test_knorm_press_one_launch_limits_and_clamps(dev):
     assert (row >= 0).all() and (row < S).all() and (row[1:] > row[:-1]).all()
     row = ib[0, 1, 1]
     assert (row[:40] >= 0).all() and (row[:40] < 50).all() and (row[40:] == -1).all()
-    big = torch.zeros((1, 1, 1, 8200, 128), device=dev)
-    with pytest.raises(_lib.FastcacheError, match="8192"):
+    big = torch.zeros((1, 1, 1, 40000, 128), device=dev)
+    assert not ops.press_column_fits(40000, 10) and ops.press_column_fits(32768, 4096)
+    with pytest.raises(_lib.FastcacheError, match="separate launches"):
         ops.knorm_press(_lib.dense_view(big), _lib.dense_view(big.clone()), 10, dev)
 
 
