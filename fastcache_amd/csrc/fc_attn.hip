@@ -89,13 +89,27 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
   const int G = Hq / Hkv;
   const int gtiles = (G + GT - 1) / GT;
   const int h = blockIdx.y / gtiles, g0 = (blockIdx.y - h * gtiles) * GT;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int t0 = split * chunk;
+  // The chunk's block-table entries, one per lane (a chunk of at most 1024 tokens in pages of at least 32 spans at
+  // most 33), fetched before anything waits for the sequence length: a tile's address then costs a lane read instead
+  // of a table load that the tile's own loads would have to wait for.
+  int ktbl = 0, vtbl = 0;
+  if constexpr (FAST) {
+    if (kc.block_tables) {
+      const int e = min((t0 >> kc.block_shift) + lane, kc.table_stride - 1);
+      ktbl = kc.block_tables[(long long)b * kc.table_stride + e];
+    }
+    if (vc.block_tables) {
+      const int e = min((t0 >> vc.block_shift) + lane, vc.table_stride - 1);
+      vtbl = vc.block_tables[(long long)b * vc.table_stride + e];
+    }
+  }
   int len = __builtin_amdgcn_readfirstlane(lens[b]);
   len = min(len, kc.max_seq_len);
-  const int t0 = split * chunk;
   if (t0 >= len) return;
   const int ntok = min(chunk, len - t0);
 
-  const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane & 31, lhalf = lane >> 5;
   const int sub = lane & 15, rg = lane >> 4;   // V rows: 16 lanes per row, 4 rows per pass
@@ -118,14 +132,14 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
   // writes LDS chunk i of the 64 chunks of those rows and fetches the global chunk (i & 15) ^ (row & 15)
   // of row i / 16 (XOR swizzle, so that the operand reads of 32 rows at the same chunk fall on
   // distinct banks).  Rows past the sequence end re-read its last row; their logits are masked.
-  auto issue = [&](const KvView& v, const char* base, int tile, int stage) {
+  auto issue = [&](const KvView& v, const char* base, int tile, int stage, int tbl_reg) {
     const int s0 = t0 + tile * DA_TILE;
     const unsigned dst = ring_lds + stage * DA_TILEB;
     const int rmax = len - 1 - s0;
     if constexpr (FAST) {
       long long tb;
       if (v.block_tables) {
-        const int blk = max(__builtin_amdgcn_readfirstlane(v.block_tables[(long long)b * v.table_stride + (s0 >> v.block_shift)]), 0);
+        const int blk = max(__builtin_amdgcn_readlane(tbl_reg, (s0 >> v.block_shift) - (t0 >> v.block_shift)), 0);
         tb = (long long)blk * v.stride_block + (long long)(s0 & (v.block_size - 1)) * v.stride_token;
       } else {
         tb = (long long)b * v.stride_batch + (long long)s0 * v.stride_token;
@@ -160,8 +174,8 @@ __global__ __launch_bounds__(DA_THREADS, 2) void decode_attn_kernel(KvView kc, K
   const int live_tiles = (ntok + DA_TILE - 1) / DA_TILE;
   const int nj = wave < live_tiles ? (live_tiles - wave + 3) / 4 : 0;   // wave-uniform
   auto issue_item = [&](int i) {
-    if (i < nj) issue(kc, kbase, wave + 4 * i, i & 1);
-    else if (i < 2 * nj) issue(vc, vbase, wave + 4 * (i - nj), i & 1);
+    if (i < nj) issue(kc, kbase, wave + 4 * i, i & 1, ktbl);
+    else if (i < 2 * nj) issue(vc, vbase, wave + 4 * (i - nj), i & 1, vtbl);
   };
   // item i has landed when at most the loads of item i + 1 (eight per lane) are outstanding
   auto wait_item = [&](int i) {
