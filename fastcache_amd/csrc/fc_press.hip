@@ -14,6 +14,18 @@
 #define KP_U 4          // key rows per lane in flight while scoring
 #define KP_WIDE_FROM 512   // sequences from this length on get 1024 threads per column, shorter ones 256
 
+// Which column a workgroup takes.  Workgroups go to the eight XCDs round-robin in launch order; columns that follow each
+// other in memory (the heads of a sequence, whose rows of one token are adjacent) are given to the same XCD, one after
+// the other, when the column count is a multiple of eight (cfg1: -1.5 %; no effect on the 256-byte rows of cfg2).
+__device__ __forceinline__ void kp_column(int& h, int& b, int& l, int H, int B, int L) {
+  const long long n = (long long)H * B * L;
+  const long long id = blockIdx.x + (long long)gridDim.x * (blockIdx.y + (long long)gridDim.y * blockIdx.z);
+  const long long col = (n % 8) == 0 ? (id % 8) * (n / 8) + id / 8 : id;
+  h = (int)(col % H);
+  b = (int)((col / H) % B);
+  l = (int)(col / ((long long)H * B));
+}
+
 template <int DTYPE, int THREADS>
 __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView vv, float* __restrict__ scores,
                                                               int score_stride, int k, const int* __restrict__ n_kept,
@@ -26,7 +38,8 @@ __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView 
   __shared__ int ktbl[CP_TBL], vtbl[CP_TBL];
   __shared__ TkShared<THREADS> sh;
 
-  const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
+  int h, b, l;
+  kp_column(h, b, l, kv.num_kv_heads, kv.batch, kv.num_layers);
   const int H = kv.num_kv_heads;
   const int tid = threadIdx.x, sub = tid % LPR, rg = tid / LPR;
   const int S = min(fc_seq_len(kv, b), smax);
@@ -83,7 +96,8 @@ __global__ __launch_bounds__(THREADS) void select_compact_kernel(KvView kv, KvVi
   int* sel = reinterpret_cast<int*>(sc + smax);
   __shared__ int ktbl[CP_TBL], vtbl[CP_TBL];
   __shared__ TkShared<THREADS> sh;
-  const int h = blockIdx.x, b = blockIdx.y, l = blockIdx.z;
+  int h, b, l;
+  kp_column(h, b, l, kv.num_kv_heads, kv.batch, kv.num_layers);
   const int tid = threadIdx.x;
   const int S = min(fc_seq_len(kv, b), smax);
   int kk = n_kept ? n_kept[b] : k;
