@@ -121,12 +121,14 @@ class Workload:
         return lambda: result
 
 
-def _column_dense(kv_cache, plane, layer, table, n):
-    """Tokens [0, n) of one sequence of one layer as a CPU tensor [1, Hkv, n, D] (HuggingFace layout)."""
+def _column_dense(kv_cache, plane, layer, table, n, cpu=True):
+    """Tokens [0, n) of one sequence of one layer as a tensor [1, Hkv, n, D] (HuggingFace layout), on the CPU or, for
+    a snapshot that must not make the GPU wait for the host, as a copy on the device."""
     bs = kv_cache.shape[3]
     blocks = torch.as_tensor(list(table)[:(n + bs - 1) // bs], device=kv_cache.device, dtype=torch.long)
     rows = kv_cache[plane, layer, blocks].reshape(-1, kv_cache.shape[4], kv_cache.shape[5])[:n]
-    return rows.permute(1, 0, 2).unsqueeze(0).cpu()
+    rows = rows.permute(1, 0, 2).unsqueeze(0)
+    return rows.cpu() if cpu else rows.contiguous()
 
 
 def _check_press_column(name, before_k, before_v, after_k, after_v, scores, ref_scores, idx, n_scored):
@@ -246,24 +248,26 @@ class SnapKVWorkload(Workload):
             self.kept, self.keep = (scores, idx), False
 
     def check_before(self):
+        # snapshots stay on the device until the comparison: no host copy, hence no idle GPU, before the timed steps
         self.cl, self.cb = self.L // 2, self.B // 2
         tab = self.case.block_tables[self.cb]
-        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
+        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S, cpu=False) for p in range(2)]
         self.keep = True
 
     def check_collect(self):
         scores, idx = self.kept
         l, b = self.cl, self.cb
         tab = self.case.block_tables[b]
-        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]    # before any later step
-        sc, ix, q = scores[l, b].cpu(), idx[l, b].cpu(), self.queries[l, b:b + 1].cpu()
+        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept, cpu=False) for p in range(2)]   # before any later step
+        sc, ix, q = scores[l, b].clone(), idx[l, b].clone(), self.queries[l, b:b + 1]
         self.kept = None
 
         def evaluate():
             from oracle import presses as opress
-            ref = opress.snapkv_score(q, self.snap[0], self.W, self.ksz, True, "sum")[0]
-            return _check_press_column(f"layer {l}, sequence {b}", self.snap[0], self.snap[1], after[0], after[1],
-                                       sc, ref, ix, self.S - self.W)
+            snap = [t.cpu() for t in self.snap]
+            ref = opress.snapkv_score(q.cpu(), snap[0], self.W, self.ksz, True, "sum")[0]
+            return _check_press_column(f"layer {l}, sequence {b}", snap[0], snap[1], after[0].cpu(), after[1].cpu(),
+                                       sc.cpu(), ref, ix.cpu(), self.S - self.W)
         return evaluate
 
     def cpu_baseline(self, budget_s=12.0):
@@ -328,21 +332,22 @@ class KnormWorkload(Workload):
     def check_before(self):
         self.cl = self.L // 2
         tab = self.case.block_tables[0]
-        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S) for p in range(2)]
+        self.snap = [_column_dense(self.case.kv_cache, p, self.cl, tab, self.S, cpu=False) for p in range(2)]
         self.keep = True
 
     def check_collect(self):
         scores, idx = self.kept
         l = self.cl
         tab = self.case.block_tables[0]
-        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept) for p in range(2)]    # before any later step
-        sc, ix = scores[l, 0].cpu(), idx[l, 0].cpu()
+        after = [_column_dense(self.case.kv_cache, p, l, tab, self.n_kept, cpu=False) for p in range(2)]   # before any later step
+        sc, ix = scores[l, 0].clone(), idx[l, 0].clone()
         self.kept = None
 
         def evaluate():
             from oracle import presses as opress
-            return _check_press_column(f"layer {l}, sequence 0", self.snap[0], self.snap[1], after[0], after[1],
-                                       sc, opress.knorm_score(self.snap[0])[0], ix, self.S)
+            snap = [t.cpu() for t in self.snap]
+            return _check_press_column(f"layer {l}, sequence 0", snap[0], snap[1], after[0].cpu(), after[1].cpu(),
+                                       sc.cpu(), opress.knorm_score(snap[0])[0], ix.cpu(), self.S)
         return evaluate
 
     def cpu_baseline(self, budget_s=12.0):
