@@ -96,9 +96,14 @@ def snapkv_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, se
     if not window_in_budget:
         kept = [min(n, k + window_size) for n, k in zip(lens, kept)]
     width = max(kept)
-    # the workgroup that scored a column also selects and compacts it when every row keeps more than the window
-    # (sequences no longer than the window keep their first positions either way)
+    # The workgroup that scored a column also selects and compacts it when every row keeps more than the window
+    # (sequences no longer than the window keep their first positions either way).  In that launch the window positions
+    # rank above every scored key, while after the window fill they TIE with scored keys that equal the layer's largest
+    # score; the two selections differ only when more such keys than a row has places outside the window tie exactly,
+    # which needs equal scores at the very top: rows with fewer scored keys than the pooling kernel is wide (every pooled
+    # score the same) take the separate launches.
     if (compact and all(k > window_size or n <= window_size for n, k in zip(lens, kept)) and width > window_size and
+            all(n <= window_size or n - window_size > kernel_size for n in lens) and
             ops.snapkv_press_fits(kview, queries.shape[-3], window_size, width) and
             ops.snapkv_splits(kview, queries.shape[-3], window_size) == 1):   # few columns: key ranges pay more
         same = len(set(kept)) == 1 and len(set(lens)) == 1

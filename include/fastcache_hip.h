@@ -136,8 +136,10 @@ int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float
  * SnapKV press in one launch: fc_snapkv_score (or fc_snapkv_score_lse when `lse` is not NULL) and, by the same
  * workgroup that scored a (layer, b, kv head) column, the selection of the column's kept positions and the compaction
  * of `keys` and `values` onto themselves.  Kept counts (k, or n_kept[b] in device memory) include the window and must
- * exceed it: the window positions rank first, as they do after fc_snapkv_fill_window, so the indices and cache bytes
- * are those of fc_snapkv_score + fc_snapkv_fill_window + fc_topk_select + fc_compact.  `scores` receives the scored
+ * exceed it: the window positions rank first, so the indices and cache bytes are those of fc_snapkv_score +
+ * fc_snapkv_fill_window + fc_topk_select + fc_compact, except where scored keys tie EXACTLY with the layer's largest
+ * score and are more than the row keeps outside the window (after the fill such keys tie with the window positions and
+ * the lower index wins; here the window wins).  `scores` receives the scored
  * positions and `row_max` (required) the per-row maxima; the caller runs fc_snapkv_fill_window afterwards if it wants
  * the window entries of `scores` filled.  Rows of sequences no longer than the window keep their first positions.
  * Takes dense views or pages of 64*2^n tokens and sequences short enough for the score row and the kept positions to

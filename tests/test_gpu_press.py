@@ -195,6 +195,24 @@ def test_snapkv_press_one_launch_equals_separate(dev, dtype, lens, Hq, H, W, ksz
     assert not torch.equal(pool_b.view(torch.uint8), case.kv_cache.to(dev).view(torch.uint8))
 
 
+def test_snapkv_paged_press_tiny_scored_part_takes_separate_launches(dev):
+    """Six scored keys under a pooling kernel of 13: every pooled score is the same and equals the layer's largest, so
+    after the window fill all 38 positions tie and the lowest indices win (position 37, a window position, is the one
+    dropped).  The one-launch press ranks the window first and would drop a scored key instead; the host sends such
+    rows through the separate launches."""
+    L, H, Hq, W, ksz, n = 2, 1, 4, 32, 13, 38
+    case = synth.make_paged_case(seed=523480996, num_layers=L, batch=1, num_kv_heads=H, seq_lens=[n], dtype=torch.bfloat16,
+                                 num_q_heads=Hq, window=W, block_size=64)
+    pool = case.kv_cache.to(dev)
+    res = paged_press.snapkv_compress_paged(pool, case.table_tensor(dev), case.lens_tensor(dev), n, case.queries.to(dev),
+                                            1.0 - 37.5 / 38, W, ksz, True, "sum")
+    torch.cuda.synchronize()
+    assert res.n_kept == 37
+    scored = res.scores[..., :n - W]
+    assert bool((scored == scored[..., :1]).all())                       # the degenerate tie is really there
+    assert torch.equal(res.indices[0, 0, 0].cpu(), torch.arange(37, dtype=torch.int32))
+
+
 def test_snapkv_press_refuses_what_it_cannot_take(dev):
     case = synth.make_paged_case(seed=2, num_layers=1, batch=1, num_kv_heads=1, seq_lens=[512], dtype=torch.bfloat16,
                                  num_q_heads=4, window=64)
