@@ -775,7 +775,7 @@ extern "C" int fc_snapkv_press(const fc_kv_view* keys, const fc_kv_view* values,
                                int32_t k, const int32_t* n_kept, int32_t* indices, int32_t index_stride,
                                void* stream) {
   const char* who = "fc_snapkv_press";
-  FC_REQUIRE(values, FC_EINVAL, "%s: null value view", who);
+  FC_REQUIRE(values && row_max, FC_EINVAL, "%s: null value view or row_max", who);
   return snapkv_score_impl(who, keys, queries, num_q_heads, window, kernel_size, causal_window, scale, out_scale,
                            scores, score_stride, row_max, lse, stream, values, k, n_kept, indices, index_stride);
 }
