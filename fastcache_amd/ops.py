@@ -158,6 +158,23 @@ def snapkv_press_fits(keys: FcKvView, num_q_heads: int, window: int, index_strid
                 0 <= keys.stride_token < (1 << 24))
 
 
+def snapkv_press_preferred(keys: FcKvView, num_q_heads: int, window: int, compute_units: int = 256) -> bool:
+    """Whether the one-launch press (whole columns) or split scoring (:func:`snapkv_splits` key ranges per column, then
+    ``select_compact``) is the faster form for a shape both take.  Whole columns cost ``rounds x column time`` with
+    ``rounds = ceil(columns / workgroups the GPU holds)`` (two per compute unit, one with 16 wavefronts), split scoring
+    grows linearly with the columns but pays a merge, a pooling and a compaction launch.  Measured on MI355X (28 x B x 4
+    and 36 x B x 8 columns of 4096 to 12000 keys): whole columns win or tie when the last round is at least 80 % full
+    or the columns are short (up to 4096 keys: 0.62 against 0.75 ms at 448 columns, 0.93 against 1.04 at 672, at worst
+    2.5 % behind); long columns in poorly filled rounds lose (320 x 12000: 1.67 against 1.40 ms)."""
+    if snapkv_splits(keys, num_q_heads, window) == 1:
+        return True
+    columns = keys.num_layers * keys.batch * keys.num_kv_heads
+    blocks = (num_q_heads // keys.num_kv_heads) * ((window + 31) // 32)
+    slots = compute_units * (2 if blocks <= 8 else 1)
+    rounds = -(-columns // slots)
+    return keys.max_seq_len <= 4096 or columns >= 0.8 * rounds * slots
+
+
 def snapkv_press(keys: FcKvView, values: FcKvView, queries: torch.Tensor, window: int, kernel_size: int, k: int,
                  causal_window: bool = True, reduction: str = "mean", scale: Optional[float] = None,
                  seq_lens: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,

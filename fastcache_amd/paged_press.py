@@ -105,7 +105,8 @@ def snapkv_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, se
     if (compact and all(k > window_size or n <= window_size for n, k in zip(lens, kept)) and width > window_size and
             all(n <= window_size or n - window_size > kernel_size for n in lens) and
             ops.snapkv_press_fits(kview, queries.shape[-3], window_size, width) and
-            ops.snapkv_splits(kview, queries.shape[-3], window_size) == 1):   # few columns: key ranges pay more
+            ops.snapkv_press_preferred(kview, queries.shape[-3], window_size,
+                                       torch.cuda.get_device_properties(kv_cache.device).multi_processor_count)):
         same = len(set(kept)) == 1 and len(set(lens)) == 1
         n_kept = None if same else torch.tensor(kept, dtype=torch.int32, device=kv_cache.device)
         scores, idx = ops.snapkv_press(kview, vview, queries, window_size, kernel_size, width, causal_window,

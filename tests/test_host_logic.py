@@ -348,6 +348,14 @@ def test_snapkv_split_heuristic():
     assert ops.snapkv_splits(view(36, 1, 8, 32768, block_size=48), 32, 64) == 1
     assert ops.snapkv_splits(view(36, 1, 8, 32768, paged=False), 32, 64) == 8
     assert ops.snapkv_splits(view(4, 1, 1, 32768), 32, 64) == 1          # 64 row blocks per kv head
+    # whole columns in one launch, or key ranges: by how full the last round of workgroups is, and the column length
+    pref = lambda v, hq: ops.snapkv_press_preferred(v, hq, 64, compute_units=256)
+    assert pref(view(36, 8, 8, 4096), 32)                                 # no split in question
+    assert pref(view(28, 4, 4, 4096), 28) and pref(view(28, 5, 4, 4096), 28)      # short columns
+    assert pref(view(32, 4, 8, 8192), 32)                                 # 1024 columns: two full rounds
+    assert pref(view(28, 8, 4, 8192), 28)                                 # 896 columns of 16 wavefronts: 3.5 rounds of 256
+    assert not pref(view(36, 1, 8, 8192), 32)                             # 288 long columns in a round of 512
+    assert not pref(view(40, 1, 8, 12000), 40)                            # 320 columns of 12000 keys
 
 
 def test_bench_counter_table_names_real_workloads():
