@@ -12,7 +12,13 @@
 
 #define KP_MAX_LDS (144 * 1024)   // the column's scores and kept positions stay in LDS: 4 * (max_seq_len + index_stride) bytes
 #define KP_U 4          // key rows per lane in flight while scoring
-#define KP_WIDE_FROM 512   // sequences from this length on get 1024 threads per column, shorter ones 256
+// 1024 threads per column from this many bytes of key rows per column on, 256 below.  More lanes finish a column sooner
+// (more rows in flight per column, fewer columns half done at any time) but idle through a short column's selection.
+// Measured, 1024 against 256 threads: the Knorm press 0.292 / 0.323 ms (1024 columns x 1024 fp32 rows), 1.166 / 1.313 ms
+// (4096 x 2048 bf16), 0.601 / 0.629 (4096 x 1024 bf16), 1.364 / 1.099 (16384 x 512 bf16), 3.67 / 1.15 (65536 x 128);
+// selection + compaction alone 0.934 / 0.956 (2048 x 4096 bf16), 0.933 / 0.915 (4096 x 2048), 1.123 / 0.881 (16384 x 512).
+#define KP_WIDE_BYTES_PRESS (384 * 1024)
+#define KP_WIDE_BYTES_SELECT (1024 * 1024)
 
 // Which column a workgroup takes.  Workgroups go to the eight XCDs round-robin in launch order; columns that follow each
 // other in memory (the heads of a sequence, whose rows of one token are adjacent) are given to the same XCD, one after
@@ -153,16 +159,15 @@ extern "C" int fc_knorm_press(const fc_kv_view* keys, const fc_kv_view* values, 
   const size_t lds = ((size_t)smax + (size_t)index_stride) * 4;
   dim3 grid(keys->num_kv_heads, keys->batch, keys->num_layers);
   hipStream_t st = (hipStream_t)stream;
-  // A column is finished sooner by more lanes (more rows in flight per column, fewer columns half done at any time):
-  // 1024 threads measured 11 % faster than 256 on 1024-token fp32 columns; short columns cannot feed that many.
 #define KP_LAUNCH(DT, TH)                                                                                        \
   do {                                                                                                           \
     FC_ALLOW_LDS((knorm_press_kernel<DT, TH>), KP_MAX_LDS);                                                       \
     hipLaunchKernelGGL((knorm_press_kernel<DT, TH>), grid, dim3(TH), lds, st, kv, vv, scores, score_stride, k,   \
                        n_kept, indices, index_stride, smax);                                                     \
   } while (0)
+  const bool wide = (long long)smax * FC_HEAD_DIM * fc_elem_bytes(keys->dtype) >= KP_WIDE_BYTES_PRESS;
 #define KP_DISPATCH(DT) \
-  if (smax >= KP_WIDE_FROM) KP_LAUNCH(DT, 1024); else KP_LAUNCH(DT, 256)
+  if (wide) KP_LAUNCH(DT, 1024); else KP_LAUNCH(DT, 256)
   switch (keys->dtype) {
     case FC_F32: KP_DISPATCH(FC_F32); break;
     case FC_F16: KP_DISPATCH(FC_F16); break;
@@ -192,10 +197,11 @@ extern "C" int fc_select_compact(const fc_kv_view* keys, const fc_kv_view* value
     hipLaunchKernelGGL((select_compact_kernel<E, TH>), grid, dim3(TH), lds, st, kv, vv, scores, score_stride, k, \
                        n_kept, indices, index_stride, smax);                                                     \
   } while (0)
+  const bool wide = (long long)smax * FC_HEAD_DIM * fc_elem_bytes(keys->dtype) >= KP_WIDE_BYTES_SELECT;
   if (keys->dtype == FC_F32) {
-    if (smax >= KP_WIDE_FROM) KP_LAUNCH(4, 1024); else KP_LAUNCH(4, 256);
+    if (wide) KP_LAUNCH(4, 1024); else KP_LAUNCH(4, 256);
   } else {
-    if (smax >= KP_WIDE_FROM) KP_LAUNCH(2, 1024); else KP_LAUNCH(2, 256);
+    if (wide) KP_LAUNCH(2, 1024); else KP_LAUNCH(2, 256);
   }
 #undef KP_LAUNCH
   FC_CHECK_LAUNCH(who);
