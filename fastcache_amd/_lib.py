@@ -90,6 +90,7 @@ SIGNATURES = {
     "fc_observed_attention_workspace_bytes": (C.c_int64, [_I, _I, _I]),
     "fc_observed_attention_score": (C.c_int, [_VP, _I, _I, _I, _I, _I, _I, _VP, _VP, C.c_int64, _VP]),
     "fc_copy_tokens": (C.c_int, [_V, _V, _I, _I, _I, _VP]),
+    "fc_copy_tokens_from_layers": (C.c_int, [_VP, _V, _V, _I, _I, _I, _VP]),
     "fc_store_kv": (C.c_int, [_V, _V, _VP, _VP, _VP, _VP]),
     "fc_store_kv_slots": (C.c_int, [_VP, C.c_int64, _VP, C.c_int64, _VP, _VP, _VP, _I, _I, _I, _VP]),
     "fc_advance_lens": (C.c_int, [_VP, _I, _I, _VP]),

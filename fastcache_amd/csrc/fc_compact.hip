@@ -16,10 +16,16 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
                                                              const int* __restrict__ indices,
                                                              int index_stride, int heads_in_index,
                                                              int k, const int* __restrict__ n_kept,
-                                                             int src_start, int dst_start) {
+                                                             int src_start, int dst_start,
+                                                             const char* const* __restrict__ src_layers,
+                                                             int rows_per_piece) {
   constexpr int LPR = FC_HEAD_DIM * EB / 16;
   __shared__ int stbl[CP_TBL], dtbl[CP_TBL];
-  const int h0 = blockIdx.x * HG, b = blockIdx.y;
+  // rows_per_piece > 0 (plain copies between buffers that cannot overlap): a column is cut into pieces of that many
+  // rows, one workgroup each, so that a few long columns still fill the GPU; blockIdx.x = piece * head groups + head group
+  const int head_groups = sk.num_kv_heads / HG;
+  const int piece = rows_per_piece > 0 ? (int)blockIdx.x / head_groups : 0;
+  const int h0 = (rows_per_piece > 0 ? (int)blockIdx.x % head_groups : (int)blockIdx.x) * HG, b = blockIdx.y;
   const int L = sk.num_layers;
   const int l = blockIdx.z % L;
   const bool is_v = blockIdx.z >= L;
@@ -33,6 +39,12 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   if (GATHER) n = min(n, index_stride);
   else n = min(n, S - src_start);
   n = min(n, dst.max_seq_len - dst_start);
+  if (!GATHER && rows_per_piece > 0) {     // this workgroup's piece of the range
+    const int first = piece * rows_per_piece;
+    src_start += first;
+    dst_start += first;
+    n = min(n - first, rows_per_piece);
+  }
   if (n <= 0) return;
 
   // block-table rows of this sequence (source and destination views may differ)
@@ -51,7 +63,9 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   const int* idx = GATHER ? indices + (((long long)l * sk.batch + b) * heads_in_index + (h % heads_in_index)) *
                                           (long long)index_stride
                           : nullptr;
-  const char* sbase = src.base + ((long long)l * src.stride_layer + (long long)h * src.stride_head) * EB + sub * 16;
+  // the source's layers may be tensors of their own (a list of per-layer tensors): their addresses then come from a table
+  const char* slayer = src_layers ? src_layers[l] : src.base + (long long)l * src.stride_layer * EB;
+  const char* sbase = slayer + (long long)h * src.stride_head * EB + sub * 16;
   char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * EB + sub * 16;
   cp_walk<EB, HG, CP_THREADS>(src, dst, stbl, s_lds, dtbl, d_lds, b, S, n, sbase, dbase, src.base + sub * 16, dst_start,
                               [&](int j) { return GATHER ? idx[j] : src_start + j; });
@@ -91,23 +105,22 @@ extern "C" int fc_compact(const fc_kv_view* src_k, const fc_kv_view* src_v, cons
   if (src_k->dtype == FC_F32 && src_k->num_kv_heads % 2 == 0 && cols >= 2048) {
     dim3 grid(src_k->num_kv_heads / 2, src_k->batch, src_k->num_layers * 2);
     hipLaunchKernelGGL((compact_kernel<4, true, 2>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
-                       index_stride, heads_in_index, k, n_kept, 0, 0);
+                       index_stride, heads_in_index, k, n_kept, 0, 0, nullptr, 0);
   } else {
     dim3 grid(src_k->num_kv_heads, src_k->batch, src_k->num_layers * 2);
     if (src_k->dtype == FC_F32)
       hipLaunchKernelGGL((compact_kernel<4, true, 1>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
-                         index_stride, heads_in_index, k, n_kept, 0, 0);
+                         index_stride, heads_in_index, k, n_kept, 0, 0, nullptr, 0);
     else
       hipLaunchKernelGGL((compact_kernel<2, true, 1>), grid, dim3(CP_THREADS), 0, st, sk, sv, dk, dv, indices,
-                         index_stride, heads_in_index, k, n_kept, 0, 0);
+                         index_stride, heads_in_index, k, n_kept, 0, 0, nullptr, 0);
   }
   FC_CHECK_LAUNCH(who);
   return FC_OK;
 }
 
-extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int32_t seg_start, int32_t count,
-                              int32_t dst_start, void* stream) {
-  const char* who = "fc_copy_tokens";
+static int copy_tokens_impl(const char* who, const void* const* src_layers, const fc_kv_view* src, const fc_kv_view* dst,
+                            int32_t seg_start, int32_t count, int32_t dst_start, void* stream) {
   int rc;
   if ((rc = fc_check_view(src, who)) || (rc = fc_check_view(dst, who)) || (rc = check_pair(src, dst, who)))
     return rc;
@@ -117,15 +130,41 @@ extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int3
              dst->max_seq_len);
   if (count == 0) return FC_OK;
   KvView s = fc_make_view(src), d = fc_make_view(dst);
+  // A pool and a dense tensor (or a list of per-layer tensors) do not overlap, so the order of the rows does not matter
+  // and a long column can be cut into pieces: enough of them for about eight workgroups per compute unit, none
+  // shorter than 512 rows.
+  int rows_per_piece = 0, pieces = 1;
+  if (src_layers || (src->block_tables == nullptr) != (dst->block_tables == nullptr)) {
+    const long long cols = (long long)src->num_kv_heads * src->batch * src->num_layers;
+    const long long want = (2048 + cols - 1) / cols;
+    pieces = (int)(want < 1 ? 1 : (want > (count + 511) / 512 ? (count + 511) / 512 : want));
+    if (pieces > 1) {
+      rows_per_piece = (count + pieces - 1) / pieces;
+      pieces = (count + rows_per_piece - 1) / rows_per_piece;
+    }
+  }
   // one plane per launch: z covers the layers only
-  dim3 grid(src->num_kv_heads, src->batch, src->num_layers);
+  dim3 grid(src->num_kv_heads * pieces, src->batch, src->num_layers);
   hipStream_t st = (hipStream_t)stream;
   if (src->dtype == FC_F32)
     hipLaunchKernelGGL((compact_kernel<4, false, 1>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
-                       nullptr, seg_start, dst_start);
+                       nullptr, seg_start, dst_start, (const char* const*)src_layers, rows_per_piece);
   else
     hipLaunchKernelGGL((compact_kernel<2, false, 1>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
-                       nullptr, seg_start, dst_start);
+                       nullptr, seg_start, dst_start, (const char* const*)src_layers, rows_per_piece);
   FC_CHECK_LAUNCH(who);
   return FC_OK;
+}
+
+extern "C" int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst, int32_t seg_start, int32_t count,
+                              int32_t dst_start, void* stream) {
+  return copy_tokens_impl("fc_copy_tokens", nullptr, src, dst, seg_start, count, dst_start, stream);
+}
+
+extern "C" int fc_copy_tokens_from_layers(const void* const* src_layers, const fc_kv_view* src, const fc_kv_view* dst,
+                                          int32_t seg_start, int32_t count, int32_t dst_start, void* stream) {
+  const char* who = "fc_copy_tokens_from_layers";
+  FC_REQUIRE(src_layers, FC_EINVAL, "%s: null layer table", who);
+  FC_REQUIRE(src && src->block_tables == nullptr, FC_EINVAL, "%s: the per-layer tensors must be dense", who);
+  return copy_tokens_impl(who, src_layers, src, dst, seg_start, count, dst_start, stream);
 }

@@ -87,8 +87,11 @@ class PagedKVRunner:
             return
         tt, ll = self._table_and_lens([table], [C])
         for p in range(2):
-            src = torch.stack([kv[p] for kv in compressed_kv])        # [L, 1, Hkv, C, D]
-            ops.copy_tokens(_lib.dense_view(src), _lib.paged_view(self.kv_cache[p], tt, ll, C), 0, C, 0)
+            dst = _lib.paged_view(self.kv_cache[p], tt, ll, C)
+            layers = [kv[p] for kv in compressed_kv]
+            if not ops.copy_tokens_from_layers(layers, dst, C):      # one launch straight from the list
+                src = torch.stack(layers)                             # [L, 1, Hkv, C, D]: tensors of mixed geometry
+                ops.copy_tokens(_lib.dense_view(src), dst, 0, C, 0)
 
     # -- compression ---------------------------------------------------------------------------------
     def _active_compressor(self):

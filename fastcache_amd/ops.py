@@ -329,6 +329,24 @@ def copy_tokens(src: FcKvView, dst: FcKvView, seg_start: int, count: int, dst_st
           "fc_copy_tokens")
 
 
+def copy_tokens_from_layers(layers, dst: FcKvView, count: int, dst_start: int = 0) -> bool:
+    """Tokens ``[0, count)`` of a list of per-layer tensors ``[B, Hkv, C, D]`` (one per layer of ``dst``, all of one
+    shape, dtype and stride pattern) -> ``dst`` tokens ``[dst_start, dst_start + count)``, in one launch and without
+    stacking the list.  Returns False (nothing done) when the tensors do not share one geometry."""
+    first = layers[0]
+    if len(layers) != dst.num_layers or any(t.shape != first.shape or t.stride() != first.stride() or t.dtype != first.dtype
+                                            or t.device != first.device for t in layers):
+        return False
+    _lib.require_gpu(first, "layer tensor")
+    view = _lib.dense_view(first)
+    view.num_layers = len(layers)
+    table = torch.tensor([t.data_ptr() for t in layers], dtype=torch.int64, pin_memory=True).to(first.device,
+                                                                                                 non_blocking=True)
+    check(fn("fc_copy_tokens_from_layers")(table.data_ptr(), C.byref(view), C.byref(dst), 0, count, dst_start,
+                                           current_stream()), "fc_copy_tokens_from_layers")
+    return True
+
+
 # ---------------------------------------------------------------------------------------------
 # CCM MLP
 # ---------------------------------------------------------------------------------------------

@@ -395,10 +395,21 @@ int fc_dequantize_group4(const uint8_t* packed, const void* scale, int64_t group
 /*
  * Plain ordered token copy src[seg_start + i] -> dst[dst_start + i], i < count, per
  * (layer, b, head); the pass-through branch of compress_layer when seg_len/cf < min_seq_len
- * (module_ccm_v11.py:674-675).  dst may alias src when dst_start <= seg_start.
+ * (module_ccm_v11.py:674-675).  dst may alias src when dst_start <= seg_start and both views are of one kind
+ * (both paged or both dense); a paged and a dense view must not overlap (their rows are copied in no particular order).
  */
 int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst,
                    int32_t seg_start, int32_t count, int32_t dst_start, void* stream);
+
+/*
+ * The same copy from a source whose layers are tensors of their own (the list of per-layer (K, V) tensors a
+ * HuggingFace-style compressor returns): src_layers[l] (a table of src->num_layers addresses in DEVICE memory) is the
+ * address of layer l's tensor, all of the one geometry `src` describes (dense, its base = the address of layer 0, its
+ * stride_layer unused).  Replaces the per-layer loop of LlavaModelRunner._write_compressed_kv_cache_fast
+ * (nanovllm/engine/llava_model_runner.py:874-912) without first stacking the layers into one tensor.
+ */
+int fc_copy_tokens_from_layers(const void* const* src_layers, const fc_kv_view* src, const fc_kv_view* dst,
+                               int32_t seg_start, int32_t count, int32_t dst_start, void* stream);
 
 /*
  * Append one new K/V row per sequence: cache[block_tables[b][len_b / bs]][len_b % bs] <- k_new[b], v_new[b]

@@ -310,6 +310,35 @@ def test_runner_compress_free_and_decode(dev, backend):
     assert ctx.slot_mapping.tolist() == exp_slots and ctx.block_tables.shape[0] == 3
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_extract_and_write_back_of_layer_lists(dev, dtype):
+    """_extract_kv_cache_fast / _write_compressed_kv_cache_fast against the oracle's paged copies: the write-back takes
+    the compressor's list of per-layer tensors as it is (slices of larger tensors: one launch from a table of layer
+    addresses) and falls back to stacking when the tensors do not share one geometry; slots past C keep their bytes."""
+    L, H, S, C, bs = 3, 2, 300, 117, 64
+    case = synth.make_paged_case(seed=4, num_layers=L, batch=2, num_kv_heads=H, seq_lens=[S, 200], dtype=dtype, block_size=bs)
+    r = PagedKVRunner(L, H, 128, case.kv_cache.shape[2], dtype, dev, block_size=bs)
+    r.kv_cache.copy_(case.kv_cache.to(dev))
+    table = case.block_tables[0]
+    hf = r._extract_kv_cache_fast(table, S)
+    ref = opaged.extract_kv(case.kv_cache, table, S)
+    for (k, v), (rk, rv) in zip(hf, ref):
+        assert torch.equal(k.cpu(), rk) and torch.equal(v.cpu(), rv)
+    g = torch.Generator().manual_seed(9)
+    wide = [(torch.randn(1, H, S, 128, generator=g).to(dtype).to(dev), torch.randn(1, H, S, 128, generator=g).to(dtype).to(dev))
+            for _ in range(L)]
+    for variant in ("slices", "mixed"):
+        comp = [(k[:, :, :C], v[:, :, :C]) for k, v in wide]                  # non-contiguous, one geometry
+        if variant == "mixed":
+            comp[1] = (comp[1][0].contiguous(), comp[1][1].contiguous())       # one layer laid out differently
+        pool = case.kv_cache.clone()
+        opaged.write_back(pool, [(k.cpu(), v.cpu()) for k, v in comp], table)
+        r.kv_cache.copy_(case.kv_cache.to(dev))
+        r._write_compressed_kv_cache_fast(comp, table)
+        torch.cuda.synchronize()
+        assert torch.equal(r.kv_cache.cpu().view(torch.uint8), pool.view(torch.uint8)), variant
+
+
 def test_background_compression_event_protocol(dev):
     dtype, L, H, S = torch.bfloat16, 2, 2, 600
     case = synth.make_paged_case(seed=4, num_layers=L, batch=2, num_kv_heads=H, seq_lens=[S, S], dtype=dtype,
