@@ -700,6 +700,10 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
     FC_REQUIRE(press_n_kept != nullptr || (press_k > window && press_k <= press_index_stride), FC_EINVAL,
                "%s: k=%d must exceed the window (%d) and fit index_stride=%d", who, press_k, window,
                press_index_stride);
+    // (two blocks of queries: fc_snapkv_score runs them with two wavefronts, the press tail needs at least four, and the
+    //  two arrangements sum a key's probabilities in different orders; refused so that both forms always agree bit for bit)
+    FC_REQUIRE(waves != 2, FC_EUNSUPPORTED,
+               "%s: columns of two 32-row query blocks take fc_snapkv_score and fc_select_compact", who);
     const int nw = waves <= 4 ? 4 : (waves <= 8 ? 8 : 16);
     const int room = nw == 4 ? sk_press_room<4>() : (nw == 8 ? sk_press_room<8>() : sk_press_room<16>());
     FC_REQUIRE(fast && sk_press_need(keys->max_seq_len, press_index_stride) <= room, FC_EUNSUPPORTED,
