@@ -700,10 +700,6 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
     FC_REQUIRE(press_n_kept != nullptr || (press_k > window && press_k <= press_index_stride), FC_EINVAL,
                "%s: k=%d must exceed the window (%d) and fit index_stride=%d", who, press_k, window,
                press_index_stride);
-    // (two blocks of queries: fc_snapkv_score runs them with two wavefronts, the press tail needs at least four, and the
-    //  two arrangements sum a key's probabilities in different orders; refused so that both forms always agree bit for bit)
-    FC_REQUIRE(waves != 2, FC_EUNSUPPORTED,
-               "%s: columns of two 32-row query blocks take fc_snapkv_score and fc_select_compact", who);
     const int nw = waves <= 4 ? 4 : (waves <= 8 ? 8 : 16);
     const int room = nw == 4 ? sk_press_room<4>() : (nw == 8 ? sk_press_room<8>() : sk_press_room<16>());
     FC_REQUIRE(fast && sk_press_need(keys->max_seq_len, press_index_stride) <= room, FC_EUNSUPPORTED,
@@ -740,12 +736,13 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
                        num_q_heads, window, kernel_size, causal_window, c, out_mul, scores, score_stride,    \
                        row_max, lse, 1, (float*)nullptr, (float*)nullptr, SkPress{});                        \
   } while (0)
-  // One wavefront per 32-row block of window queries, but never a single one: a lone wavefront has to fetch a whole key
-  // tile by itself between two barriers (one block of queries: 7.2 ms with one wavefront, 0.87 ms with four of which
-  // three only fetch, 2048 columns of 4096 keys).
+  // One wavefront per 32-row block of window queries, but never fewer than four: a lone wavefront has to fetch a whole
+  // key tile by itself between two barriers (one block of queries: 7.2 ms with one wavefront, 0.87 ms with four of
+  // which three only fetch, 2048 columns of 4096 keys); two blocks score 2-7 % slower with four wavefronts than with
+  // two, but four is what the press tail needs, and scoring and press must sum in the same order to agree bit for bit
+  // (whole pass, 2048 columns of 4096 keys and 8192 of 1024: 1.37 -> 1.34 ms and 1.41 -> 1.27 ms in one launch).
 #define SK_DISPATCH2(DT, FA)                 \
-  if (waves == 2) SK_LAUNCH(DT, 2, FA);      \
-  else if (waves <= 4) SK_LAUNCH(DT, 4, FA); \
+  if (waves <= 4) SK_LAUNCH(DT, 4, FA);      \
   else if (waves <= 8) SK_LAUNCH(DT, 8, FA); \
   else SK_LAUNCH(DT, 16, FA)
 #define SK_DISPATCH(DT) \
@@ -851,8 +848,7 @@ extern "C" int fc_snapkv_score_split(const fc_kv_view* keys, const void* queries
                        row_max, lse_use, nsplit, part, raw, SkPress{});                                          \
   } while (0)
 #define SK_SPLIT_NW(DT, MD)                     \
-  if (waves == 2) SK_SPLIT(DT, 2, MD);          \
-  else if (waves <= 4) SK_SPLIT(DT, 4, MD);     \
+  if (waves <= 4) SK_SPLIT(DT, 4, MD);          \
   else if (waves <= 8) SK_SPLIT(DT, 8, MD);     \
   else SK_SPLIT(DT, 16, MD)
   if (!lse) {   // pieces' statistics, then their merge into the log-sum-exp

@@ -141,14 +141,14 @@ def snapkv_score(keys: FcKvView, queries: torch.Tensor, window: int, kernel_size
 
 
 def snapkv_press_fits(keys: FcKvView, num_q_heads: int, window: int, index_stride: int) -> bool:
-    """Whether :func:`snapkv_press` takes this shape (otherwise: ``snapkv_score`` + ``select_compact``): 1 or 3 to 16
+    """Whether :func:`snapkv_press` takes this shape (otherwise: ``snapkv_score`` + ``select_compact``): at most 16
     blocks of 32 window queries per kv head, pages of 64*2^n tokens or a dense view, and
     the score row plus the kept positions inside the LDS of the key tiles."""
     if num_q_heads % keys.num_kv_heads:
         return False
     blocks = (num_q_heads // keys.num_kv_heads) * ((window + 31) // 32)
-    if blocks > 16 or blocks == 2:       # two blocks: the scoring alone runs with two wavefronts, the press would need four,
-        return False                     # and the two sum a key's probabilities in different orders (last-bit differences)
+    if blocks > 16:
+        return False
     waves = 4 if blocks <= 4 else (8 if blocks <= 8 else 16)
     tiles = 4 if waves >= 8 else 3
     room = tiles * 64 * 256 + (4 * waves + 4) * 64 * 4

@@ -142,7 +142,7 @@ int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float
  * the lower index wins; here the window wins).  `scores` receives the scored
  * positions and `row_max` (required) the per-row maxima; the caller runs fc_snapkv_fill_window afterwards if it wants
  * the window entries of `scores` filled.  Rows of sequences no longer than the window keep their first positions.
- * Takes columns of 1 or 3 to 16 blocks of 32 window queries per kv head, dense views or pages of 64*2^n tokens, and sequences short enough for the score row and the kept positions to
+ * Takes dense views or pages of 64*2^n tokens and sequences short enough for the score row and the kept positions to
  * fit the LDS of the key tiles: 4 * (max_seq_len + index_stride) + 6144 bytes within 54272 (up to four 32-row query
  * blocks per kv head) or 74752 (more), e.g. 13 000 tokens of which a quarter is kept; refused with FC_EUNSUPPORTED
  * otherwise.  A row whose kept count does not exceed the window (n_kept comes from device memory) is left untouched.  Replaces, for SnapKVPress, the per-sequence loop of
