@@ -29,10 +29,20 @@ __device__ __forceinline__ void cp_wait_then_barrier(bool stores_behind) {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Element offset of token s of sequence b (-1: its page is not allocated).  With the table row in LDS the page offset is
+// two 32 x 32 -> 64 bit multiply-adds when both strides fit 32 bits (which the workgroup tests once, on scalars), and
+// the unallocated page is a select, not a branch: this sits in front of every row load and store.
 __device__ __forceinline__ long long cp_offset(const KvView& v, const int* tbl, bool tbl_lds, int b, int s) {
   if (tbl_lds) {
     const int blk = tbl[s >> v.block_shift];
-    return blk < 0 ? -1 : (long long)blk * v.stride_block + (long long)(s & (v.block_size - 1)) * v.stride_token;
+    const unsigned page = (unsigned)max(blk, 0), slot = (unsigned)s & (unsigned)(v.block_size - 1);
+    long long off;
+    if ((((unsigned long long)v.stride_block | (unsigned long long)v.stride_token) >> 32) == 0ull)
+      off = (long long)((unsigned long long)page * (unsigned)v.stride_block +
+                        (unsigned long long)slot * (unsigned)v.stride_token);
+    else
+      off = (long long)page * v.stride_block + (long long)slot * v.stride_token;
+    return blk < 0 ? -1ll : off;
   }
   return fc_token_offset(v, b, s);
 }
