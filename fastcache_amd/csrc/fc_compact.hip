@@ -27,8 +27,8 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
   const int piece = rows_per_piece > 0 ? (int)blockIdx.x / head_groups : 0;
   const int h0 = (rows_per_piece > 0 ? (int)blockIdx.x % head_groups : (int)blockIdx.x) * HG, b = blockIdx.y;
   const int L = sk.num_layers;
-  const int l = blockIdx.z % L;
-  const bool is_v = blockIdx.z >= L;
+  const int l = (int)blockIdx.z % L;
+  const bool is_v = (int)blockIdx.z >= L;
   const KvView& src = is_v ? sv : sk;
   const KvView& dst = is_v ? dv : dk;
   const int tid = threadIdx.x, sub = tid % LPR, rg = tid / LPR;
