@@ -136,10 +136,22 @@ def fn(name: str):
     return f
 
 
+_enqueued = 0
+
+
 def check(rc: int, what: str) -> None:
+    global _enqueued
     if rc != 0:
         msg = fn("fc_last_error")().decode("utf-8", "replace")
         raise FastcacheError(f"{what} failed (code {rc}): {msg}")
+    _enqueued += 1
+
+
+def enqueue_count() -> int:
+    """Entry-point calls that have returned success so far in this process (each is at least one launch handed to
+    a stream).  Callers that rewrite a cache in place compare two readings to tell a failure before any launch
+    from one that may have left rows half rewritten."""
+    return _enqueued
 
 
 def dtype_code(dt: torch.dtype) -> int:

@@ -151,6 +151,38 @@ class BlockManager:
             tokens = seq.last_block()
             self._publish(self.blocks[table[-1]], page_key(tokens, parent), tokens)
 
+    # -- pages a compression rewrites ----------------------------------------------------------------------
+    def shared_positions(self, seq: Sequence, upto: int) -> List[int]:
+        """Positions below ``upto`` of the sequence's table whose page has more than one owner."""
+        return [i for i, b in enumerate(seq.block_table[:upto]) if self.blocks[b].ref_count > 1]
+
+    def unshare(self, seq: Sequence, positions: Seq[int]) -> List[tuple]:
+        """Give the sequence a page of its own at each of ``positions`` (pages it shares with other sequences):
+        a fresh page from the head of the free list replaces the shared one in the table, which loses one owner.
+        Returns ``(old page, new page)`` pairs; the caller copies the rows.  Nothing changes when the free list
+        is too short."""
+        positions = list(positions)
+        if len(positions) > len(self.free_block_ids):
+            raise RuntimeError(f"sequence {seq.seq_id} shares {len(positions)} pages it is about to rewrite and "
+                               f"only {len(self.free_block_ids)} pages are free")
+        moved = []
+        for i in positions:
+            old = seq.block_table[i]
+            fresh = self._claim_next()
+            seq.block_table[i] = fresh.block_id
+            self._release(old)
+            moved.append((old, fresh.block_id))
+        return moved
+
+    def forget_pages(self, block_ids: Seq[int]) -> None:
+        """The rows of these pages no longer are the tokens they were published under: drop their content keys
+        from the prefix cache, so that no later request is handed them."""
+        for block_id in block_ids:
+            page = self.blocks[block_id]
+            if page.hash != NO_KEY and self._prefix_index.get(page.hash) == block_id:
+                del self._prefix_index[page.hash]
+            page.forget()
+
     # -- release after compression ------------------------------------------------------------------------
     def free_blocks_after_compression(self, seq: Sequence, blocks_to_keep: int) -> None:
         """Give back the table's pages past the first ``blocks_to_keep`` (in table order) and cut the table."""

@@ -59,6 +59,7 @@ class DecodeOverlapCompressor:
             C = comp.paged_compressed_len(S, it_len)
             if C >= S:
                 continue
+            r._isolate_shared_pages(group, comp, image_len)    # the splice rewrites the leading pages in place
             tables, lens = r._table_and_lens([s.block_table for s in group], [S] * len(group))
             staging = torch.empty((2, r.num_hidden_layers, len(group), r.num_key_value_heads, C, r.head_dim),
                                   dtype=r.kv_cache.dtype, device=r.device)
@@ -87,8 +88,9 @@ class DecodeOverlapCompressor:
                 if l0 == 0:
                     self.compress_stream.wait_event(task["ready"])
                 with torch.cuda.stream(self.compress_stream):
+                    extra = {"seq_ids": [s.seq_id for s in task["seqs"]]} if getattr(comp, "wants_seq_ids", False) else {}
                     comp.paged_forward(r.kv_cache, task["tables"], task["lens"], task["S"], task["it_len"],
-                                       layers=(l0, l1), out=task["staging"])
+                                       layers=(l0, l1), out=task["staging"], **extra)
                     if l1 >= L:
                         task["done"] = torch.cuda.Event()
                         task["done"].record(self.compress_stream)

@@ -27,7 +27,8 @@ LayerKV = Tuple[torch.Tensor, torch.Tensor]
 
 class PagedKVRunner:
     def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int, num_blocks: int, dtype: torch.dtype,
-                 device, block_size: int = 256, compressor=None, batched_compressor=None, image_token_len: int = 576):
+                 device, block_size: int = 256, compressor=None, batched_compressor=None, image_token_len: int = 576,
+                 block_manager=None):
         self.num_hidden_layers, self.num_key_value_heads, self.head_dim = num_layers, num_kv_heads, head_dim
         self.block_size = block_size
         self.device = torch.device(device)
@@ -41,7 +42,24 @@ class PagedKVRunner:
         self._blocks_to_free: Dict[int, List[int]] = {}
         self._lock = threading.Lock()
         self._compress_stream: Optional[torch.cuda.Stream] = None
-        self._launch_started = False      # set once an enqueue may have begun to rewrite cache rows in place
+        # the page manager, when the caller has one: lets an in-place compression give a sequence its own copy of
+        # pages it shares with other sequences (prefix cache) before it rewrites them
+        self.block_manager = block_manager
+        self._touched = False
+        self._watch_enqueues = True
+        self._enqueue_mark = _lib.enqueue_count()
+
+    @property
+    def _launch_started(self) -> bool:
+        """Whether an enqueue since the flag was last cleared may have begun to rewrite cache rows in place: set by
+        hand, or read off the library's count of successful entry-point calls (host-side checks that raise before
+        the first launch leave it False)."""
+        return self._touched or (self._watch_enqueues and _lib.enqueue_count() != self._enqueue_mark)
+
+    @_launch_started.setter
+    def _launch_started(self, value: bool) -> None:
+        self._touched = bool(value)
+        self._enqueue_mark = _lib.enqueue_count()
 
     # -- tables -----------------------------------------------------------------------------------
     def preare_block_tables(self, seqs: Seq[Sequence]) -> torch.Tensor:
@@ -93,6 +111,69 @@ class PagedKVRunner:
                 src = torch.stack(layers)                             # [L, 1, Hkv, C, D]: tensors of mixed geometry
                 ops.copy_tokens(_lib.dense_view(src), dst, 0, C, 0)
 
+    # -- pages shared between sequences ----------------------------------------------------------------
+    def _pages_rewritten(self, comp, seq_len: int, it_len) -> int:
+        """How many leading pages an in-place compression of ``seq_len`` rows writes (all of them when the
+        compressor cannot say its output length beforehand)."""
+        rows = seq_len
+        if hasattr(comp, "paged_compressed_len"):
+            try:
+                rows = min(seq_len, int(comp.paged_compressed_len(seq_len, it_len)))
+            except Exception:
+                rows = seq_len
+        return -(-rows // self.block_size)
+
+    def _isolate_shared_pages(self, seqs: Seq[Sequence], comp, image_len: int) -> int:
+        """Full prompt pages of identical content are shared between sequences (prefix cache).  An in-place
+        compression rewrites the leading pages of every sequence of the batch in one launch, so a page that has
+        another owner, in the batch or not, must first become the sequence's own: with a page manager attached
+        the sequence gets a fresh page and the rows are copied (one ``fc_copy_tokens`` launch per plane for all
+        such pages); without one, a batch whose tables name a page twice where it would be rewritten is refused.
+        Runs before any row is rewritten; returns the number of pages copied."""
+        bm = self.block_manager
+        writes = [self._pages_rewritten(comp, len(s), [image_len, max(1, len(s) - image_len)]) for s in seqs]
+        if bm is None:
+            owners: Dict[int, int] = {}
+            for s in seqs:
+                for b in set(s.block_table):
+                    owners[b] = owners.get(b, 0) + 1
+            for s, w in zip(seqs, writes):
+                for b in s.block_table[:w]:
+                    if b >= 0 and owners[b] > 1:
+                        raise _lib.FastcacheError(
+                            f"page {b} belongs to several sequences of the batch and sequence {s.seq_id} would "
+                            "rewrite it in place; attach the page manager (block_manager=) so that it gets its own copy")
+            return 0
+        # a page shared only inside the batch stays with the last sequence that names it
+        owners = {b: bm.blocks[b].ref_count for s in seqs for b in s.block_table if b >= 0}
+        plan = []
+        for s, w in zip(seqs, writes):
+            mine = []
+            for i, b in enumerate(s.block_table[:w]):
+                if owners[b] > 1:
+                    owners[b] -= 1
+                    mine.append(i)
+            plan.append((s, mine))
+        need = sum(len(p) for _, p in plan)
+        if need == 0:
+            return 0
+        if need > len(bm.free_block_ids):
+            raise _lib.FastcacheError(f"the batch would rewrite {need} pages it shares with other sequences and only "
+                                      f"{len(bm.free_block_ids)} pages are free to copy them to")
+        moved = []
+        for s, positions in plan:
+            moved += bm.unshare(s, positions)
+        if moved:
+            old = [[a] for a, _ in moved]
+            new = [[b] for _, b in moved]
+            n = self.block_size
+            t_old, ll = self._table_and_lens(old, [n] * len(moved))
+            t_new, _ = self._table_and_lens(new, [n] * len(moved))
+            for p in range(2):
+                ops.copy_tokens(_lib.paged_view(self.kv_cache[p], t_old, ll, n),
+                                _lib.paged_view(self.kv_cache[p], t_new, ll, n), 0, n, 0)
+        return len(moved)
+
     # -- compression ---------------------------------------------------------------------------------
     def _active_compressor(self):
         if self.use_batched_compressor and self.batched_compressor is not None:
@@ -111,16 +192,23 @@ class PagedKVRunner:
             # sequence's length (and, for the MLPs, its segments) from device arrays
             lens = [len(s) for s in seqs]
             S = max(lens)
+            self._isolate_shared_pages(seqs, comp, image_len)           # may edit the tables
             tt, ll = self._table_and_lens([s.block_table for s in seqs], lens)
             it_len = [image_len, max(1, S - image_len)]
-            self._launch_started = True       # from here on a failure may leave rows partly rewritten
-            C = comp.paged_forward(self.kv_cache, tt, ll, S, it_len, host_lens=lens)
+            # from here on every successful enqueue counts: a failure after one may leave rows partly rewritten, a
+            # failure in the host-side checks before it leaves the cache as it was
+            self._watch_enqueues = True
+            self._launch_started = False
+            extra = {"seq_ids": [s.seq_id for s in seqs]} if getattr(comp, "wants_seq_ids", False) else {}
+            C = comp.paged_forward(self.kv_cache, tt, ll, S, it_len, host_lens=lens, **extra)
             per_seq = list(C) if isinstance(C, (list, tuple)) else [C] * len(seqs)
             for s, n, c in zip(seqs, lens, per_seq):
                 result[s.seq_id] = c
                 orig += 2 * L * H * D * n
                 after += 2 * L * H * D * c
         else:
+            self._watch_enqueues = False      # the extracts launch copies that leave the pages alone
+            self._isolate_shared_pages(seqs, comp, image_len)
             for s in seqs:
                 S = len(s)
                 hf = self._extract_kv_cache_fast(s.block_table, S)

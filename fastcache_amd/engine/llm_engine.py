@@ -6,9 +6,10 @@ in front of the first decode of those sequences), release the freed blocks, post
 forward is not part of this build: ``model_step(seqs, is_prefill) -> token ids`` is supplied by the caller
 (a real model writing its KV through the runner's pool, or a synthetic stand-in).
 
-``LazyCompressionEngine`` follows nanovllm_fastapi_server.py:54-153: no compression after prefill; when the
-free blocks fall under a fraction of the pool, every running sequence not yet compressed is compressed
-in one batch and its tail blocks are released.
+``LazyCompressionEngine`` plays the part of nanovllm_fastapi_server.py:54-153: no compression after prefill;
+when the free blocks fall under a fraction of the pool, every running sequence not yet compressed is
+compressed in one batch and its tail blocks are released.  It keeps no set of its own: the scheduler's
+running queue and ``Sequence.is_compressed`` are the state.
 """
 from __future__ import annotations
 
@@ -35,6 +36,8 @@ class CompressionEngine:
                  async_compression: bool = False, decode_overlap=None):
         self.scheduler = scheduler
         self.model_runner = model_runner
+        if getattr(model_runner, "block_manager", False) is None:      # lets the runner un-share pages it rewrites
+            model_runner.block_manager = scheduler.block_manager
         self.model_step = model_step
         self.enable_compression = enable_compression
         self.async_compression = async_compression
@@ -96,17 +99,45 @@ class CompressionEngine:
 
 
 class LazyCompressionEngine:
+    """Memory-pressure policy on top of a ``CompressionEngine`` (the role of nanovllm_fastapi_server.py:54-153):
+    prefills leave the caches whole; before a step, if fewer than ``compression_threshold`` of the pool's pages are
+    free, every running sequence that still holds its full cache is compressed in ONE batched pass and its tail
+    pages go back to the pool, where the same step's scheduler can hand them to waiting requests.
+
+    Nothing is remembered between steps: the candidates are read off the scheduler's running queue (a sequence is
+    there only after its prefill ran, and ``Sequence.is_compressed`` says whether it was shortened), so a pre-empted
+    or finished sequence needs no bookkeeping here.  A sequence that has decoded since its prefill holds
+    ``len(seq) - 1`` KV rows (the last token's row is written by the next step); like the reference this pass hands
+    ``len(seq)`` rows to the compressor there."""
+
     def __init__(self, llm: CompressionEngine, compression_threshold: float = 0.3,
                  compression_backend: str = "kvpress"):
         self.llm = llm
         self.compression_threshold = compression_threshold
         self.compression_backend = compression_backend
-        self.total_blocks = len(llm.scheduler.block_manager.blocks)
-        self.threshold_blocks = int(self.total_blocks * compression_threshold)
-        self.uncompressed_seqs = set()
-        self.compression_count = 0
-        self.total_compression_time = 0.0
+        self._pass_seconds: List[float] = []          # wall time of every batched pass so far
 
+    # -- the pool, as the policy sees it ---------------------------------------------------------------
+    @property
+    def total_blocks(self) -> int:
+        return len(self.llm.scheduler.block_manager.blocks)
+
+    @property
+    def threshold_blocks(self) -> int:
+        return int(self.total_blocks * self.compression_threshold)
+
+    def candidates(self) -> List[Sequence]:
+        return [s for s in self.llm.scheduler.running if not s.is_compressed]
+
+    @property
+    def uncompressed_seqs(self) -> set:
+        """Ids of the running sequences with a full cache (the reference keeps this as a mutable set)."""
+        return {s.seq_id for s in self.candidates()}
+
+    def under_pressure(self) -> bool:
+        return len(self.llm.scheduler.block_manager.free_block_ids) < self.threshold_blocks
+
+    # -- engine surface -----------------------------------------------------------------------------------
     def add_request(self, prompt, sampling_params=None):
         return self.llm.add_request(prompt, sampling_params)
 
@@ -114,35 +145,33 @@ class LazyCompressionEngine:
         return self.llm.is_finished()
 
     def step(self):
-        free_blocks = len(self.llm.scheduler.block_manager.free_block_ids)
-        if free_blocks < self.threshold_blocks and self.uncompressed_seqs:
-            self._do_batch_compression()
-        outputs, num_tokens = self.llm.step(apply_compression=False)
-        if num_tokens > 0:
-            for seq in self.llm.scheduler.running:
-                if not seq.is_compressed:
-                    self.uncompressed_seqs.add(seq.seq_id)
-        for seq_id, _ in outputs:
-            self.uncompressed_seqs.discard(seq_id)
-        return outputs, num_tokens
+        if self.under_pressure():
+            self.compress_running()
+        return self.llm.step(apply_compression=False)
 
-    def _do_batch_compression(self) -> None:
-        """One batched launch for every running sequence that still has its full cache.  A sequence that has
-        decoded since its prefill holds ``len(seq) - 1`` KV rows (the last token's row is written by the next
-        step); the reference compresses ``len(seq)`` rows there, one of them never written."""
-        seqs = [s for s in self.llm.scheduler.running if s.seq_id in self.uncompressed_seqs and not s.is_compressed]
-        if not seqs:
-            self.uncompressed_seqs.clear()
-            return
-        start = time.time()
-        self.llm.model_runner.compress_kv_cache_batch(seqs)
-        for seq in seqs:
-            self.llm._free_compressed_blocks([seq])
-            self.uncompressed_seqs.discard(seq.seq_id)
-        self.compression_count += 1
-        self.total_compression_time += time.time() - start
+    def compress_running(self) -> int:
+        """Compress every candidate now; returns how many sequences were shortened."""
+        todo = self.candidates()
+        if not todo:
+            return 0
+        t0 = time.perf_counter()
+        self.llm.model_runner.compress_kv_cache_batch(todo)
+        self.llm._free_compressed_blocks(todo)
+        self._pass_seconds.append(time.perf_counter() - t0)
+        return len(todo)
+
+    _do_batch_compression = compress_running          # the reference's name for the pass
+
+    # -- statistics ---------------------------------------------------------------------------------------
+    @property
+    def compression_count(self) -> int:
+        return len(self._pass_seconds)
+
+    @property
+    def total_compression_time(self) -> float:
+        return sum(self._pass_seconds)
 
     def get_stats(self) -> dict:
-        n = self.compression_count
-        return {"compression_count": n, "total_compression_time_ms": self.total_compression_time * 1000,
-                "avg_compression_time_ms": self.total_compression_time / n * 1000 if n > 0 else 0}
+        n, total_ms = self.compression_count, self.total_compression_time * 1000
+        return {"compression_count": n, "total_compression_time_ms": total_ms,
+                "avg_compression_time_ms": total_ms / n if n else 0}

@@ -21,23 +21,27 @@ def free_compressed_blocks(block_manager: BlockManager, model_runner: PagedKVRun
     """
     freed = 0
     for seq in seqs:
-        c = model_runner._compressed_lens.get(seq.seq_id)
-        if c is None:
+        rows = model_runner._compressed_lens.get(seq.seq_id)
+        if rows is None:
             continue
-        seq.kv_cache_len = c
+        seq.kv_cache_len = rows
         keep = model_runner.get_compressed_block_count(seq.seq_id)
-        if keep > 0 and len(seq.block_table) > keep:
-            for block_id in seq.block_table[keep:]:
-                if block_id in block_manager.used_block_ids:
-                    blk = block_manager.blocks[block_id]
-                    blk.ref_count -= 1
-                    if blk.ref_count == 0:
-                        block_manager._deallocate_block(block_id)
-                        freed += 1
+        model_runner._blocks_to_free.pop(seq.seq_id, None)
+        if keep <= 0:
+            continue
+        tail = seq.block_table[keep:]
+        if tail:
+            free_before = len(block_manager.free_block_ids)
+            block_manager.free_specific_blocks(tail)      # one owner fewer each; unowned pages join the free list in table order
+            freed += len(block_manager.free_block_ids) - free_before
             seq.block_table = seq.block_table[:keep]
-            kept = seq.block_table if reset_all_kept_hashes else seq.block_table[-1:]
-            for block_id in kept:
+        # pages whose rows the compression rewrote must not serve a later request as its prompt prefix: all kept
+        # pages (also when no page was freed), or like the reference only the last one of a table that got shorter
+        stale = seq.block_table if reset_all_kept_hashes else (seq.block_table[-1:] if tail else [])
+        if hasattr(block_manager, "forget_pages"):
+            block_manager.forget_pages(stale)             # the content keys leave the prefix index as well
+        else:                                             # a manager that only has the reference's fields
+            for block_id in stale:
                 block_manager.blocks[block_id].hash = -1
                 block_manager.blocks[block_id].token_ids = []
-        model_runner._blocks_to_free.pop(seq.seq_id, None)
     return freed

@@ -25,6 +25,7 @@ import torch
 from torch import nn
 
 from . import _lib, ops
+from ._lib import FastcacheError
 
 
 def _cache_layer_kv(cache, layer_idx):
@@ -86,6 +87,66 @@ class ScorerPress:
         ops.compact(_lib.dense_view(keys), _lib.dense_view(values), _lib.dense_view(out_k), _lib.dense_view(out_v), idx)
         return out_k, out_v
 
+    # -- nano-vllm runner hook: the press of a paged pool (llava_model_runner.py:745-786) --------------------------
+    # ``PagedKVRunner(compressor=press).compress_kv_cache_batch(seqs)`` calls ``paged_forward`` once for the whole
+    # batch, in place of the reference's per-sequence extract -> compressor -> write-back loop.
+    wants_seq_ids = True          # the runner passes ``seq_ids=``: presses that hold per-sequence inputs look them up
+
+    def paged_compressed_len(self, seq_len: int, it_len=None) -> int:
+        n = self.n_kept(seq_len)
+        return seq_len if self.compression_ratio == 0 or n >= seq_len else n
+
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        """fp32 ``[L, B, Hkv, max_seq_len]`` for the layers ``layers=(l0, l1)`` of the views; entries past a
+        sequence's length are never read by the selection."""
+        raise FastcacheError(f"{type(self).__name__} cannot score a paged pool")
+
+    @torch.no_grad()
+    def paged_forward(self, kv_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                      seq_len: int, it_len=None, layers=None, out: Optional[torch.Tensor] = None, host_lens=None,
+                      seq_ids=None):
+        """Score, select and compact every (layer, sequence, kv head) column of the pool
+        ``kv_cache [2, L, blocks, block_size, Hkv, D]``: in place (the kept rows move to the front of the same
+        pages, ascending positions), or for ``layers=(l0, l1)`` only, or into ``out [2, L, B, Hkv, C, D]`` with the
+        pages left alone.  Sequences all hold ``seq_len`` rows, or ``host_lens`` rows each (Python ints, ``seq_len``
+        their maximum; ``seq_lens`` the same numbers on the device).  Returns the kept length, or the list of kept
+        lengths when the sequences differ.  ``it_len`` (the MLP compressors' image/text split) is not used."""
+        B = block_tables.shape[0]
+        lens = list(host_lens) if host_lens is not None else [seq_len] * B
+        kept = [self.paged_compressed_len(n) for n in lens]
+        l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
+        result = kept if len(set(lens)) > 1 else kept[0]
+        if all(k >= n for k, n in zip(kept, lens)):
+            if out is not None:
+                for p in range(2):
+                    ops.copy_tokens(_lib.paged_view(kv_cache[p][l0:l1], block_tables, seq_lens, seq_len),
+                                    _lib.dense_view(out[p][l0:l1]), 0, seq_len, 0)
+            return result
+        self._paged_press(kv_cache[:, l0:l1], block_tables, seq_lens, seq_len, lens, kept, (l0, l1), out, seq_ids)
+        return result
+
+    def _paged_press(self, pool, block_tables, seq_lens, seq_len, lens, kept, layers, out, seq_ids):
+        """Scores from ``paged_scores``, then one selection + compaction launch (two when a column does not fit LDS)."""
+        from . import paged_press
+        kview, vview = paged_press._views(pool, block_tables, seq_lens, seq_len)
+        scores = self.paged_scores(kview, vview, lens, seq_lens, layers, seq_ids, pool.device)
+        if out is None:
+            paged_press._select_and_compact(kview, vview, scores, seq_lens, kept, True, pool.shape[4])
+            return
+        self._compact_into(kview, vview, scores, seq_lens, kept, pool.shape[4], out, layers)
+
+    @staticmethod
+    def _compact_into(kview, vview, scores, seq_lens, kept, heads, out, layers):
+        l0, l1 = layers
+        width = max(kept)
+        dk, dv = _lib.dense_view(out[0][l0:l1]), _lib.dense_view(out[1][l0:l1])
+        if len(set(kept)) == 1 and seq_lens is None:
+            ops.compact(kview, vview, dk, dv, ops.topk_select(scores, width))
+            return
+        n_kept = torch.tensor(kept, dtype=torch.int32, device=scores.device)
+        idx = ops.topk_select(scores, width, row_lens=seq_lens, n_kept=n_kept, rows_per_len=heads)
+        ops.compact(kview, vview, dk, dv, idx, n_kept=n_kept)
+
     # -- HuggingFace hook protocol (utils_compress.py:209-299) ---------------------------------------
     def forward_hook(self, module: nn.Module, input, kwargs: dict, output):
         cache = kwargs.get("past_key_value", kwargs.get("past_key_values"))
@@ -116,12 +177,61 @@ class ScorerPress:
                 h.remove()
 
 
+class _PerSequenceInputs:
+    """What a prefill hands to a press for the later compression of its sequences on the runner hook: tensors
+    ``[L, B, ...]`` (window queries, their log-sum-exp, query statistics), kept whole for the batch they came with
+    and, when ``seq_ids`` are given, findable per sequence so that a later batch of other composition (lazy
+    compression) can be assembled.  An entry is dropped once it has been used."""
+
+    def __init__(self):
+        self._batch = None            # (ids or None, {name: tensor [L, B, ...]})
+        self._by_seq = {}             # seq_id -> {name: tensor [L, ...]}
+
+    def put(self, tensors: dict, seq_ids=None) -> None:
+        tensors = {k: v for k, v in tensors.items() if v is not None}
+        self._batch = (None if seq_ids is None else list(seq_ids), tensors)
+        if seq_ids is not None:
+            for b, i in enumerate(seq_ids):
+                self._by_seq[i] = {k: v[:, b] for k, v in tensors.items()}
+
+    def take(self, batch: int, seq_ids=None) -> dict:
+        ids, tensors = self._batch if self._batch is not None else (None, None)
+        if tensors is not None and (ids is None or seq_ids is None or ids == list(seq_ids)):
+            if next(iter(tensors.values())).shape[1] != batch:
+                raise FastcacheError(f"the press holds inputs for {next(iter(tensors.values())).shape[1]} sequences, "
+                                     f"the batch has {batch}")
+            self._batch = None
+            for i in ids or ():
+                self._by_seq.pop(i, None)
+            return tensors
+        missing = [i for i in seq_ids if i not in self._by_seq]
+        if missing:
+            raise FastcacheError(f"the press holds no inputs for sequences {missing}")
+        rows = [self._by_seq.pop(i) for i in seq_ids]
+        self._batch = None
+        return {k: torch.stack([r[k] for r in rows], dim=1) for k in rows[0]}
+
+    def __bool__(self):
+        return self._batch is not None or bool(self._by_seq)
+
+
 @dataclass
 class KnormPress(ScorerPress):
     """``score = -||k||_2``: keys with a small norm are kept."""
 
     def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
         return ops.knorm_score(_lib.dense_view(keys), keys.device)[0]
+
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        return ops.knorm_score(kview, device)
+
+    def _paged_press(self, pool, block_tables, seq_lens, seq_len, lens, kept, layers, out, seq_ids):
+        if out is not None:
+            return super()._paged_press(pool, block_tables, seq_lens, seq_len, lens, kept, layers, out, seq_ids)
+        from . import paged_press
+        # scoring, selection and compaction of a column by one workgroup, one launch for the batch
+        paged_press.knorm_compress_paged(pool, block_tables, seq_lens, seq_len, self.compression_ratio,
+                                         host_lens=lens if len(set(lens)) > 1 else None)
 
 
 @dataclass
@@ -141,9 +251,54 @@ class SnapKVPress(ScorerPress):
     reduction: str = "mean"
     window_in_budget: bool = True
 
+    def __post_init__(self):
+        super().__post_init__()
+        self._paged_inputs = _PerSequenceInputs()
+
     def n_kept(self, q_len: int) -> int:
         n = int(q_len * (1 - self.compression_ratio))
         return n if self.window_in_budget else min(q_len, n + self.window_size)
+
+    # -- runner hook ------------------------------------------------------------------------------------------
+    def set_window_queries(self, queries: torch.Tensor, seq_ids=None, lse: Optional[torch.Tensor] = None) -> None:
+        """What a prefill hands over for the compression of its sequences on the runner hook: the rotated queries of
+        the last ``window_size`` positions of every sequence, ``[L, B, Hq, W, D]`` in the cache dtype (sequence order
+        = the order of the batch that will be compressed, or named by ``seq_ids`` so that any later batch can be
+        assembled), optionally with their log-sum-exp over the keys ``[L, B, Hq, W]`` from the attention kernel."""
+        if queries.dim() != 5 or queries.shape[3] != self.window_size:
+            raise FastcacheError(f"window queries must be [L, B, Hq, W={self.window_size}, D], got {tuple(queries.shape)}")
+        self._paged_inputs.put({"queries": queries, "lse": lse}, seq_ids)
+
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        q, lse = self._paged_window(len(lens), layers, seq_ids)
+        return ops.snapkv_score(kview, q, self.window_size, self.kernel_size, self.causal_window, self.reduction,
+                                seq_lens=seq_lens, lse=lse)
+
+    def _paged_window(self, batch, layers, seq_ids, keep: bool = False):
+        if not self._paged_inputs:
+            raise FastcacheError("SnapKVPress on the runner hook needs the window queries of the batch: call "
+                                 "set_window_queries(q[L, B, Hq, W, D]) after the prefill")
+        held = self._paged_inputs
+        got = held.take(batch, seq_ids)
+        l0, l1 = layers
+        if keep or l1 < got["queries"].shape[0]:          # layer chunks (decode overlap) come back for the rest
+            held.put(got, seq_ids)
+        return got["queries"][l0:l1], (got["lse"][l0:l1] if "lse" in got else None)
+
+    def _paged_press(self, pool, block_tables, seq_lens, seq_len, lens, kept, layers, out, seq_ids):
+        if out is not None:
+            return super()._paged_press(pool, block_tables, seq_lens, seq_len, lens, kept, layers, out, seq_ids)
+        from . import paged_press
+        q, lse = self._paged_window(len(lens), layers, seq_ids)
+        if lse is not None:          # one sweep over the keys, then selection + compaction
+            kview, vview = paged_press._views(pool, block_tables, seq_lens, seq_len)
+            scores = ops.snapkv_score(kview, q, self.window_size, self.kernel_size, self.causal_window,
+                                      self.reduction, seq_lens=seq_lens, lse=lse)
+            paged_press._select_and_compact(kview, vview, scores, seq_lens, kept, True, pool.shape[4])
+            return
+        paged_press.snapkv_compress_paged(pool, block_tables, seq_lens, seq_len, q, self.compression_ratio,
+                                          self.window_size, self.kernel_size, self.causal_window, self.reduction,
+                                          self.window_in_budget, host_lens=lens if len(set(lens)) > 1 else None)
 
     def window_queries(self, module, hidden_states, kwargs) -> torch.Tensor:
         """Rotated queries of the last ``window_size`` positions, ``[B, Hq, W, D]``: given directly as
@@ -197,6 +352,29 @@ class TOVAPress(ScorerPress):
         scores[..., S - 1] = mean.max()
         return scores
 
+    def __post_init__(self):
+        super().__post_init__()
+        self._paged_inputs = _PerSequenceInputs()
+
+    def set_window_queries(self, queries: torch.Tensor, seq_ids=None) -> None:
+        """Runner hook: the rotated query of every sequence's last position, ``[L, B, Hq, 1, D]`` (or a longer
+        window, of which the last position is used)."""
+        if queries.dim() != 5:
+            raise FastcacheError(f"queries must be [L, B, Hq, W, D], got {tuple(queries.shape)}")
+        self._paged_inputs.put({"queries": queries[:, :, :, -1:, :]}, seq_ids)
+
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        if not self._paged_inputs:
+            raise FastcacheError("TOVAPress on the runner hook needs the last queries: call set_window_queries first")
+        q = self._paged_inputs.take(len(lens), seq_ids)["queries"][layers[0]:layers[1]].contiguous()
+        sums = ops.snapkv_score(kview, q, 1, 1, True, "sum", 1.0 / math.sqrt(kview.head_dim), seq_lens=seq_lens)
+        scores = torch.full_like(sums, float("-inf"))
+        for b, n in enumerate(lens):                       # per sequence: head mean over its n - 1 other keys
+            mean = sums[:, b, :, :n - 1].sum(1, keepdim=True) / q.shape[2]
+            scores[:, b, :, :n - 1] = mean
+            scores[:, b, :, n - 1] = mean.amax(dim=(1, 2), keepdim=False)[:, None] if n > 1 else 0.0
+        return scores
+
 
 @dataclass
 class ObservedAttentionPress(ScorerPress):
@@ -208,6 +386,10 @@ class ObservedAttentionPress(ScorerPress):
     def score(self, module, hidden_states, keys, values, attentions, kwargs) -> torch.Tensor:
         assert attentions is not None, 'Set output_attentions=True and attn_implementation="eager" to use this hook'
         return ops.observed_attention_score(attentions, keys.shape[1])
+
+    def paged_forward(self, *args, **kwargs):
+        raise FastcacheError("ObservedAttentionPress needs the prefill's attention matrices, which a paged runner "
+                             "never materialises; use it through the HuggingFace hook")
 
 
 @dataclass
@@ -276,6 +458,27 @@ class ExpectedAttentionPress(ScorerPress):
         return ops.expected_attention_score(_lib.dense_view(keys), _lib.dense_view(values), mu, cov, self.n_sink,
                                             self.use_vnorm, self.epsilon)[0]
 
+    def __post_init__(self):
+        super().__post_init__()
+        self._paged_inputs = _PerSequenceInputs()
+
+    def set_query_statistics(self, mean_query: torch.Tensor, cov_query: Optional[torch.Tensor] = None,
+                             seq_ids=None) -> None:
+        """Runner hook: ``mean_query [L, B, Hq, D]`` and ``cov_query [L, B, Hq, D, D]`` of the future queries
+        (``get_query_statistics`` per layer of the prefill)."""
+        self._paged_inputs.put({"mean": mean_query, "cov": cov_query if self.use_covariance else None}, seq_ids)
+
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        if len(set(lens)) > 1:
+            raise FastcacheError("ExpectedAttentionPress on the runner hook takes sequences of one length per call")
+        if not self._paged_inputs:
+            raise FastcacheError("ExpectedAttentionPress on the runner hook needs set_query_statistics first")
+        got = self._paged_inputs.take(len(lens), seq_ids)
+        l0, l1 = layers
+        cov = got["cov"][l0:l1] if "cov" in got else None
+        return ops.expected_attention_score(kview, vview, got["mean"][l0:l1], cov, self.n_sink, self.use_vnorm,
+                                            self.epsilon)
+
 
 @dataclass
 class StreamingLLMPress(ScorerPress):
@@ -291,6 +494,15 @@ class StreamingLLMPress(ScorerPress):
         scores[:, :, self.n_sink:self.n_sink + n_pruned] = 0
         return scores
 
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        rows = torch.full((len(lens), kview.max_seq_len), float("-inf"))
+        for b, n in enumerate(lens):
+            assert n > self.n_sink, f"Input should contain more tokens than n_sink={self.n_sink}"
+            rows[b, :n] = 1.0
+            rows[b, self.n_sink:self.n_sink + n - self.paged_compressed_len(n)] = 0.0
+        L, H = layers[1] - layers[0], kview.num_kv_heads
+        return rows.to(device)[None, :, None, :].expand(L, len(lens), H, -1).contiguous()
+
 
 @dataclass
 class RandomPress(ScorerPress):
@@ -303,6 +515,16 @@ class RandomPress(ScorerPress):
         if self.seed is not None:
             g = torch.Generator(device=keys.device).manual_seed(self.seed)
         return torch.rand(keys.shape[:3], dtype=torch.float32, device=keys.device, generator=g)
+
+    def paged_scores(self, kview, vview, lens, seq_lens, layers, seq_ids, device) -> torch.Tensor:
+        g = None
+        if self.seed is not None:
+            g = torch.Generator(device=device).manual_seed(self.seed)
+        shape = (layers[1] - layers[0], len(lens), kview.num_kv_heads, kview.max_seq_len)
+        scores = torch.rand(shape, dtype=torch.float32, device=device, generator=g)
+        for b, n in enumerate(lens):
+            scores[:, b, :, n:] = float("-inf")
+        return scores
 
 
 @dataclass
@@ -340,6 +562,39 @@ class ThinKPress(ScorerPress):
         prune = torch.zeros((B, Hkv, D), dtype=torch.uint8, device=keys.device).scatter_(-1, idx, 1)
         ops.key_channel_zero(_lib.dense_view(keys), prune[None])
         return keys, values
+
+    def set_window_queries(self, queries: torch.Tensor, seq_ids=None) -> None:
+        """Runner hook: rotated queries of the last ``window_size`` positions, ``[L, B, Hq, W, D]``."""
+        if not hasattr(self, "_paged_inputs"):
+            self._paged_inputs = _PerSequenceInputs()
+        self._paged_inputs.put({"queries": queries}, seq_ids)
+
+    @torch.no_grad()
+    def paged_forward(self, kv_cache, block_tables, seq_lens, seq_len, it_len=None, layers=None, out=None,
+                      host_lens=None, seq_ids=None):
+        """Zero the pruned key channels of every (layer, sequence, kv head) column in the pages; lengths stay."""
+        B = block_tables.shape[0]
+        lens = list(host_lens) if host_lens is not None else [seq_len] * B
+        result = lens if len(set(lens)) > 1 else lens[0]
+        if out is not None:
+            raise FastcacheError("ThinKPress prunes channels in place; it has no staged output")
+        D = kv_cache.shape[-1]
+        n_pruned = int(D * self.key_channel_compression_ratio)
+        if n_pruned == 0:
+            return result
+        if not getattr(self, "_paged_inputs", None):
+            raise FastcacheError("ThinKPress on the runner hook needs set_window_queries first")
+        l0, l1 = layers if layers is not None else (0, kv_cache.shape[1])
+        q = self._paged_inputs.take(B, seq_ids)["queries"][l0:l1]                       # [L, B, Hq, W, D]
+        kview = _lib.paged_view(kv_cache[0][l0:l1], block_tables, seq_lens, seq_len)
+        Hkv = kview.num_kv_heads
+        q_energy = q.float().pow(2).mean(dim=3).view(l1 - l0, B, Hkv, q.shape[2] // Hkv, D).mean(dim=3)
+        rows = torch.tensor(lens, dtype=torch.float32, device=kv_cache.device).view(1, B, 1, 1)
+        scores = q_energy * (ops.key_channel_energy(kview, kv_cache.device) / rows)
+        idx = ops.topk_select((-scores).contiguous(), n_pruned).long()
+        prune = torch.zeros((l1 - l0, B, Hkv, D), dtype=torch.uint8, device=kv_cache.device).scatter_(-1, idx, 1)
+        ops.key_channel_zero(kview, prune)
+        return result
 
 
 @dataclass
@@ -397,6 +652,10 @@ class SimLayerKVPress(ScorerPress):
         ops.compact(_lib.dense_view(keys), _lib.dense_view(values), _lib.dense_view(out_k), _lib.dense_view(out_v), idx)
         self.compression_ratios.append((q_len - self.n_initial - self.n_recent + 1) / q_len)
         return out_k, out_v
+
+    def paged_forward(self, *args, **kwargs):
+        raise FastcacheError("SimLayerKVPress keeps a different number of tokens per layer, which one block table "
+                             "per sequence cannot hold; use it through the HuggingFace hook")
 
 
 class SimpleKVQuantizer:

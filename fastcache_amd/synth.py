@@ -62,15 +62,29 @@ def make_tables(seq_lens: List[int], num_blocks: int, g: torch.Generator, shuffl
     return tables
 
 
-def scatter_into_pool(kv_cache: torch.Tensor, plane: int, layer: int, dense: torch.Tensor,
-                      tables: List[List[int]], seq_lens: List[int]) -> None:
-    """dense ``[B, Hkv, S, D]`` -> pool pages of ``kv_cache[plane, layer]``."""
-    bs = kv_cache.shape[3]
+def pool_slot_index(tables: List[List[int]], seq_lens: List[int], block_size: int, dense_len: int, device=None):
+    """For every token of every sequence, in sequence order: its row in the flattened pool
+    (``table[s // block_size] * block_size + s % block_size``) and its row in a dense ``[B, S]`` token grid
+    (``b * dense_len + s``), as two int64 tensors."""
+    slots, rows = [], []
     for b, (tab, n) in enumerate(zip(tables, seq_lens)):
-        seq = dense[b, :, :n].permute(1, 0, 2)                   # [n, Hkv, D]
-        for i in range((n + bs - 1) // bs):
-            m = min(bs, n - i * bs)
-            kv_cache[plane, layer, tab[i], :m] = seq[i * bs:i * bs + m]
+        pos = torch.arange(n, dtype=torch.int64)
+        slots.append(torch.tensor(tab, dtype=torch.int64)[pos // block_size] * block_size + pos % block_size)
+        rows.append(pos + b * dense_len)
+    slots, rows = torch.cat(slots), torch.cat(rows)
+    return (slots.to(device), rows.to(device)) if device is not None else (slots, rows)
+
+
+def scatter_into_pool(kv_cache: torch.Tensor, plane: int, layer: int, dense: torch.Tensor,
+                      tables: List[List[int]], seq_lens: List[int], index=None) -> None:
+    """dense ``[B, Hkv, S, D]`` -> pool pages of ``kv_cache[plane, layer]``: one indexed store for the whole
+    batch (``index`` = a ``pool_slot_index`` result, to reuse it across layers and planes)."""
+    bs = kv_cache.shape[3]
+    B, H, S, D = dense.shape
+    slots, rows = index if index is not None else pool_slot_index(tables, seq_lens, bs, S, kv_cache.device)
+    flat = kv_cache[plane, layer].view(-1, H, D)                                  # [num_blocks * block_size, Hkv, D]
+    tokens = dense.permute(0, 2, 1, 3).reshape(B * S, H, D)                       # [B * S, Hkv, D]
+    flat.index_copy_(0, slots, tokens.index_select(0, rows.to(tokens.device)).to(flat.device))
 
 
 def make_paged_case(*, seed: int, num_layers: int, batch: int, num_kv_heads: int, seq_lens: List[int],
@@ -100,6 +114,7 @@ def make_paged_case(*, seed: int, num_layers: int, batch: int, num_kv_heads: int
     if keep_dense:
         dk = torch.empty((num_layers, batch, num_kv_heads, S, head_dim), dtype=dtype, device=dev)
         dv = torch.empty_like(dk)
+    index = pool_slot_index(tables, seq_lens, block_size, S, dev)
     for layer in range(num_layers):
         planes = []
         for _ in range(2):                                        # K then V
@@ -112,7 +127,7 @@ def make_paged_case(*, seed: int, num_layers: int, batch: int, num_kv_heads: int
                 x[:, :, :image_tokens] *= image_scale
             planes.append(x.to(dtype).to(dev))
         for p, x in enumerate(planes):
-            scatter_into_pool(kv_cache, p, layer, x, tables, seq_lens)
+            scatter_into_pool(kv_cache, p, layer, x, tables, seq_lens, index)
         if keep_dense:
             dk[layer], dv[layer] = planes
     q = None

@@ -52,15 +52,29 @@ def knorm_press_compressor(compression_ratio: float) -> Compressor:
 
 
 def snapkv_press_compressor(queries: torch.Tensor, compression_ratio: float, window_size: int,
-                            kernel_size: int, causal_window: bool = True, reduction: str = "mean"
-                            ) -> Compressor:
-    """Per-layer ``SnapKVPress.compress``; queries ``[L, B, Hq, W, D]`` indexed by layer and sequence."""
+                            kernel_size: int, causal_window: bool = True, reduction: str = "mean",
+                            window_in_budget: bool = True) -> Compressor:
+    """Per-layer ``SnapKVPress.compress``; queries ``[L, B, Hq, W, D]`` indexed by layer and sequence.  With
+    ``window_in_budget=False`` the window is kept on top of ``int(S * (1 - r))``."""
     def run(hf, i, n):
         out = []
         for layer, (k, v) in enumerate(hf):
             sc = presses.snapkv_score(queries[layer, i:i + 1], k, window_size, kernel_size, causal_window,
                                       reduction)
-            ck, cv, _ = presses.press_compress(k, v, sc, compression_ratio)
+            ck, cv, _ = presses.press_compress(k, v, sc, compression_ratio,
+                                               0 if window_in_budget else window_size)
+            out.append((ck, cv))
+        return out
+    return run
+
+
+def scored_press_compressor(score_fn, compression_ratio: float) -> Compressor:
+    """Any kvpress ``ScorerPress``: ``score_fn(layer, seq_index, keys, values) -> [1, Hkv, S]`` fp32, then
+    ``ScorerPress.compress``."""
+    def run(hf, i, n):
+        out = []
+        for layer, (k, v) in enumerate(hf):
+            ck, cv, _ = presses.press_compress(k, v, score_fn(layer, i, k, v), compression_ratio)
             out.append((ck, cv))
         return out
     return run

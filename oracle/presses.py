@@ -232,13 +232,15 @@ def gather_tokens(x: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
 # kvpress-style press = score + select + gather
 # --------------------------------------------------------------------------------------------
 def press_compress(keys: torch.Tensor, values: torch.Tensor, scores: torch.Tensor,
-                   compression_ratio: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """kvpress ``ScorerPress.compress``.  Returns ``(K', V', idx[B, Hkv, n_kept])``."""
+                   compression_ratio: float, extra_kept: int = 0) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """kvpress ``ScorerPress.compress``.  Returns ``(K', V', idx[B, Hkv, n_kept])``.  ``extra_kept`` adds that many
+    positions to the budget (the other reading of "keep a quarter plus the window": the SnapKV observation window,
+    which always ranks first, kept ON TOP of ``int(S * (1 - r))`` instead of inside it), capped at the length."""
     if compression_ratio == 0:
         S = keys.shape[2]
         idx = torch.arange(S).expand(keys.shape[0], keys.shape[1], S)
         return keys, values, idx
-    n = n_kept_press(keys.shape[2], compression_ratio)
+    n = min(keys.shape[2], n_kept_press(keys.shape[2], compression_ratio) + extra_kept)
     idx = topk_lowest_index(scores, n)
     return gather_tokens(keys, idx), gather_tokens(values, idx), idx
 

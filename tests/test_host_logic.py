@@ -93,6 +93,74 @@ def test_block_manager_prefix_cache_and_specific_free():
     assert not a.block_table
 
 
+def test_shared_prefix_pages_get_a_private_copy_before_they_are_rewritten():
+    """Two prompts with the same first 512 tokens share two pages.  A compression rewrites leading pages in place:
+    the page manager hands the sequence a fresh page for each shared one it will write, forgets the content keys
+    of rewritten pages, and a later request with that prefix is served only by pages that still hold prompt rows."""
+    bm = BlockManager(10, 256)
+    a = Sequence(list(range(600)))
+    b = Sequence(list(range(512)) + [9] * 88)
+    bm.allocate(a)
+    bm.allocate(b)
+    assert a.block_table[:2] == b.block_table[:2] and bm.shared_positions(a, 3) == [0, 1]
+    assert bm.shared_positions(a, 1) == [0]
+    old = a.block_table[0]
+    free_before = len(bm.free_block_ids)
+    moved = bm.unshare(a, [0])                            # a keeps 100 rows: it rewrites page 0 only
+    assert moved == [(old, a.block_table[0])] and a.block_table[0] != b.block_table[0] == old
+    assert bm.blocks[old].ref_count == 1 and bm.blocks[a.block_table[0]].ref_count == 1
+    assert len(bm.free_block_ids) == free_before - 1 and bm.blocks[a.block_table[0]].hash == -1
+    free_compressed_blocks(bm, FakeRunner({a.seq_id: 100}), [a])
+    assert len(a.block_table) == 1 and bm.blocks[b.block_table[1]].ref_count == 1      # a let go of shared page 1
+    c = Sequence(list(range(600)))                       # same prefix: served by b's untouched pages
+    bm.allocate(c)
+    assert c.block_table[:2] == b.block_table[:2] and c.num_cached_tokens == 512
+    bm.deallocate(c)
+    free_compressed_blocks(bm, FakeRunner({b.seq_id: 300}), [b])       # b rewrites both of its pages, keeps both
+    assert all(bm.blocks[p].hash == -1 and not bm.blocks[p].token_ids for p in b.block_table[:2])
+    d = Sequence(list(range(600)))
+    bm.allocate(d)
+    assert d.num_cached_tokens == 0 and not set(d.block_table) & set(b.block_table)
+    # too few free pages: refused with the tables as they were
+    e, f = Sequence(list(range(7000, 7512))), Sequence(list(range(7000, 7512)))
+    bm2 = BlockManager(2, 256)
+    bm2.allocate(e)
+    bm2.allocate(f)
+    before = list(e.block_table)
+    with pytest.raises(RuntimeError, match="only 0 pages are free"):
+        bm2.unshare(e, [0, 1])
+    assert e.block_table == before and bm2.blocks[before[0]].ref_count == 2
+
+
+def test_runner_refuses_a_batch_that_would_rewrite_a_page_twice():
+    """Without a page manager the runner cannot copy a shared page; it refuses before any launch."""
+    from fastcache_amd._lib import FastcacheError
+    runner = PagedKVRunner(1, 1, 128, num_blocks=4, dtype=torch.float16, device="cpu", image_token_len=0,
+                           compressor=KVPressCompressor("streaming_llm", 0.5))
+    a, b = Sequence(list(range(300))), Sequence(list(range(300)))
+    a.block_table, b.block_table = [0, 1], [0, 2]
+    with pytest.raises(FastcacheError, match="page 0 belongs to several sequences"):
+        runner._compress_enqueue([a, b], 0)
+    assert not runner._launch_started and not runner._compressed_lens
+
+
+def test_synthetic_pool_scatter_is_the_page_formula():
+    """``synth.scatter_into_pool`` (one indexed store per plane and layer) against the defining loop
+    ``pool[table[s // 256], s % 256] = dense[s]`` on a shuffled, ragged case; untouched slots keep the fill value."""
+    from fastcache_amd import synth
+    lens = [300, 17, 256, 513]
+    case = synth.make_paged_case(seed=5, num_layers=2, batch=4, num_kv_heads=3, seq_lens=lens, dtype=torch.float16,
+                                 keep_dense=True, fill_value=7.0, block_size=256)
+    want = torch.full_like(case.kv_cache, 7.0)
+    for layer in range(2):
+        for p, dense in enumerate((case.dense_k, case.dense_v)):
+            for b, (tab, n) in enumerate(zip(case.block_tables, lens)):
+                for t in range(n):
+                    want[p, layer, tab[t // 256], t % 256] = dense[layer, b, :, t]
+    assert torch.equal(case.kv_cache.view(torch.int16), want.view(torch.int16))
+    assert sorted(sum(case.block_tables, [])) != sum(case.block_tables, [])       # the tables really are shuffled
+
+
 def test_sequence_state():
     s = Sequence([1, 2, 3])
     assert not s.is_compressed and s.kv_cache_len == 3 and s.kv_num_blocks == 1
