@@ -1,7 +1,9 @@
-"""The compression-method adapters of the reference that carry device work: ``KVPressMethod``
-(nanovllm/autocompress/methods.py:227-495, a press by name with ``compress(keys, values, **kwargs)``) and
-``QuantizationMethod`` (:520-757), computed by HIP kernels.  The cost profiles and timing heuristics the
-reference attaches to them (A100 constants for its scheduler) are not carried over.
+"""The compression-method adapters of the reference that carry device work: ``MLPCompressionMethod``
+(nanovllm/autocompress/methods.py:122-220, a CCM compressor behind ``compress(keys, values, **kwargs)``),
+``KVPressMethod`` (:227-495, a press by name) and ``QuantizationMethod`` (:520-757), computed by HIP kernels, and
+the factory that hands them out by name (``MethodRegistry`` :787-843, ``get_method`` / ``list_methods`` :846-853).
+The cost profiles and timing heuristics the reference attaches to them (A100 constants for its scheduler) are not
+carried over.
 
 Built: ``int8`` (one scale per row of the last dimension; ``symmetric=False`` gives uint8 codes with a
 ``(scale, zero point)`` pair per row), ``int4`` and ``nf4`` (one scale per group of ``group_size`` elements, two
@@ -14,7 +16,7 @@ describe are what is built, and the third raises here as it does there.
 from __future__ import annotations
 
 from enum import Enum, auto
-from typing import Tuple
+from typing import Dict, List, Tuple
 
 import torch
 
@@ -90,10 +92,58 @@ class QuantizationMethod:
         return ops.dequantize_fp8(quantized, scale, dtype)
 
 
+class MLPCompressionMethod:
+    """A CCM MLP compressor (``BatchedGEMMCompressor``, ``KVCacheLinearDecoupleCompressor``, ...) as a method object.
+
+    ``compress(keys, values, it_len=[image, text], layer_idx=0)`` takes one layer's ``[B, Hkv, S, D]`` tensors (that
+    layer's MLP weights) or all layers' ``[L, B, Hkv, S, D]`` and returns tensors of the same rank with the token axis
+    shortened.  The reference's body stacks keys and values into one ``[2, B, Hkv, S, D]`` tensor and hands it to a
+    compressor that expects a list of per-layer ``(k, v)`` pairs (methods.py:196-207), which only unpacks for a batch
+    of exactly two; what it means to do, the compressor applied to this K and V, is what is built."""
+
+    def __init__(self, compressor=None, compression_ratio: float = 5.0, num_layers: int = 32):
+        self._compressor = compressor
+        self._compression_ratio = compression_ratio
+        self._num_layers = num_layers
+
+    @property
+    def name(self) -> str:
+        return "mlp_compress"
+
+    @property
+    def compression_ratio(self) -> float:
+        return self._compression_ratio
+
+    def compress(self, keys: torch.Tensor, values: torch.Tensor, **kwargs) -> Tuple[torch.Tensor, torch.Tensor]:
+        if self._compressor is None:
+            raise RuntimeError("MLP compressor not initialized")
+        it_len = kwargs.get("it_len", [0, keys.shape[-2]])
+        if keys.dim() == 5:
+            out = self._compressor([(k, v) for k, v in zip(keys, values)], it_len=it_len)
+            return torch.stack([k for k, _ in out]), torch.stack([v for _, v in out])
+        if keys.dim() != 4:
+            raise FastcacheError(f"keys must be [B, Hkv, S, D] or [L, B, Hkv, S, D], got {tuple(keys.shape)}")
+        layer = int(kwargs.get("layer_idx", 0))
+        if hasattr(self._compressor, "compress_layers"):
+            # the chunked entry point addresses a layer's weights by its position in the full list
+            padded = [(keys, values)] * (layer + 1)
+            out = self._compressor.compress_layers(padded, layer, layer + 1, it_len=it_len)
+        elif layer == 0:
+            out = self._compressor([(keys, values)], it_len=it_len)
+        else:
+            raise FastcacheError(f"{type(self._compressor).__name__} has no per-layer entry point (layer_idx={layer})")
+        return out[0][0], out[0][1]
+
+
 class KVPressMethod:
     """A press chosen by name, called outside a model (methods.py:227-495).  The press runs on the HIP kernels of
     ``fastcache_amd.presses``; ``compress`` forwards ``module`` / ``hidden_states`` / ``attentions`` from the keyword
     arguments and hands all of them on as the press's ``kwargs`` (``queries``, ``position_embeddings``, ...)."""
+
+    # the names the reference's registry lists (methods.py:244-330); 'h2o' and the others without a press class
+    # are listed there and rejected at first use, here as well
+    METHOD_NAMES = ("snapkv", "streaming_llm", "observed_attention", "expected_attention", "knorm", "tova", "think",
+                    "simlayer", "h2o")
 
     @staticmethod
     def _press_map():
@@ -138,3 +188,54 @@ class KVPressMethod:
         self._init_press()
         return self._press.compress(module=kwargs.get("module"), hidden_states=kwargs.get("hidden_states"),
                                     keys=keys, values=values, attentions=kwargs.get("attentions"), kwargs=kwargs)
+
+
+class MethodRegistry:
+    """Methods by name (methods.py:787-843): ``mlp`` / ``mlp_compress`` / ``batched_gemm``; ``kvpress_<press>`` or
+    a bare press name; ``quant_<type>`` or ``int8`` / ``int4`` / ``fp8`` / ``nf4``; anything registered with
+    ``register``.  Instances are cached per name and keyword arguments when the arguments are hashable (a compressor
+    module is, by identity)."""
+    _methods: Dict[str, type] = {}
+    _instances: Dict[tuple, object] = {}
+
+    @classmethod
+    def register(cls, name: str, method_class: type) -> None:
+        cls._methods[name] = method_class
+
+    @classmethod
+    def create(cls, name: str, **kwargs):
+        try:
+            key = (name, frozenset(kwargs.items()))
+            hash(key)
+        except TypeError:
+            key = None
+        if key is not None and key in cls._instances:
+            return cls._instances[key]
+        if name in ("mlp", "mlp_compress", "batched_gemm"):
+            instance = MLPCompressionMethod(**kwargs)
+        elif name.startswith("kvpress_") or name in KVPressMethod.METHOD_NAMES:
+            instance = KVPressMethod(name.replace("kvpress_", ""), **kwargs)
+        elif name.startswith("quant_") or name in ("int8", "int4", "fp8", "nf4"):
+            instance = QuantizationMethod(name.replace("quant_", ""), **kwargs)
+        elif name in cls._methods:
+            instance = cls._methods[name](**kwargs)
+        else:
+            raise ValueError(f"Unknown compression method: {name}")
+        if key is not None:
+            cls._instances[key] = instance
+        return instance
+
+    @classmethod
+    def list_methods(cls) -> List[str]:
+        names = set(cls._methods) | {"mlp", "mlp_compress"}
+        names |= {f"kvpress_{m}" for m in KVPressMethod.METHOD_NAMES}
+        names |= {"quant_int8", "quant_int4", "quant_fp8", "quant_nf4"}
+        return sorted(names)
+
+
+def get_method(name: str, **kwargs):
+    return MethodRegistry.create(name, **kwargs)
+
+
+def list_methods() -> List[str]:
+    return MethodRegistry.list_methods()

@@ -178,11 +178,24 @@ def snapkv_press_preferred(keys: FcKvView, num_q_heads: int, window: int, comput
 def snapkv_press(keys: FcKvView, values: FcKvView, queries: torch.Tensor, window: int, kernel_size: int, k: int,
                  causal_window: bool = True, reduction: str = "mean", scale: Optional[float] = None,
                  seq_lens: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                 n_kept: Optional[torch.Tensor] = None, ragged: bool = False):
+                 n_kept=None, ragged: bool = False, host_lens=None):
     """SnapKV scores, selection (the window always kept; ``k`` or ``n_kept[b]`` positions per row, window included,
     more than the window) and in-place compaction of both planes, each (layer, sequence, kv head) column by one
     workgroup in one launch; then the window fill of the scores.  Returns ``(scores, indices)`` equal to
-    ``snapkv_score`` + ``select_compact``.  Shapes must satisfy :func:`snapkv_press_fits`."""
+    ``snapkv_score`` + ``select_compact``.  Shapes must satisfy :func:`snapkv_press_fits`.
+
+    ``n_kept``: the kept counts per sequence as Python ints (checked here: the kernel leaves a sequence longer than the
+    window untouched when its count does not exceed the window, which a caller that then shortens the sequence
+    would not notice; ``host_lens`` names the sequences no longer than the window, which are exempt).  A device
+    tensor is passed through unchecked for callers that have validated the counts themselves."""
+    if n_kept is not None and not isinstance(n_kept, torch.Tensor):
+        counts = [int(c) for c in n_kept]
+        lens_h = list(host_lens) if host_lens is not None else [keys.max_seq_len] * len(counts)
+        bad = [b for b, (c, n) in enumerate(zip(counts, lens_h)) if n > window and not window < c <= min(k, n)]
+        if len(counts) != keys.batch or bad:
+            raise FastcacheError(f"snapkv_press: kept counts must exceed the window ({window}) and fit the index row "
+                                 f"({k}) for every sequence longer than the window; offending sequences: {bad}")
+        n_kept = torch.tensor(counts, dtype=torch.int32, device=queries.device)
     if queries.dim() == 4:
         queries = queries.unsqueeze(0)
         if lse is not None and lse.dim() == 3:

@@ -108,9 +108,8 @@ def snapkv_compress_paged(kv_cache: torch.Tensor, block_tables: torch.Tensor, se
             ops.snapkv_press_preferred(kview, queries.shape[-3], window_size,
                                        torch.cuda.get_device_properties(kv_cache.device).multi_processor_count)):
         same = len(set(kept)) == 1 and len(set(lens)) == 1
-        n_kept = None if same else torch.tensor(kept, dtype=torch.int32, device=kv_cache.device)
         scores, idx = ops.snapkv_press(kview, vview, queries, window_size, kernel_size, width, causal_window,
-                                       reduction, seq_lens=seq_lens, n_kept=n_kept)
+                                       reduction, seq_lens=seq_lens, n_kept=None if same else kept, host_lens=lens)
         return PressResult(idx, width, scores, None if same else list(kept))
     scores = ops.snapkv_score(kview, queries, window_size, kernel_size, causal_window, reduction,
                               seq_lens=seq_lens)

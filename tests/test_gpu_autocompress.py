@@ -348,6 +348,48 @@ def test_kvpress_method_adapter(dev):
         ac.KVPressMethod("h2o").compress(k, v)
 
 
+def test_mlp_method_adapter_and_registry(dev):
+    """``get_method('mlp', compressor=...)``: one layer's K and V (with ``layer_idx``) and all layers at once against
+    the oracle's MLP compressor; the registry resolves every family of names, caches instances and rejects others."""
+    from types import SimpleNamespace
+    from fastcache_amd.kernels import BatchedGEMMCompressor
+    from fastcache_amd.utils_ccm import KVCacheLinearDecoupleCompressor
+    dtype, L, B, H, S, cf = torch.float16, 3, 2, 2, 90, 2
+    cfg = SimpleNamespace(text_config=SimpleNamespace(num_hidden_layers=L, num_key_value_heads=H, hidden_size=H * 128,
+                                                      head_dim=128, num_attention_heads=H))
+    torch.manual_seed(11)
+    orig = KVCacheLinearDecoupleCompressor(cfg, compression_factor=cf).to(dev).to(dtype).eval()
+    sd = occm.reference_init_state_dict("linear_decouple", L, 128, cf, seed=11)
+    bat = BatchedGEMMCompressor(num_layers=L, num_heads=H, head_dim=128, compression_factor=cf)
+    bat.load_from_original_compressor(orig)
+    g = torch.Generator().manual_seed(3)
+    k = torch.randn(L, B, H, S, 128, generator=g).to(dtype)
+    v = torch.randn(L, B, H, S, 128, generator=g).to(dtype)
+    it_len = [50, 40]
+    ref = occm.linear_decouple_forward([(k[l], v[l]) for l in range(L)], it_len, sd, cf, 1)
+    m = ac.get_method("mlp", compressor=bat)
+    assert m.name == "mlp_compress" and ac.get_method("mlp", compressor=bat) is m
+    ck, cv = m.compress(k[1].to(dev), v[1].to(dev), it_len=it_len, layer_idx=1)
+    assert ck.shape == (B, H, 45, 128)
+    assert_mlp_close(ck.cpu(), ref[1][0], dtype)
+    assert_mlp_close(cv.cpu(), ref[1][1], dtype)
+    ak, av = ac.get_method("mlp_compress", compressor=orig).compress(k.to(dev), v.to(dev), it_len=it_len)
+    assert ak.shape == (L, B, H, 45, 128) and torch.equal(ak[1], ck) and torch.equal(av[1], cv)
+    for l in range(L):
+        assert_mlp_close(ak[l].cpu(), ref[l][0], dtype)
+    with pytest.raises(RuntimeError, match="not initialized"):
+        ac.MLPCompressionMethod().compress(k[0].to(dev), v[0].to(dev))
+    # the other families of names
+    assert isinstance(ac.get_method("kvpress_snapkv", compression_ratio=0.5), ac.KVPressMethod)
+    assert isinstance(ac.get_method("knorm"), ac.KVPressMethod) and ac.get_method("knorm").name == "kvpress_knorm"
+    assert ac.get_method("quant_nf4").name == "quant_nf4" and ac.get_method("int8").name == "quant_int8"
+    assert {"mlp", "kvpress_snapkv", "quant_int4"} <= set(ac.list_methods())
+    ac.MethodRegistry.register("mine", ac.MLPCompressionMethod)
+    assert "mine" in ac.list_methods() and isinstance(ac.get_method("mine"), ac.MLPCompressionMethod)
+    with pytest.raises(ValueError, match="Unknown compression method"):
+        ac.get_method("zip")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("d", [128, 64, 256, 40])
 def test_quantisers_special_rows_all_row_lengths(dev, dtype, d):

@@ -95,22 +95,30 @@ def test_config1_knorm_full(dev):
 
 
 def test_config2_snapkv_full(dev):
+    """Both readings of "keep 25 % plus the window": the window inside the budget (1024 kept, what the benchmark's
+    headline measures) and on top of it (1088 kept), each on a pool of its own, every column against the oracle."""
     L, B, Hq, Hkv, S, W, ksz, ratio = 36, 8, 32, 8, 4096, 64, 7, 0.75
     case = synth.snapkv_case(seed=0, device=dev, device_draw=True)
     pool, tables, lens = case.kv_cache, case.table_tensor(dev), case.lens_tensor(dev)
     before = pool.clone()
     res = paged_press.snapkv_compress_paged(pool, tables, lens, S, case.queries, ratio, W, ksz, True, "sum")
+    pool_top = before.clone()
+    res_top = paged_press.snapkv_compress_paged(pool_top, tables, lens, S, case.queries, ratio, W, ksz, True, "sum",
+                                                window_in_budget=False)
     torch.cuda.synchronize()
-    n = 1024
-    assert res.n_kept == n
-    check_index_properties(res.indices, S, n)
-    assert bool((res.indices[..., -W:] == torch.arange(S - W, S, device=dev, dtype=torch.int32)).all())
-    check_compaction(pool, before, tables, res.indices, S, n)
+    n, n_top = 1024, 1088
+    assert res.n_kept == n and res_top.n_kept == n_top and res_top.indices.shape[-1] == n_top
+    for r, p, m in ((res, pool, n), (res_top, pool_top, n_top)):
+        check_index_properties(r.indices, S, m)
+        assert bool((r.indices[..., -W:] == torch.arange(S - W, S, device=dev, dtype=torch.int32)).all())
+        check_compaction(p, before, tables, r.indices, S, m)
+    del pool_top
+    assert torch.equal(res.scores, res_top.scores)               # the budget does not enter the scoring
     # softmax mass: unpooled scores would sum to <= W*G per row; pooling keeps the sum within it
     body = res.scores[..., :S - W]
     assert bool((body >= 0).all()) and float(body.sum(-1).max()) <= W * (Hq // Hkv) * 1.001
     # every column against the oracle's scoring evaluated in fp32 on the device, layer by layer
-    n_tie = 0
+    n_tie = n_tie_top = 0
     for layer in range(L):
         kd = dense_from_pool(before[0, layer:layer + 1], tables, S)[0]                     # [B, Hkv, S, D]
         ref = opress.snapkv_score(case.queries[layer], kd, W, ksz, True, "sum")             # [B, Hkv, S] fp32
@@ -119,7 +127,9 @@ def test_config2_snapkv_full(dev):
         ref_full = ref.clone()
         ref_full[..., S - W:] = got[..., S - W:]
         n_tie += check_selection_against_scores(res.indices[layer], ref_full, n)
+        n_tie_top += check_selection_against_scores(res_top.indices[layer], ref_full, n_top)
     assert n_tie <= 1e-4 * L * B * Hkv * n, n_tie        # kept positions that fp32 scoring does not decide
+    assert n_tie_top <= 1e-4 * L * B * Hkv * n_top, n_tie_top
     # CPU oracle on a sample of layers and sequences
     for layer, b in ((0, 0), (17, 3), (35, 7)):
         k = dense_from_pool(before[0, layer:layer + 1], tables[b:b + 1], S)[0].cpu()
