@@ -194,12 +194,16 @@ def paged_view(plane: torch.Tensor, block_tables: torch.Tensor, seq_lens: Option
         require_gpu(seq_lens, "seq_lens")
     L, _, bs, H, D = plane.shape
     st = [plane.stride(i) if plane.shape[i] > 1 else 0 for i in range(4)]
-    return FcKvView(
+    view = FcKvView(
         base=plane.data_ptr(), stride_layer=st[0], stride_block=st[1], stride_batch=0,
         stride_token=st[2], stride_head=st[3],
         block_tables=block_tables.data_ptr(), table_stride=block_tables.shape[1], block_size=bs,
         dtype=dtype_code(plane.dtype), num_layers=L, batch=block_tables.shape[0], num_kv_heads=H,
         head_dim=D, max_seq_len=int(max_seq_len), seq_lens=ptr(seq_lens))
+    # the struct carries raw addresses: the view keeps the tensors alive, so that a table or length tensor built in
+    # the call expression cannot be handed back to the allocator (and reused) before the kernels have read it
+    view._tensors = (plane, block_tables, seq_lens)
+    return view
 
 
 def dense_view(t: torch.Tensor, seq_len: Optional[int] = None) -> FcKvView:
@@ -212,8 +216,10 @@ def dense_view(t: torch.Tensor, seq_len: Optional[int] = None) -> FcKvView:
         raise FastcacheError("dense KV must be [B, Hkv, S, D] or [L, B, Hkv, S, D] with contiguous D")
     L, B, H, S, D = t.shape
     st = [t.stride(i) if t.shape[i] > 1 else 0 for i in range(4)]  # strides of size-1 axes are arbitrary
-    return FcKvView(
+    view = FcKvView(
         base=t.data_ptr(), stride_layer=st[0], stride_block=0, stride_batch=st[1],
         stride_token=st[3], stride_head=st[2], block_tables=None, table_stride=0, block_size=1,
         dtype=dtype_code(t.dtype), num_layers=L, batch=B, num_kv_heads=H, head_dim=D,
         max_seq_len=int(S if seq_len is None else seq_len), seq_lens=None)
+    view._tensors = (t,)          # as in paged_view: the view keeps what it points at alive
+    return view

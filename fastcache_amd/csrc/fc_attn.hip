@@ -1,9 +1,9 @@
 // Decode-side kernels over the paged cache: append one K/V row per sequence, advance the lengths,
-// and single-query paged attention (split over chunks of 256 to 512 tokens, then merged).
+// and single-query paged attention (split over chunks of 256 to 1024 tokens, then merged).
 //
 // Attention is HBM-bound (one pass over K and V, ~1 FLOP per byte per query head), so the kernel is
-// organised around keeping loads in flight.  A workgroup owns one (sequence, kv head, 256-token
-// chunk) and serves all query heads of the group from the same K/V bytes; each of its four
+// organised around keeping loads in flight.  A workgroup owns one (sequence, kv head, chunk of
+// 256..1024 tokens, a multiple of 32 the host picks per launch) and serves all query heads of the group from the same K/V bytes; each of its four
 // wavefronts streams two 32-token K tiles and then the matching V tiles from global memory straight
 // into a private two-stage LDS ring (global_load_lds, rows XOR-swizzled), 16 KB per wavefront in
 // flight, no workgroup barrier between a load and its use.
@@ -15,6 +15,8 @@
 // chunks of a sequence.  Grid sizes depend only on the view's max_seq_len, never on the lengths on
 // the device, so both launches can be replayed from a graph while the lengths grow.
 #include "fc_common.h"
+#include <atomic>
+#include <stdlib.h>
 
 #define DA_THREADS 256
 #define DA_CHUNK 256               // smallest chunk (tokens per workgroup); it sizes the workspace
@@ -44,6 +46,10 @@ __device__ __forceinline__ unsigned short da_pack(float f) {
 
 #define DA_PV_MFMA_MIN 8               // heads per workgroup from which p * V runs on the matrix pipe (measured: no gain below)
 #define DA_TILE 32                     // keys per tile: one MFMA block, 8 KB of K or V rows
+// The chunk's block-table entries are prefetched one per lane of a wavefront: the largest chunk in the smallest
+// page the fast path takes (32 tokens, block_shift >= 5), starting anywhere in a page, must span at most 64 entries.
+static_assert(DA_CHUNK_MAX / DA_TILE + 1 <= 64, "a chunk's block-table entries must fit one per lane");
+static_assert(DA_CHUNK % DA_TILE == 0 && DA_CHUNK_MAX % 64 == 0, "chunk bounds: whole tiles, whole statistics registers");
 #define DA_TILEB (DA_TILE * 256)
 #define DA_RING (4 * 2 * DA_TILEB)     // four wavefronts, two stages each
 
@@ -512,14 +518,15 @@ extern "C" int64_t fc_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_h
 
 // compute units of the current device (0 if the query fails), cached per device
 static int da_compute_units() {
-  static int cus[64];
+  static std::atomic<int> cus[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (cus[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus[dev] = n;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 0) n = 0;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  return cus[dev];
+  return n;
 }
 
 // Checks and launches shared by the entry points; `workspace` is a device address.
@@ -631,7 +638,22 @@ extern "C" int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cac
 static __device__ __align__(256) unsigned char scratch[DA_STATIC_BYTES];
 
 #define DA_MAX_DEVICES 64
-static void* da_scratch_ptr[DA_MAX_DEVICES];   // filled per device on first use; a repeated look-up gives the same value
+// filled per device on first use; two threads racing here store the same value
+static std::atomic<void*> da_scratch_ptr[DA_MAX_DEVICES];
+// Every call on a device shares that device's array, so two calls whose kernels overlap (different streams, or a
+// graph replay beside an eager call) corrupt each other's chunk partials.  The library cannot see that in general
+// without synchronising; with FC_STATIC_GUARD=1 in the environment it checks the one case it can name cheaply: a
+// call on another stream than the previous call's while that stream still has work pending is refused.  The check
+// queries the previous stream, so leave it off when streams are being captured.
+static std::atomic<void*> da_last_stream[DA_MAX_DEVICES];
+static std::atomic<int> da_last_stream_set[DA_MAX_DEVICES];
+static bool da_guard_enabled() {
+  static const bool on = [] {
+    const char* e = getenv("FC_STATIC_GUARD");
+    return e && e[0] && e[0] != '0';
+  }();
+  return on;
+}
 
 extern "C" int64_t fc_decode_attn_static_capacity(void) { return DA_STATIC_BYTES; }
 
@@ -649,11 +671,25 @@ extern "C" int fc_decode_attn_static(const fc_kv_view* k_cache, const fc_kv_view
   int dev = -1;
   FC_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < DA_MAX_DEVICES, FC_EUNSUPPORTED,
              "%s: no current device below %d", who, DA_MAX_DEVICES);
-  void* ws = da_scratch_ptr[dev];
+  void* ws = da_scratch_ptr[dev].load(std::memory_order_acquire);
   if (!ws) {
     const hipError_t e = hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch));
     FC_REQUIRE(e == hipSuccess && ws, FC_ELAUNCH, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
-    da_scratch_ptr[dev] = ws;
+    da_scratch_ptr[dev].store(ws, std::memory_order_release);
+  }
+  if (da_guard_enabled()) {
+    if (da_last_stream_set[dev].load(std::memory_order_acquire)) {
+      void* last = da_last_stream[dev].load(std::memory_order_acquire);
+      if (last != stream) {
+        const hipError_t q = hipStreamQuery((hipStream_t)last);
+        if (q != hipSuccess) (void)hipGetLastError();
+        FC_REQUIRE(q != hipErrorNotReady, FC_EINVAL,
+                   "%s: the previous call on this device used another stream that still has work pending; calls "
+                   "that share the built-in buffer must not overlap", who);
+      }
+    }
+    da_last_stream[dev].store(stream, std::memory_order_release);
+    da_last_stream_set[dev].store(1, std::memory_order_release);
   }
   return da_enqueue(who, k_cache, v_cache, layer, q, out, num_q_heads, context_lens, scale, ws, DA_STATIC_BYTES,
                     stream);

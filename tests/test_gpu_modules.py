@@ -405,7 +405,9 @@ def test_async_compression_manager_states_and_effective_len(dev):
     # a compressor that works in place and fails after it may have launched: the rows are no longer trustworthy,
     # the sequence is marked FAILED and asking for its length raises instead of handing out a stale number
     class Halfway:
-        def paged_forward(self, *a, **k):
+        def paged_forward(self, kv_cache, block_tables, seq_lens, seq_len, *a, **k):
+            from fastcache_amd import _lib, ops
+            ops.knorm_score(_lib.paged_view(kv_cache[0], block_tables, seq_lens, seq_len), kv_cache.device)
             raise RuntimeError("second launch rejected")
     half = PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0, compressor=Halfway())
     hmgr = AsyncCompressionManager(half)
@@ -414,6 +416,15 @@ def test_async_compression_manager_states_and_effective_len(dev):
     assert hmgr.seq_states[seqs[0].seq_id] == CompressionState.FAILED
     with pytest.raises(Exception, match="prefill again"):
         hmgr.get_effective_kv_len(seqs[0])
+    # the same kind of compressor failing in its host-side checks, before anything was enqueued: the cache is as it was
+    class Early:
+        def paged_forward(self, *a, **k):
+            raise TypeError("image segment cannot be compressed")
+    early = PagedKVRunner(L, H, 128, num_blocks=8, dtype=dtype, device=dev, image_token_len=0, compressor=Early())
+    emgr = AsyncCompressionManager(early)
+    emgr.start_async_compression(seqs[:1], image_len=0)
+    emgr.wait_all_compressions()
+    assert emgr.seq_states[seqs[0].seq_id] == CompressionState.NONE and emgr.get_effective_kv_len(seqs[0]) == S
     assert AsyncCompressionManager(PagedKVRunner(L, H, 128, 2, dtype, dev)).start_async_compression(seqs) is None
 
 

@@ -225,13 +225,13 @@ def test_snapkv_press_refuses_what_it_cannot_take(dev):
     two = synth.make_paged_case(seed=3, num_layers=1, batch=2, num_kv_heads=1, seq_lens=[512, 300], dtype=torch.bfloat16,
                                 num_q_heads=4, window=64)
     pool2 = two.kv_cache.to(dev)
-    k2, v2 = (_lib.paged_view(pool2[p], two.table_tensor(dev), two.lens_tensor(dev), 512) for p in range(2))
+    tables2, lens2, q2 = two.table_tensor(dev), two.lens_tensor(dev), two.queries.to(dev)
+    k2, v2 = (_lib.paged_view(pool2[p], tables2, lens2, 512) for p in range(2))
     with pytest.raises(_lib.FastcacheError, match=r"offending sequences: \[1\]"):
-        ops.snapkv_press(k2, v2, two.queries.to(dev), 64, 7, 128, seq_lens=two.lens_tensor(dev), n_kept=[128, 64],
-                         host_lens=[512, 300])
+        ops.snapkv_press(k2, v2, q2, 64, 7, 128, seq_lens=lens2, n_kept=[128, 64], host_lens=[512, 300])
     assert torch.equal(pool2, two.kv_cache.to(dev))
-    ops.snapkv_press(k2, v2, two.queries.to(dev), 64, 7, 128, seq_lens=two.lens_tensor(dev), n_kept=[128, 75],
-                     host_lens=[512, 300])
+    ops.snapkv_press(k2, v2, q2, 64, 7, 128, seq_lens=lens2, n_kept=[128, 75], host_lens=[512, 300])
+    torch.cuda.synchronize()
     long = synth.make_paged_case(seed=2, num_layers=1, batch=1, num_kv_heads=1, seq_lens=[20000], dtype=torch.bfloat16,
                                  num_q_heads=4, window=64)
     pool = long.kv_cache.to(dev)
