@@ -608,30 +608,73 @@ class DecodeWorkload(Workload):
 # calibration: a plain copy of known size through fc_copy_tokens (for scaling FETCH_SIZE / WRITE_SIZE)
 # ---------------------------------------------------------------------------------------------------
 class CopyWorkload(Workload):
+    """Plain streams of known size, for the counter calibration (`copy`) and as the practical ceilings the HBM-bound
+    kernels are compared with: this library's copy kernel, the runtime's device-to-device copy (through torch and
+    called directly), a torch elementwise kernel, read-only streams (this library's and torch's reduction) and
+    write-only streams (torch's fill kernel, the runtime's memset).  Each moves 512 MiB per tensor."""
     name = "copy-calibration-1GiB"
     dtype_name = "bf16"
     kernel_name = "compact_kernel"
     metric = "tokens copied/sec"
     unit = "tokens/s"
+    KINDS = {  # kind -> (workload name, kernel name as a trace shows it, tensors read, tensors written)
+        "compact": ("copy-calibration-1GiB", "compact_kernel", 1, 1),
+        "torch-copy": ("copy-torch-copy_-1GiB", "hipMemcpyAsync device to device (torch Tensor.copy_)", 1, 1),
+        "hip-memcpy": ("copy-hipMemcpyDtoDAsync-1GiB", "hipMemcpyDtoDAsync", 1, 1),
+        "torch-kernel": ("copy-torch-elementwise-1GiB", "torch elementwise kernel (torch.neg, out=)", 1, 1),
+        "read": ("read-key-channel-energy-512MiB", "key_channel_energy_kernel", 1, 0),
+        "torch-read": ("read-torch-sum-512MiB", "torch reduce kernel (Tensor.sum over the bytes viewed as fp32)", 1, 0),
+        "torch-fill": ("write-torch-fill-512MiB", "torch fill kernel (Tensor.fill_)", 0, 1),
+        "hip-memset": ("write-hipMemsetAsync-512MiB", "hipMemsetAsync", 0, 1),
+    }
 
-    def __init__(self, seed, device):
+    def __init__(self, seed, device, kind="compact"):
         super().__init__()
-        self.device = device
-        L, B, H, S = 1, 4, 8, 65536                       # 4 * 8 * 65536 * 256 B = 512 MiB per tensor
+        self.device, self.kind = device, kind
+        self.name, self.kernel_name, n_read, n_written = self.KINDS[kind]
+        # 16 * 16 * 8 * 1024 rows of 256 B = 512 MiB per tensor, as 2048 (layer, sequence, head) columns: this library's
+        # kernels take a workgroup per column, so a tensor of a few very long columns would measure the grid, not the memory
+        L, B, H, S = 16, 16, 8, 1024
         self.src = torch.randn((L, B, H, S, D), device=device, dtype=torch.float32).to(torch.bfloat16)
         self.dst = torch.empty_like(self.src)
         self.S = S
         self.tokens_per_step = B * S
-        self.kernel_bytes = 2 * self.src.numel() * 2      # read once + written once
+        self.nbytes = self.src.numel() * 2
+        self.kernel_bytes = (n_read + n_written) * self.nbytes
         self.pass_bytes = self.kernel_bytes
+        self.n_read, self.n_written = n_read, n_written
+        self.hip = None
+        if kind in ("hip-memcpy", "hip-memset"):
+            import ctypes
+            self.hip = ctypes.CDLL("libamdhip64.so")
+            self.hip.hipMemcpyDtoDAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+            self.hip.hipMemsetAsync.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
 
     def config(self):
-        return {"workload": self.name, "bytes_read": self.kernel_bytes // 2, "bytes_written": self.kernel_bytes // 2}
+        return {"workload": self.name, "bytes_read": self.n_read * self.nbytes, "bytes_written": self.n_written * self.nbytes}
 
     def step(self):
         from fastcache_amd import _lib, ops
+        st = torch.cuda.current_stream().cuda_stream
         with self.br:
-            ops.copy_tokens(_lib.dense_view(self.src), _lib.dense_view(self.dst), 0, self.S, 0)
+            if self.kind == "compact":
+                ops.copy_tokens(_lib.dense_view(self.src), _lib.dense_view(self.dst), 0, self.S, 0)
+            elif self.kind == "torch-copy":
+                self.dst.copy_(self.src)
+            elif self.kind == "hip-memcpy":
+                if self.hip.hipMemcpyDtoDAsync(self.dst.data_ptr(), self.src.data_ptr(), self.nbytes, st) != 0:
+                    raise RuntimeError("hipMemcpyDtoDAsync failed")
+            elif self.kind == "torch-kernel":
+                torch.neg(self.src, out=self.dst)
+            elif self.kind == "read":
+                ops.key_channel_energy(_lib.dense_view(self.src), self.device)
+            elif self.kind == "torch-read":
+                self.src.view(torch.float32).sum()
+            elif self.kind == "torch-fill":
+                self.dst.fill_(1.5)
+            elif self.kind == "hip-memset":
+                if self.hip.hipMemsetAsync(self.dst.data_ptr(), 0, self.nbytes, st) != 0:
+                    raise RuntimeError("hipMemsetAsync failed")
 
     def cpu_baseline(self, budget_s=0):
         threads = _cpu_threads()
@@ -652,7 +695,11 @@ def _separate(w, three):
     return w
 
 
-WORKLOADS = {"copy": CopyWorkload, "snapkv": SnapKVWorkload, "knorm": KnormWorkload, "knorm-3": KnormThreeLaunchWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
+CEILINGS = ("compact", "torch-copy", "hip-memcpy", "torch-kernel", "read", "torch-read", "torch-fill", "hip-memset")
+
+WORKLOADS = {"copy": CopyWorkload,
+             **{f"stream-{k}": (lambda seed, dev, k=k: CopyWorkload(seed, dev, kind=k)) for k in CEILINGS},
+             "snapkv": SnapKVWorkload, "knorm": KnormWorkload, "knorm-3": KnormThreeLaunchWorkload, "ccm": CCMWorkload, "decode": DecodeWorkload,
              "hybrid": lambda seed, dev: CCMWorkload(seed, dev, hybrid=True),
              # cfg2 with the window queries' log-sum-exp handed in (not the BASELINE metric: the reference has no such input)
              "snapkv-lse": lambda seed, dev: SnapKVWorkload(seed, dev, given_lse=True),
@@ -791,6 +838,9 @@ def main():
                     help="one configuration alone; default: cfg2 as the headline plus every configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--hbm-ceilings", action="store_true",
+                    help="plain copy / read / write streams of known size (this library's, torch's, the runtime's): "
+                         "what the memory system delivers to the simplest kernels; prints one JSON line and exits")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -812,6 +862,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     cpu, check = not args.no_cpu_baseline, not args.no_check
+    if args.hbm_ceilings:
+        rows = {}
+        for kind in CEILINGS:
+            r = measure(f"stream-{kind}", args.seed, dev, args.steps, args.warmup, False, 0.0, False, min_warm_s=0.2)
+            rows[kind] = {"workload": r["config"]["workload"], "kernel": r["roofline"]["kernel"],
+                          "bytes_read": r["config"]["bytes_read"], "bytes_written": r["config"]["bytes_written"],
+                          "ms": r["roofline"]["kernel_ms"], "GB/s": r["roofline"]["achieved"],
+                          "frac_of_8TB/s": r["roofline"]["frac"],
+                          "sustained_ms": r["sustained"]["ms_per_step"] if r["sustained"] else None}
+        print(json.dumps({"hbm_ceilings": rows, "steps": args.steps, "warmup": args.warmup}), flush=True)
+        return
 
     head_name = args.workload or "snapkv"
     head = measure(head_name, args.seed, dev, args.steps, args.warmup, cpu, 12.0, check)

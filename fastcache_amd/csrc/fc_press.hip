@@ -42,7 +42,7 @@ __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView 
   extern __shared__ __align__(16) float sc[];  // [smax] scores of the column, then the kept positions
   int* sel = reinterpret_cast<int*>(sc + smax);
   __shared__ int ktbl[CP_TBL], vtbl[CP_TBL];
-  __shared__ TkShared<THREADS> sh;
+  __shared__ TkArea<THREADS> sh;
 
   int h, b, l;
   kp_column(h, b, l, kv.num_kv_heads, kv.batch, kv.num_layers);
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(THREADS) void knorm_press_kernel(KvView kv, KvView 
   int kk = n_kept ? n_kept[b] : k;
   kk = min(min(kk, S), index_stride);
   if (kk <= 0) return;
-  kp_select_and_move<EB, THREADS>(kv, vv, ktbl, k_lds, vtbl, v_lds, sc, sel, sh, l, b, h, S, kk, idx_row);
+  kp_select_and_move<EB, THREADS, false>(kv, vv, ktbl, k_lds, vtbl, v_lds, sc, sel, sh, nullptr, l, b, h, S, kk, 0, idx_row);
 }
 
 // Selection and compaction of a column from scores that another kernel wrote (any press whose scores are per
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(THREADS) void select_compact_kernel(KvView kv, KvVi
   extern __shared__ __align__(16) float sc[];  // [smax] scores of the column, then the kept positions
   int* sel = reinterpret_cast<int*>(sc + smax);
   __shared__ int ktbl[CP_TBL], vtbl[CP_TBL];
-  __shared__ TkShared<THREADS> sh;
+  __shared__ TkArea<THREADS> sh;
   int h, b, l;
   kp_column(h, b, l, kv.num_kv_heads, kv.batch, kv.num_layers);
   const int tid = threadIdx.x;
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(THREADS) void select_compact_kernel(KvView kv, KvVi
   bool k_lds, v_lds;
   kp_tables<THREADS>(kv, vv, ktbl, vtbl, b, S, k_lds, v_lds);
   __syncthreads();
-  kp_select_and_move<EB, THREADS>(kv, vv, ktbl, k_lds, vtbl, v_lds, sc, sel, sh, l, b, h, S, kk,
+  kp_select_and_move<EB, THREADS, false>(kv, vv, ktbl, k_lds, vtbl, v_lds, sc, sel, sh, nullptr, l, b, h, S, kk, 0,
                                   indices + row_id * index_stride);
 }
 

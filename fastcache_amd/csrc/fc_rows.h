@@ -120,3 +120,91 @@ __device__ __forceinline__ void cp_walk(const KvView& src, const KvView& dst, co
     behind = store_rows(bufb, okb, j0 + CH);
   }
 }
+
+// ---- the in-place walk of a paged column over precomputed page addresses ---------------------------------------------
+// cp_walk computes every row's address from the view (table look-up, two 64-bit multiply-adds, the unallocated-page
+// select), about thirty vector instructions per row and lane for source and destination together.  A press that
+// compacts a column onto itself can do with far fewer: the address of (page i, slot 0) of this column's layer and head
+// is put in LDS once per page (ptbl), a source row then costs one table read, one 24-bit multiply-add and a 64-bit
+// add, and a chunk's destination rows share one page, so their address is a scalar base plus a per-lane offset that
+// never changes.  Conditions (cp_pages_ok, and every page of the sequence allocated): power-of-two pages that hold a
+// whole chunk, at most CP_PT pages, a token stride below 2^24 bytes.
+#define CP_PT 256
+
+template <int EB, int THREADS>
+__device__ __forceinline__ bool cp_pages_ok(const KvView& v, int S) {
+  constexpr int CH = (THREADS / (FC_HEAD_DIM * EB / 16)) * CP_R;
+  return v.block_tables != nullptr && v.block_shift >= 0 && v.block_size >= CH && S > 0 &&
+         ((S - 1) >> v.block_shift) < CP_PT && v.stride_token > 0 && v.stride_token * EB < (1ll << 24);
+}
+
+// ptbl[i] = address of token 0 of page i of the column whose (layer, head) offset `colbase` carries; tbl = the
+// sequence's block-table row in LDS.  Returns (to every thread, behind a barrier) whether all pages are allocated.
+template <int EB, int THREADS>
+__device__ __forceinline__ bool cp_fill_pages(const KvView& v, const int* tbl, char* colbase, int S,
+                                              unsigned long long* ptbl) {
+  int bad = 0;
+  for (int i = threadIdx.x; i <= ((S - 1) >> v.block_shift); i += THREADS) {
+    const int blk = tbl[i];
+    bad |= blk < 0;
+    ptbl[i] = (unsigned long long)(uintptr_t)(colbase + (long long)max(blk, 0) * v.stride_block * EB);
+  }
+  return !__syncthreads_or(bad);
+}
+
+// One plane's page addresses and geometry for the walks below.
+struct CpPages {
+  const unsigned long long* ptbl;   // LDS: address of token 0 of page i (layer and head applied)
+  int shift;                        // log2 of the page size
+  unsigned tok_bytes;               // bytes between consecutive tokens of a page
+};
+
+// Rows j = 0 .. n-1 of BOTH planes: token j <- token sel[j] (ascending, sel[j] >= j, all below the sequence length; sel
+// in LDS), in place.  A chunk's K and V rows are loaded together, the workgroup waits for them and synchronises, and
+// only then are they stored; the next chunk's loads follow the stores at once (the stores are not waited for).
+template <int EB, int THREADS>
+__device__ __forceinline__ void cp_walk_pages(const CpPages& kp, const CpPages& vp, int n, const int* sel) {
+  constexpr int LPR = FC_HEAD_DIM * EB / 16;
+  constexpr int RPP = THREADS / LPR;
+  constexpr int CH = RPP * CP_R;   // tokens per chunk
+  const int tid = threadIdx.x;
+  const int tg = tid / LPR;
+  const unsigned lane_b = (unsigned)(tid % LPR) * 16u;
+
+  auto load_rows = [&](const CpPages& pl, cp_u32x4 (&buf)[CP_R], int j0) {
+    const unsigned slot_mask = (1u << pl.shift) - 1u;
+#pragma unroll
+    for (int u = 0; u < CP_R; ++u) {
+      const int j = min(j0 + u * RPP + tg, n - 1);   // rows past the end re-read the last one and are not stored
+      const unsigned s = (unsigned)sel[j];
+      const char* page = reinterpret_cast<const char*>((uintptr_t)pl.ptbl[s >> pl.shift]);
+      buf[u] = *reinterpret_cast<const cp_u32x4*>(page + (__umul24(s & slot_mask, pl.tok_bytes) + lane_b));
+    }
+  };
+  auto store_rows = [&](const CpPages& pl, const cp_u32x4 (&buf)[CP_R], int j0) {
+    // the chunk lies in one page (CH divides the page size): a wave-uniform base, a per-lane offset
+    const unsigned slot_mask = (1u << pl.shift) - 1u;
+    const unsigned long long pg = pl.ptbl[j0 >> pl.shift];
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)pg);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(pg >> 32));
+    char* base = reinterpret_cast<char*>((uintptr_t)(((unsigned long long)hi << 32) | lo)) +
+                 (unsigned long long)((unsigned)j0 & slot_mask) * pl.tok_bytes;
+    const unsigned dlane = (unsigned)tg * pl.tok_bytes + lane_b;
+#pragma unroll
+    for (int u = 0; u < CP_R; ++u) {
+      char* row = base + (unsigned long long)(unsigned)(u * RPP) * pl.tok_bytes;   // wave-uniform
+      if (j0 + u * RPP + tg < n) *reinterpret_cast<cp_u32x4*>(row + dlane) = buf[u];
+    }
+  };
+
+  cp_u32x4 kb[CP_R], vb[CP_R];
+  for (int j0 = 0; j0 < n; j0 += CH) {
+    load_rows(kp, kb, j0);
+    load_rows(vp, vb, j0);
+    // The loads follow the previous chunk's stores in issue order, so waiting for them waits for those stores as
+    // well; a store is acknowledged long before a load that misses the caches returns, so that costs nothing.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    store_rows(kp, kb, j0);
+    store_rows(vp, vb, j0);
+  }
+}

@@ -125,3 +125,133 @@ __device__ __forceinline__ void tk_select_row(TkShared<THREADS>& sh, KeyAt key_a
     out_pos += __popcll(sb);
   }
 }
+
+// The same selection with the row's keys held in registers: every wavefront owns a contiguous segment of the row and
+// its lane l the keys segment + e * 64 + l, e < KPT, read and converted ONCE (key_at is called once per key), so the
+// digit passes and the ordered pass cost a handful of vector instructions per key instead of an LDS read and a
+// conversion each.  Needs n <= THREADS * KPT.
+// A column's selection is a chain of short steps between workgroup barriers, and inside a kernel whose other
+// workgroups keep the compute unit busy every barrier costs about a microsecond, so the passes are arranged for few
+// of them: one per digit pass (every wavefront scans the 256 bins for itself instead of sharing a scan through LDS;
+// three histograms in rotation, so that clearing the next one needs no barrier of its own) and one before the
+// ordered pass.  The digit passes stop as soon as every key left in the threshold bin is kept (then no tie has to
+// be ranked): rows of distinct scores end after two or three passes.
+// Keys never produced by tk_key (0) stand for "no key here"; they rank below every real key.
+template <int THREADS>
+struct TkSharedRegs {
+  unsigned hist[3][TK_BINS];
+  unsigned w_eq[THREADS / FC_WAVE], w_gt[THREADS / FC_WAVE];
+};
+
+template <int THREADS, int KPT, typename KeyAt, typename Emit>
+__device__ __forceinline__ void tk_select_row_regs(TkSharedRegs<THREADS>& sh, KeyAt key_at, int n, int kk, Emit emit) {
+  constexpr int WAVES = THREADS / FC_WAVE;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int seg = (((n + WAVES - 1) / WAVES) + 63) & ~63;   // <= KPT * 64 by the caller's bound
+  const int beg = wave * seg;
+  const int end = min(n, beg + seg);
+  const int live_e = end > beg ? (end - beg + 63) >> 6 : 0;   // wave-uniform: 64-key groups of this wavefront
+  unsigned key[KPT];
+#pragma unroll
+  for (int e = 0; e < KPT; ++e) {
+    const int i = beg + e * 64 + lane;
+    key[e] = (e < live_e && i < end) ? key_at(i) : 0u;
+  }
+  for (int i = tid; i < 2 * TK_BINS; i += THREADS) (&sh.hist[0][0])[i] = 0;   // histograms of the first two passes
+  __syncthreads();
+  unsigned prefix = 0, mask = 0, remaining = (unsigned)kk;
+  bool whole_bin = false;   // every key that matches the prefix so far is kept
+  int pass = 0;
+  for (int shift = 24; shift >= 0 && !whole_bin; shift -= 8, ++pass) {
+    unsigned* hist = sh.hist[pass % 3];
+    if (pass >= 1)   // the histogram of the pass after this one; its last readers are two barriers back
+      for (int i = tid; i < TK_BINS; i += THREADS) sh.hist[(pass + 1) % 3][i] = 0;
+#pragma unroll
+    for (int e = 0; e < KPT; ++e) {
+      if (e < live_e) {
+        const unsigned u = key[e];
+        if (u != 0u && (u & mask) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
+      }
+    }
+    __syncthreads();
+    // every wavefront for itself: lane t holds bins 255 - 4t .. 252 - 4t (descending), suffix sums over the 256 bins
+    unsigned h4[4], incl = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      h4[r] = hist[TK_BINS - 1 - (4 * lane + r)];
+      incl += h4[r];
+    }
+    const unsigned own = incl;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const unsigned up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    unsigned excl = incl - own;   // keys in bins above this lane's four
+    int found = -1;
+    unsigned left = 0, size = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (found < 0 && excl < remaining && remaining <= excl + h4[r]) {
+        found = TK_BINS - 1 - (4 * lane + r);
+        left = remaining - excl;
+        size = h4[r];
+      }
+      excl += h4[r];
+    }
+    const unsigned long long who = __ballot(found >= 0);   // exactly one lane
+    const int src = __ffsll((long long)who) - 1;
+    const unsigned bin = (unsigned)__shfl(found, src, 64);
+    remaining = __shfl(left, src, 64);
+    whole_bin = __shfl(size, src, 64) == remaining;
+    prefix |= bin << shift;
+    mask |= 255u << shift;
+  }
+  // kept: keys whose masked bits exceed the prefix, and of those that equal it the first `remaining` by index
+  // (all of them when whole_bin; after four passes the masked bits are the whole key)
+  const unsigned T = prefix;
+  const unsigned need = remaining;
+  unsigned eq_cnt = 0, gt_cnt = 0;
+#pragma unroll
+  for (int e = 0; e < KPT; ++e) {
+    if (e < live_e) {
+      const unsigned u = key[e], m = u & mask;
+      eq_cnt += __popcll(__ballot(u != 0u && m == T));
+      gt_cnt += __popcll(__ballot(u != 0u && m > T));
+    }
+  }
+  if (lane == 0) { sh.w_eq[wave] = eq_cnt; sh.w_gt[wave] = gt_cnt; }
+  __syncthreads();
+  unsigned eq_seen = 0, out_pos = 0;
+  {
+    unsigned eq_run = 0;
+    for (int w = 0; w < wave; ++w) {
+      unsigned take = need > eq_run ? min(need - eq_run, sh.w_eq[w]) : 0u;
+      out_pos += sh.w_gt[w] + take;
+      eq_run += sh.w_eq[w];
+    }
+    eq_seen = eq_run;
+  }
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int e = 0; e < KPT; ++e) {
+    if (e < live_e) {
+      const unsigned u = key[e], m = u & mask;
+      const bool is_eq = u != 0u && m == T;
+      const unsigned long long eqb = __ballot(is_eq);
+      const unsigned my_rank = eq_seen + __popcll(eqb & lt_mask);
+      const bool sel = u != 0u && (m > T || (is_eq && my_rank < need));
+      const unsigned long long sb = __ballot(sel);
+      if (sel) emit((int)(out_pos + __popcll(sb & lt_mask)), beg + e * 64 + lane);
+      eq_seen += __popcll(eqb);
+      out_pos += __popcll(sb);
+    }
+  }
+}
+
+// LDS of whichever form of the selection a kernel ends up calling
+template <int THREADS>
+union TkArea {
+  TkShared<THREADS> lds_keys;
+  TkSharedRegs<THREADS> reg_keys;
+};

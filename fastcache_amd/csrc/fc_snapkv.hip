@@ -67,7 +67,7 @@ struct SkPress {
 template <int NW>
 constexpr int sk_press_room() { return SkCfg<NW>::ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4; }
 __host__ __device__ constexpr int sk_press_need(int max_seq_len, int index_stride) {
-  return 4 * max_seq_len + 4 * index_stride + 4 * SK_TBL + 2048;
+  return 4 * max_seq_len + 4 * index_stride + 4 * SK_TBL + 4096 + 16 * CP_PT;   // + the selection's counters, page addresses
 }
 
 template <int DTYPE, int NW, bool FAST, int MODE, bool PRESS = false>
@@ -516,9 +516,9 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     }
   }
   // ---- press: select and compact this column --------------------------------------------------------------
-  // The window positions rank above every scored key (the caller fills them with the layer's largest score afterwards;
-  // here they are +inf), so with more kept positions than window positions the selection equals the one over the
-  // filled row.  The score row is read back from memory (this workgroup wrote it; its stores are waited for) into the
+  // The window positions rank above every scored key (the caller fills them with the layer's largest score
+  // afterwards), so with more kept positions than window positions the selection over the filled row is: the window,
+  // plus the kk - W best of the scored keys; only those enter the selection.  The score row is read back from memory (this workgroup wrote it; its stores are waited for) into the
   // LDS that held the key tiles.
   if constexpr (PRESS) {
     static_assert(MODE == 0 && NW >= 4, "the press tail needs a whole column and at least 256 threads");
@@ -530,8 +530,12 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
     float* sc = reinterpret_cast<float*>(smem);
     int* sel = reinterpret_cast<int*>(smem) + S;
     int* vtbl = sel + press.index_stride;
-    TkShared<THREADS>& sh = *reinterpret_cast<TkShared<THREADS>*>(vtbl + SK_TBL);
-    for (int s = tid; s < S; s += THREADS) sc[s] = s < SW ? out_row[s] : INFINITY;
+    TkArea<THREADS>& sh = *reinterpret_cast<TkArea<THREADS>*>(vtbl + SK_TBL);
+    static_assert(sizeof(TkArea<THREADS>) <= 4096 - 8, "the selection's counters outgrew their share of the LDS budget");
+    // page addresses of the column for the compaction: 8-byte words behind the counters (smem is 16-byte aligned)
+    const int ptbl_word = (S + press.index_stride + SK_TBL + (int)(sizeof(TkArea<THREADS>) / 4) + 1) & ~1;
+    unsigned long long* ptbl = reinterpret_cast<unsigned long long*>(reinterpret_cast<int*>(smem) + ptbl_word);
+    for (int s = tid; s < SW; s += THREADS) sc[s] = out_row[s];
     const KvView& vv = press.vv;
     const int nblk_v = vv.block_shift >= 0 ? ((S - 1) >> vv.block_shift) + 1 : 0;
     const bool v_lds = vv.block_tables && vv.block_shift >= 0 && nblk_v <= SK_TBL;
@@ -539,7 +543,7 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
       for (int i = tid; i < nblk_v; i += THREADS) vtbl[i] = vv.block_tables[(long long)b * vv.table_stride + i];
     __syncthreads();
     int* idx_row = press.indices + (((long long)l * kv.batch + b) * Hkv + h) * (long long)press.index_stride;
-    kp_select_and_move<2, THREADS>(kv, vv, tbl, tbl_lds, vtbl, v_lds, sc, sel, sh, l, b, h, S, kk, idx_row);
+    kp_select_and_move<2, THREADS, true>(kv, vv, tbl, tbl_lds, vtbl, v_lds, sc, sel, sh, ptbl, l, b, h, S, kk, W, idx_row);
   }
 }
 
@@ -704,7 +708,7 @@ static int snapkv_score_impl(const char* who, const fc_kv_view* keys, const void
     const int room = nw == 4 ? sk_press_room<4>() : (nw == 8 ? sk_press_room<8>() : sk_press_room<16>());
     FC_REQUIRE(fast && sk_press_need(keys->max_seq_len, press_index_stride) <= room, FC_EUNSUPPORTED,
                "%s: the one-launch press takes dense views or pages of 64*2^n tokens and 4*(max_seq_len + "
-               "index_stride) + 6144 <= %d bytes (got max_seq_len %d, index_stride %d); use fc_snapkv_score and "
+               "index_stride) + 12288 <= %d bytes (got max_seq_len %d, index_stride %d); use fc_snapkv_score and "
                "fc_select_compact", who, room, keys->max_seq_len, press_index_stride);
     SkPress press;
     press.vv = fc_make_view(values);

@@ -154,7 +154,7 @@ def snapkv_press_fits(keys: FcKvView, num_q_heads: int, window: int, index_strid
     room = tiles * 64 * 256 + (4 * waves + 4) * 64 * 4
     paged_ok = (not keys.block_tables) or (keys.block_size >= 64 and keys.block_size & (keys.block_size - 1) == 0
                                            and (keys.max_seq_len - 1) // keys.block_size < 1024)
-    return bool(paged_ok and 4 * (keys.max_seq_len + index_stride) + 6144 <= room and
+    return bool(paged_ok and 4 * (keys.max_seq_len + index_stride) + 12288 <= room and
                 0 <= keys.stride_token < (1 << 24))
 
 
