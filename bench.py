@@ -719,24 +719,24 @@ WORKLOADS = {"copy": CopyWorkload,
 # HBM-side bytes per launch of a workload's dominant kernel, from two rocprofv3 counter runs
 # (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter reads for the
 # copy workload below, whose traffic is known (512 MiB read, 512 MiB written):
-#   copy:   FETCH_SIZE 2.623e5 KiB -> scale 1.999;  WRITE_SIZE 5.244e5 KiB -> scale 1.000
+#   copy:   FETCH_SIZE 2.623e5 KiB -> scale 1.999;  WRITE_SIZE 5.284e5 KiB -> scale 0.992
 # The commands and raw readings are in profiles/*_hbm_traffic.txt.
 _COUNTER_RUN = {"commit": "76bf753", "date": "2026-11-25"}   # the tree whose kernels the counter runs below measured
-# (cfg5's MLP launch keeps an earlier reading, commit 3ee0b1a: the later counter run of that workload ended in a host-side
-#  crash of the profiled process inside the profiler's dispatch hook, while torch was still building the inputs)
-_COUNTER_RUN_OF = {"cfg5-ccm-hybrid-minicpm-v-2.6": {"commit": "3ee0b1a", "date": "2026-11-25"},
-                   "cfg1-knorm-llama-7b": {"commit": "f22b65d", "date": "2026-11-25"},
-                   "cfg2-snapkv-qwen3-8b": {"commit": "f63ab2e", "date": "2026-11-25"}}
+# (the press launches of cfg1 and cfg2, the calibration and cfg5's MLP launch were counted again at commit cbd5ec4;
+#  cfg5's readings came out as at commit 3ee0b1a)
+_COUNTER_RUN_OF = {"cfg5-ccm-hybrid-minicpm-v-2.6": {"commit": "cbd5ec4", "date": "2026-11-25"},
+                   "cfg1-knorm-llama-7b": {"commit": "cbd5ec4", "date": "2026-11-25"},
+                   "cfg2-snapkv-qwen3-8b": {"commit": "cbd5ec4", "date": "2026-11-25"}}
 _FETCH_SCALE = 524288 / 2.623e5
-_WRITE_SCALE = 524288 / 5.244e5
+_WRITE_SCALE = 524288 / 5.284e5
 _COUNTER_KIB = {  # workload name -> (FETCH_SIZE, WRITE_SIZE) per dispatch of the dominant kernel
-    "cfg1-knorm-llama-7b": (5.246e5, 5.304e5),
+    "cfg1-knorm-llama-7b": (5.247e5, 5.304e5),
     "cfg1-knorm-llama-7b-three-launches": (2.641e5, 5.263e5),
-    "cfg2-snapkv-qwen3-8b": (2.994e6, 1.225e6),                       # the one-launch press: kept rows moved as well
+    "cfg2-snapkv-qwen3-8b": (3.004e6, 1.225e6),                       # the one-launch press: kept rows moved as well
     "cfg2-snapkv-qwen3-8b-two-launches": (2.390e6, 3.636e4),
     "cfg2-snapkv-qwen3-8b+given-lse-two-launches": (1.273e6, 3.636e4),           # one sweep: K is read once
     "cfg3-ccm-linear-decouple-llava-1.5-7b": (1.861e6, 1.845e6),      # mean over the 4 launches of a step
-    "cfg5-ccm-hybrid-minicpm-v-2.6": (3.919e6, 1.468e6),
+    "cfg5-ccm-hybrid-minicpm-v-2.6": (3.921e6, 1.468e6),
     # The decode launches were counted without the graph, 4 steps per bracket (the profiler is not run on the long
     # graphs).  A launch reads every cached token once and the caches grow by a token per step, so the reading
     # is scaled from that run's algorithmic bytes per launch (third entry) to those of the measured graph.
