@@ -14,11 +14,17 @@
 #define KP_U 4          // key rows per lane in flight while scoring
 // 1024 threads per column from this many bytes of key rows per column on, 256 below.  More lanes finish a column sooner
 // (more rows in flight per column, fewer columns half done at any time) but idle through a short column's selection.
-// Measured, 1024 against 256 threads: the Knorm press 0.292 / 0.323 ms (1024 columns x 1024 fp32 rows), 1.166 / 1.313 ms
-// (4096 x 2048 bf16), 0.601 / 0.629 (4096 x 1024 bf16), 1.364 / 1.099 (16384 x 512 bf16), 3.67 / 1.15 (65536 x 128);
-// selection + compaction alone 0.934 / 0.956 (2048 x 4096 bf16), 0.933 / 0.915 (4096 x 2048), 1.123 / 0.881 (16384 x 512).
-#define KP_WIDE_BYTES_PRESS (384 * 1024)
+// The figures behind both constants are in profiles/launch_shape_crossovers.txt (the library built with the
+// constants forced to 0 and to 2e9, `python -m fastcache_amd.crossovers knorm select` on each): the Knorm press with
+// 1024 against 256 threads 1.07 / 1.31 ms (4096 columns x 2048 bf16 rows), 0.555 / 0.608 (4096 x 1024), 1.30 / 1.08
+// (16384 x 512), 3.59 / 1.04 (65536 x 128); selection + compaction alone 0.509 / 0.519 (2304 x 4096), 0.467 / 0.451
+// (4096 x 2048), 0.935 / 0.459 (16384 x 512).
+#ifndef KP_WIDE_BYTES_PRESS
+#define KP_WIDE_BYTES_PRESS (256 * 1024)
+#endif
+#ifndef KP_WIDE_BYTES_SELECT
 #define KP_WIDE_BYTES_SELECT (1024 * 1024)
+#endif
 
 // Which column a workgroup takes.  Workgroups go to the eight XCDs round-robin in launch order; columns that follow each
 // other in memory (the heads of a sequence, whose rows of one token are adjacent) are given to the same XCD, one after

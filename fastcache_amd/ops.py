@@ -64,9 +64,10 @@ def key_channel_zero(keys: FcKvView, prune: torch.Tensor) -> None:
 
 
 def snapkv_splits(keys: FcKvView, num_q_heads: int, window: int) -> int:
-    """Key ranges per column for :func:`snapkv_score`.  Measured on MI355X (window 64, group of 4-7 heads): with
+    """Key ranges per column for :func:`snapkv_score`.  Measured on MI355X (window 64, group of 4-7 heads;
+    ``python -m fastcache_amd.crossovers splits``, figures in profiles/launch_shape_crossovers.txt): with
     1000 or more (layer, sequence, kv head) columns one workgroup per column is fastest; below that the GPU is not
-    filled and cutting the columns pays: 576 columns -19 % with 4 pieces, 288 columns -32 % with 8, 112 columns -40 %.
+    filled and cutting the columns pays: 576 columns -13 % with 4 pieces, 288 columns -26 % with 8, 112 columns -39 %.
     A piece keeps at least 8 key tiles of 64.  1 also when the split kernels do not apply (more than 16 query row
     blocks per kv head, pages that are no multiple of 64 tokens)."""
     columns = keys.num_layers * keys.batch * keys.num_kv_heads
@@ -163,9 +164,10 @@ def snapkv_press_preferred(keys: FcKvView, num_q_heads: int, window: int, comput
     ``select_compact``) is the faster form for a shape both take.  Whole columns cost ``rounds x column time`` with
     ``rounds = ceil(columns / workgroups the GPU holds)`` (two per compute unit, one with 16 wavefronts), split scoring
     grows linearly with the columns but pays a merge, a pooling and a compaction launch.  Measured on MI355X (28 x B x 4
-    and 36 x B x 8 columns of 4096 to 12000 keys): whole columns win or tie when the last round is at least 80 % full
-    or the columns are short (up to 4096 keys: 0.62 against 0.75 ms at 448 columns, 0.93 against 1.04 at 672, at worst
-    2.5 % behind); long columns in poorly filled rounds lose (320 x 12000: 1.67 against 1.40 ms)."""
+    and 36 x B x 8 columns of 4096 to 12000 keys; ``python -m fastcache_amd.crossovers press``, figures in
+    profiles/launch_shape_crossovers.txt): whole columns win or tie when the last round is at least 80 % full
+    or the columns are short (up to 4096 keys: 0.64 against 0.72 ms at 448 columns, 0.92 against 1.01 at 672, at worst
+    2.5 % behind); long columns in poorly filled rounds lose (320 x 12000: 1.64 against 1.37 ms)."""
     if snapkv_splits(keys, num_q_heads, window) == 1:
         return True
     columns = keys.num_layers * keys.batch * keys.num_kv_heads

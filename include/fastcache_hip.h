@@ -19,7 +19,8 @@
  *     saying that its limit has been raised (hipFuncSetAttribute on the first
  *     launch on a device; unsynchronised, setting it twice is harmless); the
  *     compute-unit count of each device; and, for fc_decode_attn_static only,
- *     the device address of its built-in buffer.  The first launch of a kernel
+ *     the device address of its built-in buffer (and, with FC_STATIC_GUARD=1 in the
+ *     environment, the stream of the previous call on each device).  The first launch of a kernel
  *     on a device therefore does host-side work: make it outside a graph
  *     capture;
  *   - return value: FC_OK (0) or a negative FC_E* code; nothing is enqueued
@@ -37,6 +38,14 @@
 extern "C" {
 #endif
 
+/*
+ * Version of the SIGNATURES and STRUCT LAYOUTS below, returned by fc_abi_version().  The policy is additive: a
+ * release may add entry points and error codes without changing the number (a binding looks an optional entry point
+ * up by name and does without it when the look-up fails); the number changes only when an existing entry point's
+ * arguments or meaning, or a struct's layout, change, and a binding that was written for another number must refuse
+ * to run.  Everything added since the first release (the one-launch presses, the ragged MLP, the entry point with a
+ * built-in buffer, the optional FC_STATIC_GUARD check) left the existing signatures as they were: still 1.
+ */
 #define FC_ABI_VERSION 1
 
 enum { FC_F32 = 0, FC_F16 = 1, FC_BF16 = 2 };
@@ -143,8 +152,8 @@ int fc_snapkv_score_lse(const fc_kv_view* keys, const void* queries, const float
  * positions and `row_max` (required) the per-row maxima; the caller runs fc_snapkv_fill_window afterwards if it wants
  * the window entries of `scores` filled.  Rows of sequences no longer than the window keep their first positions.
  * Takes dense views or pages of 64*2^n tokens and sequences short enough for the score row and the kept positions to
- * fit the LDS of the key tiles: 4 * (max_seq_len + index_stride) + 6144 bytes within 54272 (up to four 32-row query
- * blocks per kv head) or 74752 (more), e.g. 13 000 tokens of which a quarter is kept; refused with FC_EUNSUPPORTED
+ * fit the LDS of the key tiles: 4 * (max_seq_len + index_stride) + 12288 bytes within 54272 (up to four 32-row query
+ * blocks per kv head) or 74752 (more), e.g. 12 000 tokens of which a quarter is kept; refused with FC_EUNSUPPORTED
  * otherwise.  A row whose kept count does not exceed the window (n_kept comes from device memory) is left untouched.  Replaces, for SnapKVPress, the per-sequence loop of
  * LlavaModelRunner.compress_kv_cache_batch (nanovllm/engine/llava_model_runner.py:745-786).
  */
@@ -460,6 +469,9 @@ int fc_decode_attn(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t
  * fc_decode_attn_workspace_bytes() exceed the capacity are rejected with FC_EUNSUPPORTED.  All calls on one GPU
  * share the one buffer: calls that overlap on a GPU (different streams, concurrent graphs) race; calls on one
  * stream are ordered and safe.  Nothing in the buffer has to start at zero, so no clearing is done.
+ * With FC_STATIC_GUARD=1 in the environment (read once) the call remembers the stream of the previous call on the
+ * device and returns FC_EINVAL when another stream calls while that one still has work pending (it queries the
+ * previous stream, so leave the variable unset while streams are being captured).
  */
 int64_t fc_decode_attn_static_capacity(void);
 int fc_decode_attn_static(const fc_kv_view* k_cache, const fc_kv_view* v_cache, int32_t layer,

@@ -54,3 +54,51 @@ def test_static_scratch_entry_rejects_oversize(dev):
     rc = _lib.fn("fc_decode_attn_static")(C.byref(views[0]), C.byref(views[1]), 0, q.data_ptr(), q.data_ptr(), Hq,
                                           lens.data_ptr(), 1.0, None)
     assert rc == -2 and b"built-in" in _lib.fn("fc_last_error")()
+
+
+_GUARD_CHILD = r"""
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+from fastcache_amd import _lib, ops
+dev = torch.device("cuda:0")
+pool = torch.randn(2, 1, 8, 256, 2, 128, device=dev).half()
+tab = torch.arange(8, dtype=torch.int32, device=dev).view(2, 4)
+lens = torch.tensor([700, 300], dtype=torch.int32, device=dev)
+views = [_lib.paged_view(pool[i], tab, None, 1024) for i in range(2)]
+q = torch.randn(2, 4, 128, device=dev).half()
+out = torch.empty_like(q)
+side = torch.cuda.Stream()
+ops.decode_attn_static(views[0], views[1], 0, q, lens, 0.088, out)          # first call: nothing to compare with
+torch.cuda.synchronize()
+ref = out.clone()
+torch.cuda._sleep(2_000_000_000)                                            # about a second of pending work on the main stream
+ops.decode_attn_static(views[0], views[1], 0, q, lens, 0.088, out)
+refused = False
+with torch.cuda.stream(side):
+    try:
+        ops.decode_attn_static(views[0], views[1], 0, q, lens, 0.088, out)
+    except _lib.FastcacheError as e:
+        refused = "another stream" in str(e)
+torch.cuda.synchronize()                                                    # the main stream has drained: the side stream may call
+with torch.cuda.stream(side):
+    ops.decode_attn_static(views[0], views[1], 0, q, lens, 0.088, out)
+torch.cuda.synchronize()
+print("REFUSED" if refused else "ACCEPTED", "SAME" if torch.equal(out, ref) else "DIFFERENT")
+"""
+
+
+def test_static_scratch_guard_refuses_an_overlapping_stream(dev, tmp_path):
+    """FC_STATIC_GUARD=1 (read once per process, hence a child process): a call on another stream while the previous
+    call's stream still has work pending is refused before anything is enqueued; once that stream has drained the
+    same call goes through and gives the same bytes.  Without the variable the library does not look."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = tmp_path / "guard_child.py"
+    script.write_text(_GUARD_CHILD)
+    for guard, want in (("1", "REFUSED SAME"), ("", "ACCEPTED SAME")):
+        env = dict(os.environ, FC_STATIC_GUARD=guard)
+        res = subprocess.run([sys.executable, str(script), root], capture_output=True, text=True, env=env, timeout=100)
+        assert res.returncode == 0, res.stderr[-2000:]
+        assert res.stdout.strip().splitlines()[-1] == want, (guard, res.stdout, res.stderr[-500:])
