@@ -195,6 +195,57 @@ def test_snapkv_press_one_launch_equals_separate(dev, dtype, lens, Hq, H, W, ksz
     assert not torch.equal(pool_b.view(torch.uint8), case.kv_cache.to(dev).view(torch.uint8))
 
 
+@pytest.mark.parametrize("period,keep", [(50, [600, 300]), (7, [1100, 300]), (256, [70, 650])])
+def test_snapkv_press_exact_ties_from_periodic_keys(dev, period, keep):
+    """Keys that repeat with a period give bit-identical scores period apart (same logits, same exponentials, same
+    pooled neighbourhoods), so every row is full of exact ties, among them the threshold's: the one-launch press
+    (selection over register-held keys) and the separate launches (the stand-alone top-k kernel) must both keep the
+    lowest positions of a tie, and both must equal the stable selection on the kernel's own scores.  (Kept counts are
+    chosen so that the threshold does not fall into the group of keys that tie with the row's LARGEST score: there the
+    two forms differ by design, the filled window ties with those keys in the separate launches and outranks them in
+    the one launch.)"""
+    dtype, L, H, G, W, ksz, lens = torch.bfloat16, 2, 2, 2, 32, 5, [1500, 700]
+    B, S = len(lens), max(lens)
+    g = torch.Generator().manual_seed(period)
+    base = torch.randn(L, B, H, period, 128, generator=g)
+    reps = -(-S // period)
+    dense_k = base.repeat(1, 1, 1, reps, 1)[:, :, :, :S].to(dtype)
+    dense_v = torch.randn(L, B, H, S, 128, generator=g).to(dtype)
+    q = torch.randn(L, B, H * G, W, 128, generator=g).to(dtype)
+    need = [-(-n // 256) for n in lens]
+    tables = [list(range(sum(need[:b]), sum(need[:b + 1]))) for b in range(B)]
+    pool = torch.zeros(2, L, sum(need), 256, H, 128, dtype=dtype)
+    for l in range(L):
+        synth.scatter_into_pool(pool, 0, l, dense_k[l], tables, lens)
+        synth.scatter_into_pool(pool, 1, l, dense_v[l], tables, lens)
+    pa = pool.to(dev)
+    pb = pa.clone()
+    tt = torch.tensor([t + [-1] * (max(need) - len(t)) for t in tables], dtype=torch.int32, device=dev)
+    ll = torch.tensor(lens, dtype=torch.int32, device=dev)
+    nk = torch.tensor(keep, dtype=torch.int32, device=dev)
+    qd, width = q.to(dev), max(keep)
+    ka, va = (_lib.paged_view(pa[p], tt, ll, S) for p in range(2))
+    sa = ops.snapkv_score(ka, qd, W, ksz, True, "sum", seq_lens=ll, splits=1)
+    ia = ops.topk_select(sa, width, row_lens=ll, n_kept=nk, rows_per_len=H)
+    ops.compact(ka, va, ka, va, ia, n_kept=nk)
+    kb, vb = (_lib.paged_view(pb[p], tt, ll, S) for p in range(2))
+    assert ops.snapkv_press_fits(kb, H * G, W, width)
+    sb, ib = ops.snapkv_press(kb, vb, qd, W, ksz, width, True, "sum", seq_lens=ll, n_kept=keep, host_lens=lens)
+    torch.cuda.synchronize()
+    assert torch.equal(sa.view(torch.int32), sb.view(torch.int32))
+    assert torch.equal(ia, ib)
+    assert torch.equal(pa.view(torch.uint8), pb.view(torch.uint8))
+    for b, n in enumerate(lens):
+        row = sb[:, b, :, :n].cpu()
+        body = row[..., ksz:n - W - ksz - period]                         # away from the zero-padded borders
+        shifted = row[..., ksz + period:n - W - ksz]
+        assert bool((body == shifted).all()), "the scores are not periodic: the test lost its ties"
+        want = opress.topk_lowest_index(row, keep[b])
+        assert torch.equal(ib[:, b, :, :keep[b]].cpu().long(), want)
+        kth = row.gather(-1, want).min(-1).values
+        assert bool(((row == kth[..., None]).sum(-1) > 1).all()), "no tie at the threshold"
+
+
 def test_snapkv_paged_press_tiny_scored_part_takes_separate_launches(dev):
     """Six scored keys under a pooling kernel of 13: every pooled score is the same and equals the layer's largest, so
     after the window fill all 38 positions tie and the lowest indices win (position 37, a window position, is the one
