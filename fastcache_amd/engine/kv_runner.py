@@ -29,16 +29,33 @@ class PagedKVRunner:
     def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int, num_blocks: int, dtype: torch.dtype,
                  device, block_size: int = 256, compressor=None, batched_compressor=None, image_token_len: int = 576,
                  block_manager=None):
-        self.num_hidden_layers, self.num_key_value_heads, self.head_dim = num_layers, num_kv_heads, head_dim
-        self.block_size = block_size
-        self.device = torch.device(device)
-        self.kv_cache = torch.zeros(2, num_layers, num_blocks, block_size, num_kv_heads, head_dim, dtype=dtype,
-                                    device=self.device)
+        pool = torch.zeros(2, num_layers, num_blocks, block_size, num_kv_heads, head_dim, dtype=dtype,
+                           device=torch.device(device))
+        self._setup(pool, compressor, batched_compressor, image_token_len, block_manager, None)
+
+    @classmethod
+    def adopt(cls, kv_cache: torch.Tensor, compressor=None, batched_compressor=None, image_token_len: int = 576,
+              block_manager=None, compressed_lens: Optional[Dict[int, int]] = None) -> "PagedKVRunner":
+        """A runner over a pool that already exists (``kv_cache [2, L, blocks, block_size, Hkv, D]``, e.g. the one
+        ``LlavaModelRunner.allocate_kv_cache`` made, llava_model_runner.py:526-529) instead of one of its own;
+        ``compressed_lens`` lets the host runner and this one share the ``_compressed_lens`` dictionary."""
+        if kv_cache.dim() != 6 or kv_cache.shape[0] != 2:
+            raise _lib.FastcacheError("kv_cache must be [2, L, num_blocks, block_size, Hkv, D]")
+        self = cls.__new__(cls)
+        self._setup(kv_cache, compressor, batched_compressor, image_token_len, block_manager, compressed_lens)
+        return self
+
+    def _setup(self, kv_cache, compressor, batched_compressor, image_token_len, block_manager, compressed_lens):
+        _, L, _, bs, H, D = kv_cache.shape
+        self.num_hidden_layers, self.num_key_value_heads, self.head_dim = L, H, D
+        self.block_size = bs
+        self.device = kv_cache.device
+        self.kv_cache = kv_cache
         self.compressor = compressor
         self.batched_compressor = batched_compressor
         self.use_batched_compressor = batched_compressor is not None
         self.image_token_len = image_token_len
-        self._compressed_lens: Dict[int, int] = {}
+        self._compressed_lens: Dict[int, int] = {} if compressed_lens is None else compressed_lens
         self._blocks_to_free: Dict[int, List[int]] = {}
         self._lock = threading.Lock()
         self._compress_stream: Optional[torch.cuda.Stream] = None
