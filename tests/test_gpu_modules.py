@@ -504,7 +504,7 @@ def test_lazy_compression_engine_on_the_pool(dev):
     assert len(bm.free_block_ids) == 9 and not bm.used_block_ids and llm.total_freed_blocks == 6
 
 
-@pytest.mark.parametrize("backend", ["mlp", "kvpress"])
+@pytest.mark.parametrize("backend", ["mlp", "kvpress", "knorm-press", "snapkv-press"])
 def test_decode_overlap_compression_splices_generated_rows(dev, backend):
     """A few layers per decode step on a side stream; at the end the pages hold compress(prefill rows) followed by
     the rows generated meanwhile, and the untouched pages served the steps in between."""
@@ -518,9 +518,18 @@ def test_decode_overlap_compression_splices_generated_rows(dev, backend):
         comp = KVCacheLinearDecoupleCompressor(llava_cfg(L, H), compression_factor=2).to(dev).to(dtype).eval()
         sd = {k: v.detach().cpu().float() for k, v in comp.state_dict().items()}
         oracle = lambda hf, n: occm.linear_decouple_forward(hf, [img, max(1, n - img)], sd, 2, 1)
-    else:
+    elif backend == "kvpress":
         comp = KVPressCompressor("knorm", 0.5)
         oracle = lambda hf, n: [opress.adapter_compress_layer("knorm", k, v, 0.5) for k, v in hf]
+    elif backend == "knorm-press":
+        comp = KnormPress(0.5)
+        oracle = lambda hf, n: opipe.knorm_press_compressor(0.5)(hf, 0, n)
+    else:
+        # the press object with its window queries named by sequence: the two length groups (600, 600 | 520) and the
+        # layer chunks of every step find their own slices again
+        from fastcache_amd.presses import SnapKVPress
+        comp = SnapKVPress(0.5, window_size=16, kernel_size=5)
+        wq = torch.randn(L, 3, 2 * H, 16, 128, generator=torch.Generator().manual_seed(5)).to(dtype)
     runner = PagedKVRunner(L, H, 128, num_blocks=16, dtype=dtype, device=dev, image_token_len=img, compressor=comp)
     bm = BlockManager(16, 256)
     seqs = [Sequence(list(range(1000 * i, 1000 * i + n))) for i, n in enumerate(lens)]
@@ -528,6 +537,10 @@ def test_decode_overlap_compression_splices_generated_rows(dev, backend):
         bm.allocate(s)
     _fill_pool_from_case(runner, case, seqs)
     before = runner.kv_cache.cpu()
+    if backend == "snapkv-press":
+        comp.set_window_queries(wq.to(dev), seq_ids=[s.seq_id for s in seqs])
+        index_of = {s.seq_id: i for i, s in enumerate(seqs)}
+        oracle = lambda hf, n, _s=None: None      # replaced per sequence below
 
     ov = DecodeOverlapCompressor(runner, layers_per_step=2)
     ov.start_decode_overlap_compression(seqs)
@@ -557,7 +570,14 @@ def test_decode_overlap_compression_splices_generated_rows(dev, backend):
     torch.cuda.synchronize()
     for s, n in zip(seqs, lens):
         hf = opaged.extract_kv(before, s.block_table, n)
-        ref = oracle(hf, n)
+        if backend == "snapkv-press":
+            i = index_of[s.seq_id]
+            ref = opipe.snapkv_press_compressor(wq[:, i:i + 1], 0.5, 16, 5)(hf, 0, n)
+            ties = any(bool(opress.near_tie_rows(opress.snapkv_score(wq[l, i:i + 1], k, 16, 5)[..., :n - 16],
+                                                 n // 2 - 16).any()) for l, (k, _) in enumerate(hf))
+            assert not ties, "a score within 1e-5 of a threshold: pick another seed"
+        else:
+            ref = oracle(hf, n)
         C = ref[0][0].shape[2]
         assert runner._compressed_lens[s.seq_id] == C + 3 and not ov.pending(s.seq_id)
         got = opaged.extract_kv(runner.kv_cache.cpu(), s.block_table, C + 3)
@@ -569,6 +589,8 @@ def test_decode_overlap_compression_splices_generated_rows(dev, backend):
                     assert torch.equal(got[layer][p][:, :, :C], ref[layer][p])
                 tail = torch.stack([r[p, layer] for r in appended[s.seq_id]], dim=1).unsqueeze(0)   # [1, H, 3, D]
                 assert torch.equal(got[layer][p][:, :, C:], tail)
+    if backend == "snapkv-press":
+        assert not comp._paged_inputs                                   # every slice was used up by the last layer chunk
     freed = free_compressed_blocks(bm, runner, seqs)
     assert freed == sum(-(-(n + 3) // 256) - (-(-(runner_len) // 256)) for n, runner_len in
                         zip(lens, [s.kv_cache_len for s in seqs]))

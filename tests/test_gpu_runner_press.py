@@ -292,3 +292,35 @@ def test_shared_prefix_pages_survive_the_compression_of_one_owner(dev):
     with pytest.raises(_lib.FastcacheError, match="needs the window queries"):
         runner._compress_enqueue([d], 0)
     assert not runner._launch_started
+
+
+def test_snapkv_press_object_with_the_prefill_log_sum_exp(dev):
+    """``set_window_queries(..., lse=)``: with the window queries' log-sum-exp from the prefill's attention kernel the
+    press reads the keys once (single-sweep scoring, then selection + compaction); same kept rows as without it."""
+    dtype, L, B, Hq, Hkv, S, ratio = torch.float16, 2, 2, 4, 2, 700, 0.5
+    case = synth.make_paged_case(seed=19, num_layers=L, batch=B, num_kv_heads=Hkv, seq_lens=[S] * B, dtype=dtype,
+                                 shuffle_tables=False, extra_blocks=0, keep_dense=True)
+    q = torch.randn(L, B, Hq, W, 128, generator=torch.Generator().manual_seed(2)).to(dtype)
+    G = Hq // Hkv
+    mask = torch.triu(torch.full((W, S), float("-inf")), diagonal=S - W + 1)
+    lse = torch.empty(L, B, Hq, W)
+    for l in range(L):
+        k = case.dense_k[l].float().repeat_interleave(G, dim=1)                              # [B, Hq, S, D]
+        lse[l] = torch.logsumexp(torch.matmul(q[l].float(), k.transpose(2, 3)) * 128 ** -0.5 + mask, dim=-1)
+    pools = []
+    for given in (False, True):
+        press = SnapKVPress(ratio, window_size=W, kernel_size=KSZ)
+        runner, bm, seqs = _runner_with_case(dev, case, [S] * B, dtype, press, L, Hkv)
+        press.set_window_queries(q.to(dev), lse=lse.to(dev) if given else None)
+        runner.compress_kv_cache_batch(seqs)
+        assert [runner._compressed_lens[s.seq_id] for s in seqs] == [350, 350] and not press._paged_inputs
+        pools.append((runner.kv_cache.cpu(), [list(s.block_table) for s in seqs]))
+    tie = False
+    for l in range(L):
+        sc = opress.snapkv_score(q[l], case.dense_k[l], W, KSZ)
+        tie |= bool(opress.near_tie_rows(sc[..., :S - W], 350 - W).any())
+    assert not tie, "a score within 1e-5 of a threshold: pick another seed"
+    for b in range(B):
+        for (ak, av), (bk, bv) in zip(opaged.extract_kv(pools[0][0], pools[0][1][b], 350),
+                                      opaged.extract_kv(pools[1][0], pools[1][1][b], 350)):
+            assert torch.equal(ak, bk) and torch.equal(av, bv)

@@ -161,6 +161,20 @@ def test_synthetic_pool_scatter_is_the_page_formula():
     assert sorted(sum(case.block_tables, [])) != sum(case.block_tables, [])       # the tables really are shuffled
 
 
+def test_runner_adopts_an_existing_pool():
+    """``PagedKVRunner.adopt``: a runner over the host runner's own pool tensor and ``_compressed_lens`` dictionary."""
+    pool = torch.zeros(2, 3, 5, 256, 4, 128, dtype=torch.float16)
+    lens = {}
+    r = PagedKVRunner.adopt(pool, compressor=KVPressCompressor("knorm", 0.5), image_token_len=0, compressed_lens=lens)
+    assert r.kv_cache is pool and r._compressed_lens is lens
+    assert (r.num_hidden_layers, r.num_key_value_heads, r.head_dim, r.block_size) == (3, 4, 128, 256)
+    assert r.block_manager is None and not r._launch_started and r.get_compressed_block_count(7) == -1
+    lens[7] = 300
+    assert r.get_compressed_block_count(7) == 2
+    with pytest.raises(Exception, match="kv_cache must be"):
+        PagedKVRunner.adopt(pool[0])
+
+
 def test_sequence_state():
     s = Sequence([1, 2, 3])
     assert not s.is_compressed and s.kv_cache_len == 3 and s.kv_num_blocks == 1
