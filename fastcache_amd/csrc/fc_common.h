@@ -146,6 +146,26 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 // C[32][32] += A[32][16] * B[16][32] in fp32 (v_mfma_f32_32x32x16).  Operands: lane (row or column l % 32,
 // half l / 32) holds the 8 consecutive k = half * 8 .. half * 8 + 7 as 16 bytes.  Result: the lane holds column
 // l % 32 and, in register i, row (i / 4) * 8 + half * 4 + i % 4.
+#ifdef FC_ABLATE_MFMA16
+// Timing-only ablation (results are wrong): the multiply-accumulates of one v_mfma_f32_32x32x16 as two
+// v_mfma_f32_16x16x32 on the same operand registers; which two quarters of the accumulator they write alternates with
+// the k-step, so that every accumulator register stays the result of matrix instructions.
+typedef float fc_f32x4 __attribute__((ext_vector_type(4)));
+template <int DTYPE>
+__device__ __forceinline__ f32x16 fc_mfma(const uint4& a, const uint4& b, f32x16 c, int ks) {
+  const int o = (ks & 1) * 8;
+  fc_f32x4 q0 = {c[o], c[o + 1], c[o + 2], c[o + 3]}, q1 = {c[o + 4], c[o + 5], c[o + 6], c[o + 7]};
+  q0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), q0, 0, 0, 0);
+  q1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, b), __builtin_bit_cast(bf16x8, a), q1, 0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    c[o + i] = q0[i];
+    c[o + 4 + i] = q1[i];
+  }
+  return c;
+}
+#endif
+
 template <int DTYPE>
 __device__ __forceinline__ f32x16 fc_mfma(const uint4& a, const uint4& b, f32x16 c) {
   if constexpr (DTYPE == FC_BF16)

@@ -245,7 +245,11 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       const uint4 kf = fc_lds_read128(a0 ^ (unsigned)(ks * 32));
+      #ifdef FC_ABLATE_MFMA16
+      acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc, ks) : fc_mfma<DTYPE>(qf[ks], kf, acc, ks);
+#else
       acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc) : fc_mfma<DTYPE>(qf[ks], kf, acc);
+#endif
     }
   };
   // The same for the loops that walk whole tiles: the eight fragment addresses of a tile's first block are
@@ -262,7 +266,11 @@ __global__ __launch_bounds__(NW * 64, (NW <= 8 ? 4 : 2)) void snapkv_kernel(
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       const uint4 kf = fc_lds_read128(adr[ks] + (unsigned)(cb * 8192));
+      #ifdef FC_ABLATE_MFMA16
+      acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc, ks) : fc_mfma<DTYPE>(qf[ks], kf, acc, ks);
+#else
       acc = keys_rows ? fc_mfma<DTYPE>(kf, qf[ks], acc) : fc_mfma<DTYPE>(qf[ks], kf, acc);
+#endif
     }
   };
   // ask the scheduler to spread the VALU work of one block between the MFMAs of the next
