@@ -43,7 +43,10 @@ template <int NW>
 struct SkCfg {
   static constexpr int ST = NW >= 8 ? 4 : 3;   // key tiles resident or in flight per workgroup
   // + 256: the key tiles start on a 256-byte LDS address (see the operand reads)
-  static constexpr int LDS = ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4 + SK_TBL * 4 + 256;
+#ifndef SK_LDS_PAD
+#define SK_LDS_PAD 0   // experiments: extra LDS per workgroup, to hold the number of workgroups per compute unit down
+#endif
+  static constexpr int LDS = ST * SK_TILEB + (4 * NW + 4) * SK_KT * 4 + SK_TBL * 4 + 256 + SK_LDS_PAD;
 };
 
 // MODE 0: the whole kernel for one (layer, sequence, kv head) column.
