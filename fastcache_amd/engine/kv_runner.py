@@ -172,14 +172,18 @@ class PagedKVRunner:
                     mine.append(i)
             plan.append((s, mine))
         need = sum(len(p) for _, p in plan)
-        if need == 0:
-            return 0
         if need > len(bm.free_block_ids):
             raise _lib.FastcacheError(f"the batch would rewrite {need} pages it shares with other sequences and only "
                                       f"{len(bm.free_block_ids)} pages are free to copy them to")
         moved = []
         for s, positions in plan:
             moved += bm.unshare(s, positions)
+        # From the first launch on, the pages about to be rewritten no longer hold the tokens they were published
+        # under.  Their content keys leave the prefix cache now, not when the engine later shortens the tables: with
+        # the compression on a side stream, a prefill of the same prompt can be scheduled in between.
+        if hasattr(bm, "forget_pages"):
+            for s, w in zip(seqs, writes):
+                bm.forget_pages([b for b in s.block_table[:w] if b >= 0])
         if moved:
             old = [[a] for a, _ in moved]
             new = [[b] for _, b in moved]

@@ -294,6 +294,32 @@ def test_shared_prefix_pages_survive_the_compression_of_one_owner(dev):
     assert not runner._launch_started
 
 
+def test_rewritten_pages_leave_the_prefix_cache_when_the_compression_starts(dev):
+    """With the compression on the side stream the engine shortens the tables only in front of the sequence's next
+    decode step; a prefill of the same prompt scheduled in between must not be handed the pages being rewritten."""
+    dtype, L, H, nb = torch.float16, 2, 2, 12
+    bm = BlockManager(nb, 256)
+    runner = PagedKVRunner(L, H, 128, num_blocks=nb, dtype=dtype, device=dev, image_token_len=0,
+                           compressor=KVPressCompressor("knorm", 0.5), block_manager=bm)
+    a = Sequence(list(range(600)))
+    bm.allocate(a)
+    runner.kv_cache.copy_(torch.randn(runner.kv_cache.shape, generator=torch.Generator().manual_seed(8)).to(dtype))
+    start = runner.kv_cache.cpu()
+    tab_a = list(a.block_table)
+    done = runner.start_background_compression([a])          # 300 rows kept: pages 0 and 1 are rewritten, page 2 is not
+    twin = Sequence(list(range(600)))
+    bm.allocate(twin)
+    assert twin.num_cached_tokens == 0 and not set(twin.block_table) & set(a.block_table)
+    assert all(bm.blocks[p].hash == -1 for p in tab_a[:2])
+    runner.wait_compression(done)
+    ref_pool = start.clone()
+    oracle_comp = lambda hf, i, n: [opress.adapter_compress_layer("knorm", k, v, 0.5) for k, v in hf]
+    opipe.compress_batch(ref_pool, [tab_a], [600], oracle_comp)
+    for (gk, gv), (rk, rv) in zip(opaged.extract_kv(runner.kv_cache.cpu(), tab_a, 300),
+                                  opaged.extract_kv(ref_pool, tab_a, 300)):
+        assert torch.equal(gk, rk) and torch.equal(gv, rv)
+
+
 def test_snapkv_press_object_with_the_prefill_log_sum_exp(dev):
     """``set_window_queries(..., lse=)``: with the window queries' log-sum-exp from the prefill's attention kernel the
     press reads the keys once (single-sweep scoring, then selection + compaction); same kept rows as without it."""
