@@ -614,11 +614,13 @@ class CopyWorkload(Workload):
     write-only streams (torch's fill kernel, the runtime's memset).  Each moves 512 MiB per tensor."""
     name = "copy-calibration-1GiB"
     dtype_name = "bf16"
-    kernel_name = "compact_kernel"
+    kernel_name = "copy_rows_kernel"
     metric = "tokens copied/sec"
     unit = "tokens/s"
     KINDS = {  # kind -> (workload name, kernel name as a trace shows it, tensors read, tensors written)
-        "compact": ("copy-calibration-1GiB", "compact_kernel", 1, 1),
+        "compact": ("copy-calibration-1GiB", "copy_rows_kernel", 1, 1),
+        # the same bytes between two sets of pages of ONE pool: the views may overlap, so the rows move in order
+        "compact-ordered": ("copy-ordered-walk-1GiB", "compact_kernel", 1, 1),
         "torch-copy": ("copy-torch-copy_-1GiB", "hipMemcpyAsync device to device (torch Tensor.copy_)", 1, 1),
         "hip-memcpy": ("copy-hipMemcpyDtoDAsync-1GiB", "hipMemcpyDtoDAsync", 1, 1),
         "torch-kernel": ("copy-torch-elementwise-1GiB", "torch elementwise kernel (torch.neg, out=)", 1, 1),
@@ -635,8 +637,15 @@ class CopyWorkload(Workload):
         # 16 * 16 * 8 * 1024 rows of 256 B = 512 MiB per tensor, as 2048 (layer, sequence, head) columns: this library's
         # kernels take a workgroup per column, so a tensor of a few very long columns would measure the grid, not the memory
         L, B, H, S = 16, 16, 8, 1024
-        self.src = torch.randn((L, B, H, S, D), device=device, dtype=torch.float32).to(torch.bfloat16)
-        self.dst = torch.empty_like(self.src)
+        if kind == "compact-ordered":
+            pages = S // 256
+            self.pool = torch.randn((L, 2 * B * pages, 256, H, D), device=device, dtype=torch.float32).to(torch.bfloat16)
+            t = torch.arange(B * pages, dtype=torch.int32, device=device).view(B, pages)
+            self.tables = (t, t + B * pages)
+            self.src = self.pool[:, :B * pages]
+        else:
+            self.src = torch.randn((L, B, H, S, D), device=device, dtype=torch.float32).to(torch.bfloat16)
+            self.dst = torch.empty_like(self.src)
         self.S = S
         self.tokens_per_step = B * S
         self.nbytes = self.src.numel() * 2
@@ -659,6 +668,9 @@ class CopyWorkload(Workload):
         with self.br:
             if self.kind == "compact":
                 ops.copy_tokens(_lib.dense_view(self.src), _lib.dense_view(self.dst), 0, self.S, 0)
+            elif self.kind == "compact-ordered":
+                ops.copy_tokens(_lib.paged_view(self.pool, self.tables[0], None, self.S),
+                                _lib.paged_view(self.pool, self.tables[1], None, self.S), 0, self.S, 0)
             elif self.kind == "torch-copy":
                 self.dst.copy_(self.src)
             elif self.kind == "hip-memcpy":
@@ -695,7 +707,7 @@ def _separate(w, three):
     return w
 
 
-CEILINGS = ("compact", "torch-copy", "hip-memcpy", "torch-kernel", "read", "torch-read", "torch-fill", "hip-memset")
+CEILINGS = ("compact", "compact-ordered", "torch-copy", "hip-memcpy", "torch-kernel", "read", "torch-read", "torch-fill", "hip-memset")
 
 WORKLOADS = {"copy": CopyWorkload,
              **{f"stream-{k}": (lambda seed, dev, k=k: CopyWorkload(seed, dev, kind=k)) for k in CEILINGS},

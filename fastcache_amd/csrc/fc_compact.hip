@@ -71,6 +71,99 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
                               [&](int j) { return GATHER ? idx[j] : src_start + j; });
 }
 
+// Copies and gathers between buffers that cannot overlap need no order among their rows, and a copy is fastest on
+// this part as many short-lived workgroups that each load a few rows and store them: a workgroup moves CR_V passes of
+// 256 / LPR token rows of one head of one plane and ends (no loop, no barrier, no table in LDS).  Such a workgroup
+// lives a few microseconds, so what it computes before its first load counts: one plane per launch (no choice between
+// views), blockIdx.x / blockIdx.y = head and chunk of rows in the order the host picked (heads_fast: consecutive
+// workgroups take consecutive heads of the same tokens, for a destination that keeps a token's heads together;
+// otherwise consecutive chunks of one head), blockIdx.z = layer * sequences + sequence (the layer is the slowest index
+// of every layout this library meets), split with a multiplier the host precomputed (exact for every z below 2^16).  GATHER: source token = indices[j].
+#ifndef CR_V
+#define CR_V 1
+#endif
+template <int EB, bool GATHER>
+__global__ __launch_bounds__(CP_THREADS) void copy_rows_kernel(KvView src, KvView dst, const int* __restrict__ indices,
+                                                               int index_stride, int heads_in_index, int k,
+                                                               const int* __restrict__ n_kept, int src_start,
+                                                               int dst_start, const char* const* __restrict__ src_layers,
+                                                               int heads_fast, unsigned long long inv_batch) {
+  constexpr int LPR = FC_HEAD_DIM * EB / 16, RPP = CP_THREADS / LPR;
+  const int h = heads_fast ? blockIdx.x : blockIdx.y;
+  const int chunk = heads_fast ? blockIdx.y : blockIdx.x;
+  const int l = (int)((blockIdx.z * inv_batch) >> 32);
+  const int b = (int)blockIdx.z - l * src.batch;
+  const int S = fc_seq_len(src, b);
+  // a count read from device memory is never trusted beyond what the host validated
+  int n = n_kept ? n_kept[b] : k;
+  n = GATHER ? min(n, index_stride) : min(n, S - src_start);
+  n = min(n, dst.max_seq_len - dst_start);
+  const int tid = threadIdx.x, sub = tid % LPR, tg = tid / LPR;
+  const int j0 = chunk * (RPP * CR_V);
+  if (j0 >= n) return;
+  const int* idx = GATHER ? indices + (((long long)l * src.batch + b) * heads_in_index + (h % heads_in_index)) *
+                                          (long long)index_stride
+                          : nullptr;
+  const char* slayer = src_layers ? src_layers[l] : src.base + (long long)l * src.stride_layer * EB;
+  const char* sbase = slayer + (long long)h * src.stride_head * EB + sub * 16;
+  char* dbase = dst.base + ((long long)l * dst.stride_layer + (long long)h * dst.stride_head) * EB + sub * 16;
+  const char* safe = slayer + sub * 16;      // the first 16-byte pieces of the layer: readable whatever the view
+  cp_u32x4 buf[CR_V];
+  long long doff[CR_V];
+  // every lane always loads (rows that do not exist read `safe`), so that all CR_V loads are in flight together
+#pragma unroll
+  for (int u = 0; u < CR_V; ++u) {
+    const int j = j0 + u * RPP + tg;
+    long long so = -1;
+    doff[u] = -1;
+    if (j < n) {
+      const int st = GATHER ? idx[j] : src_start + j;
+      if (st >= 0 && st < S) so = fc_token_offset(src, b, st);
+    }
+    if (so >= 0) doff[u] = fc_token_offset(dst, b, dst_start + j);
+    buf[u] = *reinterpret_cast<const cp_u32x4*>(doff[u] >= 0 ? sbase + so * EB : safe);
+  }
+#pragma unroll
+  for (int u = 0; u < CR_V; ++u)
+    if (doff[u] >= 0) *reinterpret_cast<cp_u32x4*>(dbase + doff[u] * EB) = buf[u];
+}
+
+// Whether the bytes two views can reach cannot overlap: a pool and a dense tensor never do (different tensors by
+// construction of the callers), two dense tensors do not when the byte ranges they span are disjoint.  Two views of
+// one pool are never taken as apart.
+static bool cp_views_apart(const fc_kv_view* a, const fc_kv_view* b) {
+  if ((a->block_tables == nullptr) != (b->block_tables == nullptr)) return true;
+  if (a->block_tables) return false;
+  const auto span = [](const fc_kv_view* v, const char*& lo, const char*& hi) {
+    const int eb = v->dtype == FC_F32 ? 4 : 2;
+    const long long last = (long long)(v->num_layers - 1) * v->stride_layer + (long long)(v->batch - 1) * v->stride_batch +
+                           (long long)(v->num_kv_heads - 1) * v->stride_head +
+                           (long long)(v->max_seq_len - 1) * v->stride_token + FC_HEAD_DIM;
+    lo = (const char*)v->base;
+    hi = lo + last * eb;
+  };
+  const char *alo, *ahi, *blo, *bhi;
+  span(a, alo, ahi);
+  span(b, blo, bhi);
+  return ahi <= blo || bhi <= alo;
+}
+
+#ifndef CR_ONESHOT
+#define CR_ONESHOT 1
+#endif
+// grid of the one-shot kernel for `rows` rows per column of one plane; false when the shape does not fit one launch
+static bool cp_oneshot_grid(const fc_kv_view* v, int rows, bool heads_fast, dim3& grid, unsigned long long& inv_batch) {
+  const int eb = v->dtype == FC_F32 ? 4 : 2;
+  const int per_wg = (CP_THREADS / (FC_HEAD_DIM * eb / 16)) * CR_V;
+  const long long chunks = ((long long)rows + per_wg - 1) / per_wg;
+  const long long z = (long long)v->batch * v->num_layers;
+  const long long x = heads_fast ? v->num_kv_heads : chunks, y = heads_fast ? chunks : v->num_kv_heads;
+  if (x > 0x7fffffffLL || y > 65535 || z > 65535 || chunks < 1) return false;
+  grid = dim3((unsigned)x, (unsigned)y, (unsigned)z);
+  inv_batch = (0x100000000ULL + (unsigned)v->batch - 1) / (unsigned)v->batch;   // ceil(2^32 / sequences)
+  return true;
+}
+
 static int check_pair(const fc_kv_view* a, const fc_kv_view* b, const char* who) {
   FC_REQUIRE(a->dtype == b->dtype && a->num_layers == b->num_layers && a->batch == b->batch &&
                  a->num_kv_heads == b->num_kv_heads,
@@ -100,6 +193,26 @@ extern "C" int fc_compact(const fc_kv_view* src_k, const fc_kv_view* src_v, cons
   if (!n_kept && k == 0) return FC_OK;
   KvView sk = fc_make_view(src_k), sv = fc_make_view(src_v), dk = fc_make_view(dst_k), dv = fc_make_view(dst_v);
   hipStream_t st = (hipStream_t)stream;
+  {  // no destination can overlap a source: rows in any order, short-lived workgroups, one launch per plane
+    dim3 grid;
+    unsigned long long inv;
+    const bool heads_fast = dk.stride_head < dk.stride_token;
+    if (CR_ONESHOT && cp_views_apart(src_k, dst_k) && cp_views_apart(src_k, dst_v) && cp_views_apart(src_v, dst_k) &&
+        cp_views_apart(src_v, dst_v) && cp_oneshot_grid(src_k, n_kept ? index_stride : k, heads_fast, grid, inv)) {
+      for (int plane = 0; plane < 2; ++plane) {
+        const KvView& s1 = plane ? sv : sk;
+        const KvView& d1 = plane ? dv : dk;
+        if (src_k->dtype == FC_F32)
+          hipLaunchKernelGGL((copy_rows_kernel<4, true>), grid, dim3(CP_THREADS), 0, st, s1, d1, indices, index_stride,
+                             heads_in_index, k, n_kept, 0, 0, nullptr, (int)heads_fast, inv);
+        else
+          hipLaunchKernelGGL((copy_rows_kernel<2, true>), grid, dim3(CP_THREADS), 0, st, s1, d1, indices, index_stride,
+                             heads_in_index, k, n_kept, 0, 0, nullptr, (int)heads_fast, inv);
+        FC_CHECK_LAUNCH(who);
+      }
+      return FC_OK;
+    }
+  }
   // 512-byte (fp32) rows: two heads per workgroup measured faster, as long as the grid stays large
   const long long cols = 2LL * src_k->num_layers * src_k->batch * src_k->num_kv_heads;
   if (src_k->dtype == FC_F32 && src_k->num_kv_heads % 2 == 0 && cols >= 2048) {
@@ -134,7 +247,24 @@ static int copy_tokens_impl(const char* who, const void* const* src_layers, cons
   // and a long column can be cut into pieces: enough of them for about eight workgroups per compute unit, none
   // shorter than 512 rows.
   int rows_per_piece = 0, pieces = 1;
-  if (src_layers || (src->block_tables == nullptr) != (dst->block_tables == nullptr)) {
+  const bool apart = src_layers || cp_views_apart(src, dst);
+  hipStream_t st = (hipStream_t)stream;
+  {
+    dim3 grid;
+    unsigned long long inv;
+    const bool heads_fast = d.stride_head < d.stride_token;
+    if (CR_ONESHOT && apart && cp_oneshot_grid(src, count, heads_fast, grid, inv)) {
+      if (src->dtype == FC_F32)
+        hipLaunchKernelGGL((copy_rows_kernel<4, false>), grid, dim3(CP_THREADS), 0, st, s, d, nullptr, 0, 1, count, nullptr,
+                           seg_start, dst_start, (const char* const*)src_layers, (int)heads_fast, inv);
+      else
+        hipLaunchKernelGGL((copy_rows_kernel<2, false>), grid, dim3(CP_THREADS), 0, st, s, d, nullptr, 0, 1, count, nullptr,
+                           seg_start, dst_start, (const char* const*)src_layers, (int)heads_fast, inv);
+      FC_CHECK_LAUNCH(who);
+      return FC_OK;
+    }
+  }
+  if (apart) {
     const long long cols = (long long)src->num_kv_heads * src->batch * src->num_layers;
     const long long want = (2048 + cols - 1) / cols;
     pieces = (int)(want < 1 ? 1 : (want > (count + 511) / 512 ? (count + 511) / 512 : want));
@@ -145,7 +275,6 @@ static int copy_tokens_impl(const char* who, const void* const* src_layers, cons
   }
   // one plane per launch: z covers the layers only
   dim3 grid(src->num_kv_heads * pieces, src->batch, src->num_layers);
-  hipStream_t st = (hipStream_t)stream;
   if (src->dtype == FC_F32)
     hipLaunchKernelGGL((compact_kernel<4, false, 1>), grid, dim3(CP_THREADS), 0, st, s, s, d, d, nullptr, 0, 1, count,
                        nullptr, seg_start, dst_start, (const char* const*)src_layers, rows_per_piece);

@@ -173,3 +173,86 @@ def test_compact_rejects_bad_arguments(dev):
         ops.compact(view, view, view, view, torch.zeros(1, 1, 2, 4, dtype=torch.int64, device=dev))       # not int32
     with pytest.raises(_lib.FastcacheError):
         ops.compact(view, view, view, view, torch.zeros(2, 1, 2, 4, dtype=torch.int32, device=dev))       # layer mismatch
+
+
+def _copy_reference(src_rows, src_ok, dst_old, dst_ok, lens, seg_start, count, dst_start):
+    """Row j of sequence b goes from token seg_start + j to token dst_start + j when j < min(count, len - seg_start),
+    the source token's page exists and the destination token's page exists; everything else keeps its bytes.
+    src_rows / dst_old [L, B, H, S, D]; src_ok / dst_ok [B, S] bool."""
+    out = dst_old.clone()
+    for b, n in enumerate(lens):
+        for j in range(max(0, min(count, n - seg_start, out.shape[3] - dst_start))):
+            if src_ok[b, seg_start + j] and dst_ok[b, dst_start + j]:
+                out[:, b, :, dst_start + j] = src_rows[:, b, :, seg_start + j]
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("block_size", [256, 16, 48])
+def test_copy_between_a_pool_and_dense_tensors(dev, dtype, block_size):
+    """Copies whose source and destination cannot overlap take short-lived workgroups in no particular order: pool ->
+    dense, dense -> pool and a list of per-layer tensors -> pool, with sequences of different lengths, offsets on both
+    sides, a missing source page and a missing destination page, against a row-by-row restatement."""
+    L, H, lens = 3, 4, [700, 64, 301, 0]
+    B = len(lens)
+    case = synth.make_paged_case(seed=21, num_layers=L, batch=B, num_kv_heads=H, seq_lens=[max(n, 1) for n in lens],
+                                 dtype=dtype, keep_dense=True, block_size=block_size, fill_value=7.0)
+    S = max(lens)
+    pool = case.kv_cache.to(dev)
+    tab = case.table_tensor(dev)
+    hole = tab.clone()
+    hole[0, 1] = -1                                             # sequence 0 lacks its second page
+    page_ok = torch.ones(B, S, dtype=torch.bool)
+    page_ok[0, block_size:2 * block_size] = False
+    all_ok = torch.ones(B, S, dtype=torch.bool)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device=dev)
+    dense_k = case.dense_k                                      # [L, B, H, S', D] with S' >= S
+    for seg_start, count, dst_start in ((0, S, 0), (5, 300, 9), (block_size - 1, 2, 0)):
+        # pool -> dense, with and without the hole
+        for t, ok in ((tab, all_ok), (hole, page_ok)):
+            out = torch.full((L, B, H, S + 16, 128), 3.0, dtype=dtype, device=dev)
+            ops.copy_tokens(_lib.paged_view(pool[0], t, lens_d, S), _lib.dense_view(out[:, :, :, :S]), seg_start, count,
+                            dst_start)
+            want = _copy_reference(dense_k[:, :, :, :S], ok, torch.full((L, B, H, S, 128), 3.0, dtype=dtype), all_ok, lens,
+                                   seg_start, count, dst_start)
+            got = out.cpu()
+            assert torch.equal(got[:, :, :, :S], want), (seg_start, count, dst_start)
+            assert bool((got[:, :, :, S:] == 3.0).all())
+        # dense -> pool (the V plane of the pool as the destination), destination with and without the hole;
+        # a dense source has no lengths of its own, so every sequence gets `count` rows as far as its pages reach
+        rows = _payload((L, B, H, S, 128), dtype, 5)
+        full = [S] * B
+        for t, ok in ((tab, all_ok), (hole, page_ok)):
+            dst = pool[1].clone()
+            old = torch.stack([torch.stack([_rows_of_table(dst[l].cpu(), case.block_tables[b], S, H) for b in range(B)])
+                               for l in range(L)])                                         # [L, B, H, S, D]
+            ops.copy_tokens(_lib.dense_view(rows.to(dev)), _lib.paged_view(dst, t, None, S), seg_start, count, dst_start)
+            reach = torch.zeros(B, S, dtype=torch.bool)
+            for b in range(B):
+                reach[b, :len(case.block_tables[b]) * block_size] = True
+            want = _copy_reference(rows, all_ok, old, ok & reach, full, seg_start, count, dst_start)
+            after = dst.cpu()
+            got = torch.stack([torch.stack([_rows_of_table(after[l], case.block_tables[b], S, H) for b in range(B)])
+                               for l in range(L)])
+            assert torch.equal(got, want), (seg_start, count, dst_start)
+            used = {blk for tb in case.block_tables for blk in tb}
+            spare = [i for i in range(after.shape[1]) if i not in used]
+            assert bool((after[:, spare] == 7.0).all())
+    # a list of per-layer tensors as the source
+    layers = [_payload((B, H, S, 128), dtype, 30 + l).to(dev) for l in range(L)]
+    dst = pool[1].clone()
+    assert ops.copy_tokens_from_layers(layers, _lib.paged_view(dst, tab, None, S), 200, 3)
+    after = dst.cpu()
+    for l in range(L):
+        for b in range(B):
+            n = min(200, max(0, len(case.block_tables[b]) * block_size - 3))
+            got = _rows_of_table(after[l], case.block_tables[b], S, H)
+            assert torch.equal(got[:, 3:3 + n], layers[l][b, :, :n].cpu()), (l, b)
+
+
+def _rows_of_table(plane, table, S, H):
+    """[H, S, D] rows of one sequence of one layer's plane [blocks, block_size, H, D]; tokens past its pages are 0."""
+    rows = torch.cat([plane[blk] for blk in table])[:S]
+    if rows.shape[0] < S:
+        rows = torch.cat([rows, torch.zeros(S - rows.shape[0], *rows.shape[1:], dtype=rows.dtype)])
+    return rows.permute(1, 0, 2)
