@@ -234,7 +234,8 @@ int fc_select_compact(const fc_kv_view* keys, const fc_kv_view* values, const fl
  * Gather + compaction.  For each (layer, b, kv head): dst token j <- src token
  * indices[(l*batch + b)*heads_in_index + (h % heads_in_index)][j] for j < n_kept[b] (or k).
  * `dst` may alias `src` (same pool, same tables): indices must then be ascending, and the
- * copy is ordered so that no source row is overwritten before it is read.
+ * copy is ordered so that no source row is overwritten before it is read.  When no destination view can overlap a
+ * source view (one paged and one dense, or dense views with disjoint byte ranges) the rows move in no particular order.
  * Replaces keys.gather(2, idx) (nanovllm/kernels/kvpress_compressor.py:241-249) followed by
  * LlavaModelRunner._write_compressed_kv_cache_fast (llava_model_runner.py:874-912), and the
  * generated sparse_gather kernel (nanovllm/autocompress/kernels.py:321-346).
@@ -405,7 +406,9 @@ int fc_dequantize_group4(const uint8_t* packed, const void* scale, int64_t group
  * Plain ordered token copy src[seg_start + i] -> dst[dst_start + i], i < count, per
  * (layer, b, head); the pass-through branch of compress_layer when seg_len/cf < min_seq_len
  * (module_ccm_v11.py:674-675).  dst may alias src when dst_start <= seg_start and both views are of one kind
- * (both paged or both dense); a paged and a dense view must not overlap (their rows are copied in no particular order).
+ * (both paged or both dense): the rows then move in ascending order.  A paged and a dense view must not overlap; they,
+ * and two dense views whose byte ranges are disjoint, are copied in no particular order (short-lived workgroups, the
+ * fastest form of a copy on this part).
  */
 int fc_copy_tokens(const fc_kv_view* src, const fc_kv_view* dst,
                    int32_t seg_start, int32_t count, int32_t dst_start, void* stream);
