@@ -6,7 +6,11 @@
 
 #define TH_THREADS 512
 #define TH_U 4            // rows per lane in flight
-#define TH_CHUNK 2048     // tokens per workgroup of the zeroing kernel
+// tokens per workgroup of the zeroing kernel: one pass of its 16 rows of 256 bytes, so that the workgroup loads, masks,
+// stores and ends (measured on 2304 columns of 4096 bf16 rows: 0.867 ms against 0.929 / 0.963 ms with 256 / 2048 tokens)
+#ifndef TH_CHUNK
+#define TH_CHUNK 16
+#endif
 
 // energy[l][b][h][d] = sum over the tokens s < len(b) of k[l][b][h][s][d]^2, fp32, fixed summation order
 template <int DTYPE>
