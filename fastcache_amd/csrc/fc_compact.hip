@@ -78,7 +78,8 @@ __global__ __launch_bounds__(CP_THREADS) void compact_kernel(KvView sk, KvView s
 // views), blockIdx.x / blockIdx.y = head and chunk of rows in the order the host picked (heads_fast: consecutive
 // workgroups take consecutive heads of the same tokens, for a destination that keeps a token's heads together;
 // otherwise consecutive chunks of one head), blockIdx.z = layer * sequences + sequence (the layer is the slowest index
-// of every layout this library meets), split with a multiplier the host precomputed (exact for every z below 2^16).  GATHER: source token = indices[j].
+// of every layout this library meets), split with a multiplier the host precomputed (exact for every z below 2^16).
+// GATHER: source token = indices[j].
 #ifndef CR_V
 #define CR_V 1
 #endif
