@@ -843,8 +843,8 @@ def measure(workload, seed, dev, steps, warmup, cpu_baseline=True, cpu_budget_s=
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
                     help="one configuration alone; default: cfg2 as the headline plus every configuration")
